@@ -1,0 +1,78 @@
+"""ctypes loader for ``libarcq_hip.so`` (the C ABI declared in ``include/arcq_hip.h``).
+
+There is deliberately no fallback: if the shared library has not been built,
+every op raises, so a GPU run can never silently go through something else.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libarcq_hip.so")
+
+ARCQ_F32 = 0
+ARCQ_F16 = 1
+
+_c_i64 = ctypes.c_int64
+_c_int = ctypes.c_int
+_c_ptr = ctypes.c_void_p
+_c_f32 = ctypes.c_float
+
+# name -> argtypes, in the order of include/arcq_hip.h
+_SIGNATURES = {
+    "arcq_pack_codes": [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_ptr],
+    "arcq_unpack_codes": [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_ptr],
+    "arcq_unpack_codes_u8": [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_ptr],
+    "arcq_act_quant": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                       _c_i64, _c_i64, _c_int, _c_int, _c_f32, _c_ptr],
+    "arcq_weight_dequant": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_int, _c_int,
+                            _c_ptr],
+    "arcq_linear_fused": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                          _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
+    "arcq_linear_otf": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                        _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
+    "arcq_linear_forward_packed": [_c_ptr] * 11 + [_c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_ptr],
+    "arcq_linear_forward_u8": [_c_ptr] * 11 + [_c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
+}
+EXPORTED_SYMBOLS = ("arcq_version", "arcq_last_error") + tuple(_SIGNATURES)
+
+_lib = None
+_lock = threading.Lock()
+
+
+class ARCQLibraryMissing(ImportError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise ARCQLibraryMissing(
+                    f"ARCQ HIP library is not built ({LIB_PATH} missing). "
+                    "Run `python -m arcq_vit_amd.build` (needs hipcc) first.")
+            lib = ctypes.CDLL(LIB_PATH)
+            lib.arcq_version.restype = _c_int
+            lib.arcq_version.argtypes = []
+            lib.arcq_last_error.restype = ctypes.c_char_p
+            lib.arcq_last_error.argtypes = []
+            for name, argtypes in _SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.restype = _c_int
+                fn.argtypes = argtypes
+            _lib = lib
+    return _lib
+
+
+def check(rc: int) -> None:
+    """Raise ``RuntimeError`` for a non-zero return, as ``TORCH_CHECK`` does in the reference's
+    host wrappers (e.g. EXT/arcq_activation_kernel.cu:194-202)."""
+    if rc != 0:
+        msg = load().arcq_last_error().decode("utf-8", "replace")
+        raise RuntimeError(msg or f"libarcq_hip call failed with code {rc}")

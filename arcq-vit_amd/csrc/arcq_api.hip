@@ -1,0 +1,50 @@
+// Library-level pieces of libarcq_hip.so: version, per-thread error text and
+// the whole-layer entry point that chains stage 1 into the fused stages 2+3.
+#include <stdarg.h>
+#include <string.h>
+
+#include "arcq_common.h"
+
+namespace arcq {
+
+static thread_local char g_last_error[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int launch_status(const char *what)
+{
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return ARCQ_OK;
+    return fail(static_cast<int>(e), "%s: launch failed: %s", what, hipGetErrorString(e));
+}
+
+}  // namespace arcq
+
+ARCQ_API int arcq_version(void) { return ARCQ_VERSION; }
+
+ARCQ_API const char *arcq_last_error(void) { return arcq::g_last_error; }
+
+// FQ/arcq_packed_on_the_fly.py:137-161: quantize+reconstruct the activation
+// into an fp16 buffer, then run the fused unpack+GEMM on it.
+ARCQ_API int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const float *a_codebook,
+                             const uint8_t *packed_w, const float *w_codebook,
+                             const float *w_center, const float *w_scale, const float *w_code_sum,
+                             const float *bias, void *x_hat_ws, void *y, int y_dtype,
+                             int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
+{
+    if (!x_hat_ws) return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf: x_hat_ws must not be NULL");
+    if (x_hat_ws == x && x_dtype != ARCQ_F16)
+        return arcq::fail(ARCQ_ERR_DTYPE, "arcq_linear_otf: x_hat_ws may alias x only when x is fp16");
+    int rc = arcq_act_quant(x, x_dtype, a_thresholds, a_codebook, nullptr, nullptr, nullptr, nullptr, nullptr,
+                            x_hat_ws, ARCQ_F16, M, K, bits, group_size, 1.0e-6f, stream);
+    if (rc != ARCQ_OK) return rc;
+    return arcq_linear_fused(x_hat_ws, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype,
+                             M, N, K, bits, group_size, stream);
+}

@@ -1,0 +1,58 @@
+// Shared host/device helpers for the ARCQ HIP kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "arcq_hip.h"
+
+#define ARCQ_API extern "C" __attribute__((visibility("default")))
+
+namespace arcq {
+
+// Records a message for arcq_last_error() and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// Turns hipGetLastError() after a launch into the ABI's return value.
+int launch_status(const char *what);
+
+__host__ __device__ inline bool bits_ok(int bits) { return bits == 2 || bits == 3 || bits == 4; }
+__host__ __device__ inline int64_t packed_cols(int64_t length, int bits) { return (length * bits + 7) / 8; }
+inline bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// Code j of a row whose packed bytes start at `row` (EXT/arcq_pack_kernel.cu:8-20).
+// The second byte is read only when the code really straddles, so the read
+// never leaves the row.
+__device__ __forceinline__ int get_code(const uint8_t *__restrict__ row, int64_t idx, int bits)
+{
+    const int64_t bit_offset = idx * bits;
+    const int64_t byte_idx = bit_offset >> 3;
+    const int shift = static_cast<int>(bit_offset & 7);
+    unsigned v = static_cast<unsigned>(row[byte_idx]) >> shift;
+    if (shift + bits > 8) v |= static_cast<unsigned>(row[byte_idx + 1]) << (8 - shift);
+    return static_cast<int>(v & ((1u << bits) - 1u));
+}
+
+// Eight consecutive codes starting at a multiple of eight occupy exactly `BITS`
+// bytes.  Returns them as one little-endian integer (code i at bit i*BITS).
+template <int BITS>
+__device__ __forceinline__ uint32_t load_codes8(const uint8_t *__restrict__ p)
+{
+    if constexpr (BITS == 4) {
+        return *reinterpret_cast<const uint32_t *>(p);
+    } else if constexpr (BITS == 2) {
+        return *reinterpret_cast<const uint16_t *>(p);
+    } else {
+        return static_cast<uint32_t>(p[0]) | (static_cast<uint32_t>(p[1]) << 8) | (static_cast<uint32_t>(p[2]) << 16);
+    }
+}
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(__half v) { return __half2float(v); }
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ __half from_float<__half>(float v) { return __float2half_rn(v); }
+
+}  // namespace arcq

@@ -1,0 +1,235 @@
+// Stages 2+3 fused: y[M,N] = x_hat[M,K] * w_hat[N,K]^T + bias, with w_hat
+// reconstructed on the fly from packed codes (never written to HBM).
+//
+// Reference semantics: unpack_weight_triton (FQ/arcq_packed_triton.py:11-74)
+// followed by F.linear in fp16 (FQ/arcq_packed_on_the_fly.py:159-160):
+// w_hat = fp16(fma(cb[code] - S/gs, s, mu)); products of fp16 operands are
+// accumulated in fp32; bias is added in fp32; the result is rounded once.
+//
+// Kernel shape (gs == 64): the K step of the main loop is one quantization group,
+// so each weight row needs exactly one (mu, s, S) triple per step.  Both
+// operands are K-contiguous, which is the layout v_mfma_f32_32x32x16_f16 wants:
+// lane l supplies 8 consecutive k for row (l % 32), k offset 8*(l / 32).
+#include "arcq_common.h"
+
+namespace arcq {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 64;            // one quantization group per main-loop step
+constexpr int LDS_STRIDE = 72;    // halves per tile row: 64 + 8 pad (144 B) -> conflict-free b128 reads
+
+// Reads the 32 codes [32*h, 32*h+32) of group g of one packed weight row.
+template <int BITS>
+__device__ __forceinline__ void load_codes32(const uint8_t *__restrict__ row_g, int h, uint32_t (&w)[BITS])
+{
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(row_g + h * (4 * BITS));
+    if constexpr (BITS == 4) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(p);
+        w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    } else if constexpr (BITS == 2) {
+        const uint2 v = *reinterpret_cast<const uint2 *>(p);
+        w[0] = v.x; w[1] = v.y;
+    } else {
+        w[0] = p[0]; w[1] = p[1]; w[2] = p[2];
+    }
+}
+
+// Code q (0..31) out of the little-endian bit string held in w[].
+template <int BITS>
+__device__ __forceinline__ int code_at(const uint32_t (&w)[BITS], int q)
+{
+    const int bit = q * BITS;
+    const int d = bit >> 5, sh = bit & 31;
+    uint32_t v = w[d] >> sh;
+    if (sh + BITS > 32) v |= w[d + 1] << (32 - sh);   // only for BITS == 3
+    return static_cast<int>(v & ((1u << BITS) - 1u));
+}
+
+template <int BITS, typename TOUT, int BM, int BN>
+__global__ void __launch_bounds__(256)
+gemm_fused_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, const float *__restrict__ cb,
+                  const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
+                  const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K)
+{
+    static_assert(BM % 64 == 0 && BN == 128, "tile shape");
+    constexpr int L = 1 << BITS;
+    constexpr int WM = BM / 2;          // wave tile rows (2x2 waves)
+    constexpr int WN = BN / 2;          // wave tile cols
+    constexpr int TI = WM / 32, TJ = WN / 32;
+    constexpr int A_PASSES = BM / 32;   // 256 threads x 16 B cover 32 rows of 64 halves
+
+    __shared__ __attribute__((aligned(16))) _Float16 sa[BM * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) _Float16 sb[BN * LDS_STRIDE];
+    __shared__ float lut[L * 64];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * BM;
+    const int n0 = blockIdx.x * BN;
+    const int G = K / BK;
+    const int64_t pcols = static_cast<int64_t>(K) * BITS / 8;
+
+    if (tid < 64) {
+#pragma unroll
+        for (int c = 0; c < L; ++c) lut[c * 64 + lane] = cb[c];
+    }
+
+    // global -> register staging
+    const int a_row = tid >> 3, a_col = (tid & 7) * 8;
+    const int b_row = tid >> 1, b_h = tid & 1;
+    const int bn = min(n0 + b_row, N - 1);
+    const uint8_t *pw_row = pw + static_cast<int64_t>(bn) * pcols;
+    const float *wc_row = wc + static_cast<int64_t>(bn) * G;
+    const float *ws_row = ws + static_cast<int64_t>(bn) * G;
+    const float *wcs_row = wcs + static_cast<int64_t>(bn) * G;
+
+    uint4 a_reg[A_PASSES];
+    uint32_t b_reg[BITS];
+    float b_c, b_s, b_m;
+
+    auto fetch = [&](int g) {
+#pragma unroll
+        for (int p = 0; p < A_PASSES; ++p) {
+            const int r = min(m0 + p * 32 + a_row, M - 1);
+            a_reg[p] = *reinterpret_cast<const uint4 *>(a + static_cast<int64_t>(r) * K + g * BK + a_col);
+        }
+        load_codes32<BITS>(pw_row + g * (8 * BITS), b_h, b_reg);
+        b_c = wc_row[g];
+        b_s = ws_row[g];
+        b_m = wcs_row[g] / 64.0f;
+    };
+
+    auto stage = [&]() {
+#pragma unroll
+        for (int p = 0; p < A_PASSES; ++p)
+            *reinterpret_cast<uint4 *>(&sa[(p * 32 + a_row) * LDS_STRIDE + a_col]) = a_reg[p];
+        _Float16 *dst = &sb[b_row * LDS_STRIDE + b_h * 32];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            half8_t hv;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int code = code_at<BITS>(b_reg, q4 * 8 + q);
+                hv[q] = static_cast<_Float16>(__fmaf_rn(lut[code * 64 + lane] - b_m, b_s, b_c));
+            }
+            *reinterpret_cast<half8_t *>(dst + q4 * 8) = hv;
+        }
+    };
+
+    float16_t acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    if (G > 0) fetch(0);
+    __syncthreads();  // lut visible
+    for (int g = 0; g < G; ++g) {
+        stage();
+        __syncthreads();
+        if (g + 1 < G) fetch(g + 1);
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+            half8_t af[TI], bf[TJ];
+            const int kof = kk * 16 + 8 * (lane >> 5);
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+                af[i] = *reinterpret_cast<const half8_t *>(&sa[(wm * WM + i * 32 + (lane & 31)) * LDS_STRIDE + kof]);
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+                bf[j] = *reinterpret_cast<const half8_t *>(&sb[(wn * WN + j * 32 + (lane & 31)) * LDS_STRIDE + kof]);
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+                for (int j = 0; j < TJ; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // Epilogue.  Accumulator element v of lane l is C[8*(v/4) + 4*(l/32) + v%4][l%32].
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) {
+        const int col = n0 + wn * WN + j * 32 + (lane & 31);
+        if (col >= N) continue;
+        const float bv = bias ? bias[col] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = m0 + wm * WM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (row < M) y[static_cast<int64_t>(row) * N + col] = from_float<TOUT>(acc[i][j][v] + bv);
+            }
+        }
+    }
+}
+
+template <int BITS, typename TOUT>
+static void launch_bits(const void *x_hat, const uint8_t *pw, const float *cb, const float *wc, const float *ws,
+                        const float *wcs, const float *bias, void *y, int M, int N, int K, hipStream_t stream)
+{
+    const __half *a = static_cast<const __half *>(x_hat);
+    TOUT *out = static_cast<TOUT *>(y);
+    // Small M (batch 1: 197 tokens) gets the 64-row tile so more workgroups exist.
+    const int64_t wg128 = static_cast<int64_t>((M + 127) / 128) * ((N + 127) / 128);
+    if (wg128 >= 256) {
+        dim3 grid((N + 127) / 128, (M + 127) / 128);
+        hipLaunchKernelGGL((gemm_fused_kernel<BITS, TOUT, 128, 128>), grid, dim3(256), 0, stream, a, pw, cb, wc, ws,
+                           wcs, bias, out, M, N, K);
+    } else {
+        dim3 grid((N + 127) / 128, (M + 63) / 64);
+        hipLaunchKernelGGL((gemm_fused_kernel<BITS, TOUT, 64, 128>), grid, dim3(256), 0, stream, a, pw, cb, wc, ws,
+                           wcs, bias, out, M, N, K);
+    }
+}
+
+template <typename TOUT>
+static void launch_out(const void *x_hat, const uint8_t *pw, const float *cb, const float *wc, const float *ws,
+                       const float *wcs, const float *bias, void *y, int M, int N, int K, int bits, hipStream_t stream)
+{
+    if (bits == 4) launch_bits<4, TOUT>(x_hat, pw, cb, wc, ws, wcs, bias, y, M, N, K, stream);
+    else if (bits == 3) launch_bits<3, TOUT>(x_hat, pw, cb, wc, ws, wcs, bias, y, M, N, K, stream);
+    else launch_bits<2, TOUT>(x_hat, pw, cb, wc, ws, wcs, bias, y, M, N, K, stream);
+}
+
+}  // namespace arcq
+
+using namespace arcq;
+
+ARCQ_API int arcq_linear_fused(const void *x_hat,
+                               const uint8_t *packed_w, const float *w_codebook,
+                               const float *w_center, const float *w_scale, const float *w_code_sum,
+                               const float *bias, void *y, int y_dtype,
+                               int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
+{
+    if (!bits_ok(bits)) return fail(ARCQ_ERR_BITS, "arcq_linear_fused: bits must be 2, 3, or 4");
+    if (M < 0 || N < 0 || K < 0 || group_size <= 0) return fail(ARCQ_ERR_SHAPE, "arcq_linear_fused: bad sizes");
+    if (K % group_size != 0)
+        return fail(ARCQ_ERR_GROUP, "arcq_linear_fused: in_features must be divisible by group_size");
+    if (group_size != 64)
+        return fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_fused: only group_size 64 is built (got %d)", group_size);
+    if (y_dtype != ARCQ_F16 && y_dtype != ARCQ_F32)
+        return fail(ARCQ_ERR_DTYPE, "arcq_linear_fused: y must be float16 or float32");
+    if (M * N == 0) return ARCQ_OK;
+    if (!y) return fail(ARCQ_ERR_NULL, "arcq_linear_fused: y must not be NULL");
+    if (K > 0 && (!x_hat || !packed_w || !w_codebook || !w_center || !w_scale || !w_code_sum))
+        return fail(ARCQ_ERR_NULL, "arcq_linear_fused: NULL tensor pointer");
+    if (M >= (int64_t(1) << 31) - 256 || N >= (int64_t(1) << 31) - 256 || K >= (int64_t(1) << 31) - 256 ||
+        (N + 127) / 128 > 0x7fffffff || (M + 63) / 64 > 65535)
+        return fail(ARCQ_ERR_SHAPE, "arcq_linear_fused: M, N or K too large");
+    if (!aligned(x_hat, 16) || !aligned(y, 16) || !aligned(packed_w, 16))
+        return fail(ARCQ_ERR_ALIGN, "arcq_linear_fused: x_hat, y and packed_w must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
+    if (y_dtype == ARCQ_F16)
+        launch_out<__half>(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, m, n, k, bits, st);
+    else
+        launch_out<float>(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, m, n, k, bits, st);
+    return launch_status("arcq_linear_fused");
+}

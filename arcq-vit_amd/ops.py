@@ -1,0 +1,349 @@
+"""Operator layer: the reference extension's eight functions, same names, argument order and
+returns, on top of ``libarcq_hip.so``.
+
+Reference binding table: FQ/arcq_infer_cuda/arcq_infer_bind.cpp:57-66 (``FQ`` =
+``methods/fair_qat_framework/fair_qat``).  Also here: the two launchers of
+FQ/arcq_packed_triton.py (``unpack_weight_triton`` :77-120, ``dequant_activation_triton``
+:181-215) under HIP names, and the fused entry points that have no counterpart in the
+reference (``linear_fused``, ``linear_otf``).
+
+All tensors must live on the GPU; outputs are allocated with torch on the same device and the
+kernels are enqueued on torch's current stream.  Nothing here synchronises.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from . import _lib
+from ._lib import ARCQ_F16, ARCQ_F32
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def _check(cond: bool, msg: str) -> None:
+    # TORCH_CHECK raises c10::Error, which Python sees as RuntimeError.
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _dtype_code(t: torch.Tensor, name: str) -> int:
+    if t.dtype == torch.float32:
+        return ARCQ_F32
+    if t.dtype == torch.float16:
+        return ARCQ_F16
+    raise RuntimeError(f"{name} must be float32 or float16")
+
+
+def _check_bits(bits: int) -> None:
+    _check(bits in (2, 3, 4), "bits must be 2, 3, or 4")
+
+
+def _f32c(t: torch.Tensor) -> torch.Tensor:
+    return t.to(torch.float32).contiguous()
+
+
+# ---------------------------------------------------------------------------------------------
+# bit packing -- EXT/arcq_pack_kernel.cu:94-158
+# ---------------------------------------------------------------------------------------------
+def pack_codes(codes: torch.Tensor, bits: int) -> torch.Tensor:
+    """int codes ``[rows, length]`` -> ``uint8 [rows, ceil(length*bits/8)]`` (LSB-first bitstream)."""
+    _check(codes.is_cuda, "codes must be CUDA tensor")
+    _check_bits(bits)
+    _check(codes.dim() == 2, "codes must have shape [rows, length]")
+    c = codes.to(torch.int64).contiguous()
+    rows, length = c.shape
+    packed = torch.empty((rows, (length * bits + 7) // 8), dtype=torch.uint8, device=c.device)
+    with torch.cuda.device(c.device):
+        _lib.check(_lib.load().arcq_pack_codes(_ptr(c), _ptr(packed), rows, length, bits, _stream()))
+    return packed
+
+
+def _unpack(packed: torch.Tensor, bits: int, length: int, out_dtype: torch.dtype) -> torch.Tensor:
+    _check(packed.is_cuda, "packed must be CUDA tensor")
+    _check(packed.dtype == torch.uint8, "packed must be uint8")
+    _check_bits(bits)
+    _check(packed.dim() == 2, "packed must have shape [rows, packed_cols]")
+    length = int(length)
+    _check(length >= 0 and (length * bits + 7) // 8 <= packed.shape[1], "length exceeds the packed row")
+    p = packed.contiguous()
+    rows = p.shape[0]
+    # The kernels index rows by ceil(length*bits/8); hand them exactly that row pitch.
+    pc = (length * bits + 7) // 8
+    if p.shape[1] != pc:
+        p = p[:, :pc].contiguous()
+    codes = torch.empty((rows, length), dtype=out_dtype, device=p.device)
+    fn = _lib.load().arcq_unpack_codes if out_dtype == torch.int64 else _lib.load().arcq_unpack_codes_u8
+    with torch.cuda.device(p.device):
+        _lib.check(fn(_ptr(p), _ptr(codes), rows, length, bits, _stream()))
+    return codes
+
+
+def unpack_codes(packed: torch.Tensor, bits: int, length: int) -> torch.Tensor:
+    """Inverse of :func:`pack_codes`, int64 out (EXT/arcq_pack_kernel.cu:116-136)."""
+    return _unpack(packed, bits, length, torch.int64)
+
+
+def unpack_codes_u8(packed: torch.Tensor, bits: int, length: int) -> torch.Tensor:
+    """Inverse of :func:`pack_codes`, uint8 out (EXT/arcq_pack_kernel.cu:138-158)."""
+    return _unpack(packed, bits, length, torch.uint8)
+
+
+# ---------------------------------------------------------------------------------------------
+# stage 1 -- EXT/arcq_activation_kernel.cu:188-326
+# ---------------------------------------------------------------------------------------------
+def _act_quant(x: torch.Tensor, thresholds: torch.Tensor, codebook: torch.Tensor, bits: int, group_size: int,
+               want_packed: bool = False, want_u8: bool = False, want_meta: bool = False,
+               x_hat: Optional[torch.Tensor] = None, strict_f32: bool = True, eps: float = 1.0e-6):
+    _check(x.is_cuda, "x must be CUDA tensor")
+    _check(thresholds.is_cuda, "thresholds must be CUDA tensor")
+    _check(codebook.is_cuda, "codebook must be CUDA tensor")
+    _check_bits(bits)
+    _check(x.dim() == 2, "x must have shape [rows, cols]")
+    if strict_f32:
+        _check(x.dtype == torch.float32, "x must be float32")
+    _check(thresholds.dtype == torch.float32, "thresholds must be float32")
+    _check(codebook.dtype == torch.float32, "codebook must be float32")
+    group_size = int(group_size)
+    _check(group_size > 0 and x.shape[1] % group_size == 0, "in_features must be divisible by group_size")
+    _check(codebook.numel() == (1 << bits), f"codebook must have {1 << bits} entries for {bits}-bit codes")
+    _check(thresholds.numel() == codebook.numel() - 1, "thresholds must have one entry fewer than the codebook")
+    x = x.contiguous()
+    thresholds = thresholds.contiguous()
+    codebook = codebook.contiguous()
+    rows, cols = x.shape
+    groups = cols // group_size
+    dev = x.device
+    packed = torch.empty((rows, (cols * bits + 7) // 8), dtype=torch.uint8, device=dev) if want_packed else None
+    codes = torch.empty((rows, cols), dtype=torch.uint8, device=dev) if want_u8 else None
+    center = torch.empty((rows, groups), dtype=torch.float32, device=dev) if want_meta else None
+    scale = torch.empty((rows, groups), dtype=torch.float32, device=dev) if want_meta else None
+    code_sum = torch.empty((rows, groups), dtype=torch.float32, device=dev) if want_meta else None
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().arcq_act_quant(
+            _ptr(x), _dtype_code(x, "x"), _ptr(thresholds), _ptr(codebook), _ptr(packed), _ptr(codes), _ptr(center),
+            _ptr(scale), _ptr(code_sum), _ptr(x_hat), _dtype_code(x_hat, "x_hat") if x_hat is not None else ARCQ_F32,
+            rows, cols, bits, group_size, float(eps), _stream()))
+    return packed, codes, center, scale, code_sum
+
+
+def quantize_activation(x: torch.Tensor, thresholds: torch.Tensor, codebook: torch.Tensor, bits: int,
+                        group_size: int) -> List[torch.Tensor]:
+    """-> ``[packed u8 [rows, cols*bits/8], center, scale, code_sum f32 [rows, groups]]``
+    (EXT/arcq_activation_kernel.cu:188-237)."""
+    packed, _, center, scale, code_sum = _act_quant(x, thresholds, codebook, bits, group_size, want_packed=True,
+                                                    want_meta=True)
+    return [packed, center, scale, code_sum]
+
+
+def quantize_activation_u8(x: torch.Tensor, thresholds: torch.Tensor, codebook: torch.Tensor, bits: int,
+                           group_size: int) -> List[torch.Tensor]:
+    """-> ``[codes u8 [rows, cols], center, scale, code_sum]`` (EXT/arcq_activation_kernel.cu:239-285)."""
+    _, codes, center, scale, code_sum = _act_quant(x, thresholds, codebook, bits, group_size, want_u8=True,
+                                                   want_meta=True)
+    return [codes, center, scale, code_sum]
+
+
+def quantize_activation_dequant(x: torch.Tensor, thresholds: torch.Tensor, codebook: torch.Tensor, bits: int,
+                                group_size: int) -> torch.Tensor:
+    """-> ``x_hat f32 [rows, cols]`` (EXT/arcq_activation_kernel.cu:287-326)."""
+    _check(x.is_cuda, "x must be CUDA tensor")
+    _check(x.dim() == 2, "x must have shape [rows, cols]")
+    _check(x.dtype == torch.float32, "x must be float32")
+    x = x.contiguous()
+    x_hat = torch.empty_like(x)
+    _act_quant(x, thresholds, codebook, bits, group_size, x_hat=x_hat)
+    return x_hat
+
+
+def dequant_activation_hip(x: torch.Tensor, thresholds: torch.Tensor, codebook: torch.Tensor, group_size: int,
+                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Fused quantize+reconstruct, fp16 or fp32, optionally in place (``out=x``).
+
+    Same contract as ``dequant_activation_triton`` (FQ/arcq_packed_triton.py:181-215), including its
+    ``out`` checks; statistics are always taken in fp32, also for fp16 input.
+    """
+    _check(x.dim() == 2, "x must have shape [rows, cols]")
+    x = x.contiguous()
+    thresholds = thresholds.contiguous().float()
+    codebook = codebook.contiguous().float()
+    levels = codebook.numel()
+    bits = levels.bit_length() - 1
+    if out is None:
+        out = torch.empty_like(x)
+    else:
+        if out.shape != x.shape:
+            raise ValueError(f"dequant_activation out shape {tuple(out.shape)} != input shape {tuple(x.shape)}")
+        if out.dtype != x.dtype:
+            raise ValueError(f"dequant_activation out dtype {out.dtype} != input dtype {x.dtype}")
+        if not out.is_contiguous():
+            raise ValueError("dequant_activation out must be contiguous")
+    _act_quant(x, thresholds, codebook, bits, group_size, x_hat=out, strict_f32=False)
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# stage 2 -- FQ/arcq_packed_triton.py:77-120
+# ---------------------------------------------------------------------------------------------
+def unpack_weight_hip(packed: torch.Tensor, codebook: torch.Tensor, center: torch.Tensor, scale: torch.Tensor,
+                      code_sum: torch.Tensor, bits: int, group_size: int,
+                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """packed codes + metadata -> fp16 weight ``[out_f, in_f]``.
+
+    Same contract as ``unpack_weight_triton``: ``out`` may be a larger flat fp16 buffer shared by all
+    layers (FQ/arcq_packed_on_the_fly.py:149-157); the first ``out_f*in_f`` elements are written and the
+    buffer itself is returned.
+    """
+    _check(packed.is_cuda, "packed must be CUDA tensor")
+    _check(packed.dtype == torch.uint8, "packed must be uint8")
+    _check_bits(bits)
+    out_f = packed.shape[0]
+    groups = center.shape[1]
+    in_f = groups * int(group_size)
+    _check(packed.shape[1] == (in_f * bits + 7) // 8, "packed row length does not match in_features*bits/8")
+    packed = packed.contiguous()
+    codebook, center, scale, code_sum = _f32c(codebook), _f32c(center), _f32c(scale), _f32c(code_sum)
+    if out is None:
+        out = torch.empty((out_f, in_f), dtype=torch.float16, device=packed.device)
+    else:
+        _check(out.is_cuda and out.is_contiguous() and out.numel() >= out_f * in_f, "out buffer too small")
+        _check(out.dtype in (torch.float16, torch.float32), "out must be float16 or float32")
+    with torch.cuda.device(packed.device):
+        _lib.check(_lib.load().arcq_weight_dequant(
+            _ptr(packed), _ptr(codebook), _ptr(center), _ptr(scale), _ptr(code_sum), _ptr(out),
+            _dtype_code(out, "out"), out_f, in_f, bits, int(group_size), _stream()))
+    return out
+
+
+# Import-compatible aliases for code written against FQ/arcq_packed_triton.py.
+dequant_activation_triton = dequant_activation_hip
+unpack_weight_triton = unpack_weight_hip
+
+
+# ---------------------------------------------------------------------------------------------
+# stages 2+3 fused / whole layer -- no counterpart function in the reference; they replace the
+# unpack + F.linear pair at FQ/arcq_packed_on_the_fly.py:148-160
+# ---------------------------------------------------------------------------------------------
+def linear_fused(x_hat: torch.Tensor, packed_w: torch.Tensor, w_codebook: torch.Tensor, w_center: torch.Tensor,
+                 w_scale: torch.Tensor, w_code_sum: torch.Tensor, bias: Optional[torch.Tensor], bits: int,
+                 group_size: int, out_dtype: torch.dtype = torch.float16) -> torch.Tensor:
+    """``y = x_hat @ w_hat.T + bias`` with ``w_hat`` rebuilt from packed codes inside the GEMM."""
+    _check(x_hat.is_cuda and packed_w.is_cuda, "x_hat and packed_w must be CUDA tensors")
+    _check(x_hat.dim() == 2 and x_hat.dtype == torch.float16, "x_hat must be float16 [M, K]")
+    _check(packed_w.dtype == torch.uint8 and packed_w.dim() == 2, "packed_w must be uint8 [N, K*bits/8]")
+    _check_bits(bits)
+    x_hat = x_hat.contiguous()
+    m, k = x_hat.shape
+    n = packed_w.shape[0]
+    _check(packed_w.shape[1] == (k * bits + 7) // 8, "packed_w row length does not match K*bits/8")
+    y = torch.empty((m, n), dtype=out_dtype, device=x_hat.device)
+    b = None if bias is None or bias.numel() == 0 else _f32c(bias)
+    w = [packed_w.contiguous(), _f32c(w_codebook), _f32c(w_center), _f32c(w_scale), _f32c(w_code_sum)]
+    with torch.cuda.device(x_hat.device):
+        _lib.check(_lib.load().arcq_linear_fused(
+            _ptr(x_hat), *[_ptr(t) for t in w], _ptr(b), _ptr(y), _dtype_code(y, "y"),
+            m, n, k, bits, int(group_size), _stream()))
+    return y
+
+
+def linear_otf(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Tensor, packed_w: torch.Tensor,
+               w_codebook: torch.Tensor, w_center: torch.Tensor, w_scale: torch.Tensor, w_code_sum: torch.Tensor,
+               bias: Optional[torch.Tensor], bits: int, group_size: int, out_dtype: torch.dtype = torch.float16,
+               x_hat_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Whole packed on-the-fly layer on ``x [M, K]`` (fp16 or fp32): stage 1 into ``x_hat_ws`` (fp16
+    ``[M, K]``, allocated if not given), then the fused GEMM."""
+    _check(x.is_cuda and packed_w.is_cuda, "x and packed_w must be CUDA tensors")
+    _check(x.dim() == 2, "x must have shape [M, K]")
+    _check_bits(bits)
+    x = x.contiguous()
+    m, k = x.shape
+    n = packed_w.shape[0]
+    _check(packed_w.shape[1] == (k * bits + 7) // 8, "packed_w row length does not match K*bits/8")
+    if x_hat_ws is None:
+        x_hat_ws = torch.empty((m, k), dtype=torch.float16, device=x.device)
+    else:
+        _check(x_hat_ws.dtype == torch.float16 and x_hat_ws.is_contiguous() and x_hat_ws.numel() >= m * k,
+               "x_hat_ws must be a contiguous float16 buffer of at least M*K elements")
+    y = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    b = None if bias is None or bias.numel() == 0 else _f32c(bias)
+    a = [_f32c(a_thresholds), _f32c(a_codebook)]
+    w = [packed_w.contiguous(), _f32c(w_codebook), _f32c(w_center), _f32c(w_scale), _f32c(w_code_sum)]
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().arcq_linear_otf(
+            _ptr(x), _dtype_code(x, "x"), *[_ptr(t) for t in a], *[_ptr(t) for t in w], _ptr(b), _ptr(x_hat_ws),
+            _ptr(y), _dtype_code(y, "y"), m, n, k, bits, int(group_size), _stream()))
+    return y
+
+
+# ---------------------------------------------------------------------------------------------
+# index-space linears -- EXT/arcq_linear_kernel.cu:206-353
+# ---------------------------------------------------------------------------------------------
+def arcq_linear_forward(packed_x: torch.Tensor, x_center: torch.Tensor, x_scale: torch.Tensor,
+                        x_code_sum: torch.Tensor, packed_w: torch.Tensor, w_center: torch.Tensor,
+                        w_scale: torch.Tensor, w_code_sum: torch.Tensor, product_table: torch.Tensor,
+                        bias: Optional[torch.Tensor], bits: int, group_size: int, in_features: int,
+                        out_features: int) -> torch.Tensor:
+    """fp64-accumulated product-table linear on packed codes (EXT/arcq_linear_kernel.cu:206-278)."""
+    _check(packed_x.is_cuda, "packed_x must be CUDA tensor")
+    _check(packed_w.is_cuda, "packed_w must be CUDA tensor")
+    _check(packed_x.dtype == torch.uint8, "packed_x must be uint8")
+    _check(packed_w.dtype == torch.uint8, "packed_w must be uint8")
+    _check_bits(bits)
+    _check(int(in_features) % int(group_size) == 0, "in_features must be divisible by group_size")
+    _check(product_table.dtype == torch.float32, "product_table must be float32")
+    pc = (int(in_features) * bits + 7) // 8
+    _check(packed_x.dim() == 2 and packed_x.shape[1] == pc, "packed_x row length does not match in_features*bits/8")
+    _check(packed_w.dim() == 2 and packed_w.shape == (int(out_features), pc),
+           "packed_w shape does not match [out_features, in_features*bits/8]")
+    rows = packed_x.shape[0]
+    levels = product_table.shape[0]
+    y = torch.empty((rows, int(out_features)), dtype=torch.float32, device=packed_x.device)
+    b = None
+    if bias is not None and bias.numel() > 0:
+        _check(bias.is_cuda, "bias must be CUDA tensor")
+        b = _f32c(bias)
+    tensors = [packed_x.contiguous(), _f32c(x_center), _f32c(x_scale), _f32c(x_code_sum), packed_w.contiguous(),
+               _f32c(w_center), _f32c(w_scale), _f32c(w_code_sum), _f32c(product_table)]
+    with torch.cuda.device(packed_x.device):
+        _lib.check(_lib.load().arcq_linear_forward_packed(
+            *[_ptr(t) for t in tensors], _ptr(b), _ptr(y), rows, int(out_features), int(in_features), bits,
+            int(group_size), levels, _stream()))
+    return y
+
+
+def arcq_linear_forward_u8(x_codes: torch.Tensor, x_center: torch.Tensor, x_scale: torch.Tensor,
+                           x_code_sum: torch.Tensor, w_codes: torch.Tensor, w_center: torch.Tensor,
+                           w_scale: torch.Tensor, w_code_sum: torch.Tensor, product_table: torch.Tensor,
+                           bias: Optional[torch.Tensor], group_size: int) -> torch.Tensor:
+    """fp32 product-table linear on byte codes, 32-lane summation order (EXT/arcq_linear_kernel.cu:280-353)."""
+    _check(x_codes.is_cuda, "x_codes must be CUDA tensor")
+    _check(w_codes.is_cuda, "w_codes must be CUDA tensor")
+    _check(x_codes.dtype == torch.uint8, "x_codes must be uint8")
+    _check(w_codes.dtype == torch.uint8, "w_codes must be uint8")
+    _check(x_codes.dim() == 2, "x_codes must have shape [rows, in_features]")
+    _check(w_codes.dim() == 2, "w_codes must have shape [out_features, in_features]")
+    _check(x_codes.shape[1] == w_codes.shape[1], "x_codes and w_codes in_features must match")
+    _check(x_codes.shape[1] % int(group_size) == 0, "in_features must be divisible by group_size")
+    _check(product_table.dtype == torch.float32, "product_table must be float32")
+    rows, in_features = x_codes.shape
+    out_features = w_codes.shape[0]
+    levels = product_table.shape[0]
+    y = torch.empty((rows, out_features), dtype=torch.float32, device=x_codes.device)
+    b = None
+    if bias is not None and bias.numel() > 0:
+        _check(bias.is_cuda, "bias must be CUDA tensor")
+        b = _f32c(bias)
+    tensors = [x_codes.contiguous(), _f32c(x_center), _f32c(x_scale), _f32c(x_code_sum), w_codes.contiguous(),
+               _f32c(w_center), _f32c(w_scale), _f32c(w_code_sum), _f32c(product_table)]
+    with torch.cuda.device(x_codes.device):
+        _lib.check(_lib.load().arcq_linear_forward_u8(
+            *[_ptr(t) for t in tensors], _ptr(b), _ptr(y), rows, out_features, in_features, int(group_size), levels,
+            _stream()))
+    return y

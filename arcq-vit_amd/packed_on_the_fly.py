@@ -1,0 +1,107 @@
+"""``ARCQPackedLinearOnTheFly``: the packed on-the-fly layer (the path the reference's README
+benchmarks), constructor and buffers as FQ/arcq_packed_on_the_fly.py:93-135.
+
+Reference forward (:137-161): fp16 copy of x -> Triton quantize+reconstruct in place -> Triton
+unpack of the whole weight into an fp16 buffer in HBM -> cuBLAS ``F.linear``.  Here: one HIP
+stage-1 kernel writes x_hat (fp16) into a workspace, and one HIP kernel streams the packed
+codes, rebuilds the weight tile by tile in LDS and feeds fp16 MFMA; the dense weight never
+exists in HBM.  Differences a caller can observe: the input tensor is never overwritten (the
+reference overwrites a contiguous fp16 input), statistics are taken in fp32 even for fp16 input,
+and ``_weight_buffer`` is accepted but unused.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import ops
+
+# One reusable fp16 x_hat workspace per (device, stream): layers run back to back on a stream, and
+# stream order makes the reuse safe.  Grown on demand, never shrunk.
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, numel: int) -> torch.Tensor:
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < numel:
+        ws = torch.empty(max(numel, 1), dtype=torch.float16, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+class ARCQPackedLinearOnTheFly(nn.Module):
+    """Stores packed codes + codebooks + per-group metadata + bias only (no dense weight)."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool,
+                 packed_weight_codes: torch.Tensor, weight_codebook: torch.Tensor,
+                 weight_center: torch.Tensor, weight_scale: torch.Tensor, weight_code_sum: torch.Tensor,
+                 activation_codebook: torch.Tensor, activation_thresholds: torch.Tensor,
+                 bits: int, group_size: int, bias_tensor: Optional[torch.Tensor]):
+        super().__init__()
+        self.in_features = int(in_features)
+        self.out_features = int(out_features)
+        self.bits = int(bits)
+        self.group_size = int(group_size)
+        self.groups = self.in_features // self.group_size
+        if self.bits not in (2, 3, 4):
+            raise ValueError(f"packed kernel supports bits 2/3/4, got {self.bits}")
+        if self.in_features % self.group_size != 0:
+            raise ValueError(f"in_features={self.in_features} must be divisible by group_size={self.group_size}")
+        if tuple(packed_weight_codes.shape) != (self.out_features, (self.in_features * self.bits + 7) // 8):
+            raise ValueError(f"packed_weight_codes has shape {tuple(packed_weight_codes.shape)}, expected "
+                             f"{(self.out_features, (self.in_features * self.bits + 7) // 8)}")
+        self.register_buffer("packed_weight_codes", packed_weight_codes)
+        self.register_buffer("weight_codebook", weight_codebook)
+        self.register_buffer("weight_center", weight_center)
+        self.register_buffer("weight_scale", weight_scale)
+        self.register_buffer("weight_code_sum", weight_code_sum)
+        self.register_buffer("activation_codebook", activation_codebook)
+        self.register_buffer("activation_thresholds", activation_thresholds)
+        if bias and bias_tensor is not None and bias_tensor.numel() > 0:
+            self.register_buffer("bias_tensor", bias_tensor)
+        else:
+            self.register_buffer("bias_tensor", torch.empty(0))
+        self.out_dtype = torch.float16
+
+    @classmethod
+    def from_packed(cls, packed_layer: nn.Module) -> "ARCQPackedLinearOnTheFly":
+        """From an ``ARCQPackedLinear`` (what scripts/benchmark_arcq_on_the_fly.py:151-170 does)."""
+        b = packed_layer.bias if packed_layer.bias.numel() > 0 else None
+        return cls(packed_layer.in_features, packed_layer.out_features, b is not None,
+                   packed_layer.packed_weight_codes, packed_layer.weight_codebook, packed_layer.weight_center,
+                   packed_layer.weight_scale, packed_layer.weight_code_sum, packed_layer.activation_codebook,
+                   packed_layer.activation_thresholds, packed_layer.bits, packed_layer.group_size, b)
+
+    def _apply(self, fn, *args, **kwargs):
+        # model.half() must not narrow the fp32 metadata (the reference undoes it afterwards,
+        # scripts/benchmark_arcq_on_the_fly.py:63-85); keep those buffers fp32 through any cast.
+        super()._apply(fn, *args, **kwargs)
+        for name in ("weight_codebook", "weight_center", "weight_scale", "weight_code_sum",
+                     "activation_codebook", "activation_thresholds", "bias_tensor"):
+            buf = self._buffers.get(name)
+            if buf is not None and buf.is_floating_point() and buf.dtype != torch.float32:
+                self._buffers[name] = buf.float()
+        return self
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        original_shape = x.shape
+        if original_shape[-1] != self.in_features:
+            raise ValueError(f"expected last dim {self.in_features}, got {original_shape[-1]}")
+        x2 = x.reshape(-1, self.in_features)
+        if x2.dtype not in (torch.float16, torch.float32):
+            x2 = x2.to(torch.float16)
+        x2 = x2.contiguous()
+        ws = _workspace(x2.device, x2.numel())
+        bias = self.bias_tensor if self.bias_tensor.numel() > 0 else None
+        y = ops.linear_otf(x2, self.activation_thresholds, self.activation_codebook, self.packed_weight_codes,
+                           self.weight_codebook, self.weight_center, self.weight_scale, self.weight_code_sum,
+                           bias, self.bits, self.group_size, out_dtype=self.out_dtype, x_hat_ws=ws)
+        return y.reshape(*original_shape[:-1], self.out_features)
+
+    def estimated_persistent_mb(self) -> float:
+        """MiB held by this layer's buffers (FQ/arcq_packed_on_the_fly.py:163-169)."""
+        return sum(b.numel() * b.element_size() for b in self.buffers()) / 1024 / 1024

@@ -1,0 +1,131 @@
+"""Minimal DeiT / ViT skeleton whose submodule names match timm's ``VisionTransformer``
+(``patch_embed.proj``, ``cls_token``, ``pos_embed``, ``blocks.N.{norm1,attn.{qkv,proj},norm2,
+mlp.{fc1,fc2}}``, ``norm``, ``head``), so packed-checkpoint keys produced from a timm model
+(FQ/timm_quant_models.py:155-182) line up.  timm itself is not available offline.
+
+Only the four block linears are quantized (the packed path's scope); patch embedding, LayerNorm,
+softmax attention, GELU and the head stay in floating point, as the reference's README states.
+"""
+from __future__ import annotations
+
+from typing import Callable, Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .packed_convert import convert_arcq_linear_to_packed, to_on_the_fly
+from .quant_source import QuantLinearPCARCQ
+from .synth import MODEL_DIMS, SEED, quantile_codebook
+
+LinearFactory = Callable[[int, int, bool], nn.Module]
+
+
+class PatchEmbed(nn.Module):
+    def __init__(self, dim: int, patch: int = 16, in_ch: int = 3):
+        super().__init__()
+        self.proj = nn.Conv2d(in_ch, dim, kernel_size=patch, stride=patch)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.proj(x).flatten(2).transpose(1, 2)
+
+
+class Attention(nn.Module):
+    def __init__(self, dim: int, heads: int, linear: LinearFactory):
+        super().__init__()
+        self.num_heads = heads
+        self.qkv = linear(dim, dim * 3, True)
+        self.proj = linear(dim, dim, True)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        b, n, c = x.shape
+        qkv = self.qkv(x).reshape(b, n, 3, self.num_heads, c // self.num_heads).permute(2, 0, 3, 1, 4)
+        q, k, v = qkv.unbind(0)
+        y = F.scaled_dot_product_attention(q, k, v)
+        return self.proj(y.transpose(1, 2).reshape(b, n, c))
+
+
+class Mlp(nn.Module):
+    def __init__(self, dim: int, hidden: int, linear: LinearFactory):
+        super().__init__()
+        self.fc1 = linear(dim, hidden, True)
+        self.act = nn.GELU()
+        self.fc2 = linear(hidden, dim, True)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.fc2(self.act(self.fc1(x)))
+
+
+class Block(nn.Module):
+    def __init__(self, dim: int, heads: int, hidden: int, linear: LinearFactory):
+        super().__init__()
+        self.norm1 = nn.LayerNorm(dim, eps=1e-6)
+        self.attn = Attention(dim, heads, linear)
+        self.norm2 = nn.LayerNorm(dim, eps=1e-6)
+        self.mlp = Mlp(dim, hidden, linear)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        x = x + self.attn(self.norm1(x))
+        return x + self.mlp(self.norm2(x))
+
+
+class VisionTransformer(nn.Module):
+    def __init__(self, dim: int, depth: int, heads: int, mlp: int, num_classes: int = 1000,
+                 linear: Optional[LinearFactory] = None, img: int = 224, patch: int = 16):
+        super().__init__()
+        linear = linear or (lambda i, o, b: nn.Linear(i, o, bias=b))
+        self.embed_dim = dim
+        self.patch_embed = PatchEmbed(dim, patch)
+        n_patches = (img // patch) ** 2
+        self.cls_token = nn.Parameter(torch.zeros(1, 1, dim))
+        self.pos_embed = nn.Parameter(torch.zeros(1, n_patches + 1, dim))
+        self.blocks = nn.Sequential(*[Block(dim, heads, mlp, linear) for _ in range(depth)])
+        self.norm = nn.LayerNorm(dim, eps=1e-6)
+        self.head = nn.Linear(dim, num_classes)
+
+    def forward_features(self, x: torch.Tensor) -> torch.Tensor:
+        x = self.patch_embed(x)
+        x = torch.cat([self.cls_token.expand(x.shape[0], -1, -1).to(x.dtype), x], dim=1) + self.pos_embed.to(x.dtype)
+        return self.norm(self.blocks(x))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.head(self.forward_features(x)[:, 0])
+
+
+def build_fakequant_vit(model: str, bits: int, group_size: int = 64, seed: int = SEED,
+                        num_classes: int = 1000) -> VisionTransformer:
+    """Random-init ViT whose block linears are ``QuantLinearPCARCQ`` with quantile codebooks
+    (weights N(0, 0.02^2), as timm's trunc_normal_(std=.02) init; biases N(0, 0.01^2))."""
+    cfg = MODEL_DIMS[model]
+    cb = quantile_codebook(bits)
+
+    def make(i: int, o: int, b: bool) -> nn.Module:
+        layer = QuantLinearPCARCQ(i, o, b, bits, bits, group_size)
+        layer.act_quant.set_codebook(cb)
+        layer.weight_quant.set_codebook(cb)
+        return layer
+
+    g = torch.Generator().manual_seed(int(seed))
+    vit = VisionTransformer(cfg["dim"], cfg["depth"], cfg["heads"], cfg["mlp"], num_classes, linear=make)
+    with torch.no_grad():
+        for name, p in vit.named_parameters():
+            if p.dim() >= 2:
+                p.copy_(torch.randn(p.shape, generator=g) * 0.02)
+            elif name.endswith("bias"):
+                p.copy_(torch.randn(p.shape, generator=g) * 0.01)
+            # LayerNorm weights keep their default of one
+    return vit.eval()
+
+
+def build_packed_vit(model: str, bits: int, group_size: int = 64, seed: int = SEED, num_classes: int = 1000,
+                     device: str = "cuda", half_chain: bool = True) -> VisionTransformer:
+    """Fake-quant ViT -> packed (``convert_arcq_linear_to_packed``) -> on-the-fly layers -> device,
+    the sequence of scripts/benchmark_arcq_on_the_fly.py:88-199.  ``half_chain`` casts the
+    floating-point rest of the model to fp16 (packed metadata stays fp32)."""
+    vit = build_fakequant_vit(model, bits, group_size, seed, num_classes)
+    convert_arcq_linear_to_packed(vit, runtime_code_format="packed")
+    to_on_the_fly(vit)
+    vit = vit.to(device)
+    if half_chain:
+        vit = vit.half()
+    return vit.eval()

@@ -1,0 +1,273 @@
+#!/usr/bin/env python3
+"""Benchmark of the packed on-the-fly quantized-linear hot path on one MI355X.
+
+Workload (BASELINE.json configs[1]): the 48 packed linears of DeiT-Small (12 blocks x qkv 384->1152,
+proj 384->384, fc1 384->1536, fc2 1536->384), W4A4, group size 64, fp16 activations in and out,
+batch 64 (M = 64*197 = 12608 tokens).  One step = one pass over all 48 layers: stage 1 (activation
+group-residual quantize + reconstruct) and the fused unpack+GEMM for each.  Inputs (one synthetic
+activation tensor per layer shape, packed weights of 48 distinct random layers) are resident in HBM
+before the timed region starts.
+
+Prints ONE JSON line.  ``value`` is images/s of that step.  ``roofline`` is for the dominant kernel,
+the fused GEMM: algorithmic flops (2*M*N*K summed over the 48 launches of a step) divided by the
+time of those launches alone, measured here with HIP events on the launch stream in a GEMM-only
+loop.  ``cpu_baseline`` times the oracle's restatement of the reference's fake-quant CPU path
+(quantize + reconstruct activation and weight, fp32 matmul) on a bounded sample on this host.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--model", default="deit_small")
+    ap.add_argument("--bits", type=int, default=4)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-bs1", action="store_true")
+    return ap.parse_args()
+
+
+class Layer:
+    """Device buffers of one packed layer plus the raw C-ABI argument lists for a fixed M."""
+
+    def __init__(self, name, k, n, bits, seed, dev):
+        import torch
+        from arcq_vit_amd import synth
+        from arcq_vit_amd.packed_linear import _quantize_weight_reference
+        from arcq_vit_amd.pack_py import pack_codes_py
+        cb = synth.quantile_codebook(bits)
+        thr = synth.midpoint_thresholds(cb)
+        w = synth.make_weight(n, k, seed)
+        codes, center, scale, code_sum = _quantize_weight_reference(w, thr, cb, 64, 1e-6)
+        self.name, self.k, self.n, self.bits = name, k, n, bits
+        self.packed = pack_codes_py(codes, bits).to(dev)
+        self.cb, self.thr = cb.to(dev), thr.to(dev)
+        self.center, self.scale, self.code_sum = center.to(dev), scale.to(dev), code_sum.to(dev)
+        self.bias = synth.make_bias(n, seed).to(dev)
+        self.w_fp32 = w  # CPU, for the CPU baseline only
+
+    def otf_args(self, x, ws, y, stream):
+        from arcq_vit_amd._lib import ARCQ_F16
+        m = x.shape[0]
+        return (x.data_ptr(), ARCQ_F16, self.thr.data_ptr(), self.cb.data_ptr(), self.packed.data_ptr(),
+                self.cb.data_ptr(), self.center.data_ptr(), self.scale.data_ptr(), self.code_sum.data_ptr(),
+                self.bias.data_ptr(), ws.data_ptr(), y.data_ptr(), ARCQ_F16, m, self.n, self.k, self.bits, 64, stream)
+
+    def gemm_args(self, ws, y, m, stream):
+        from arcq_vit_amd._lib import ARCQ_F16
+        return (ws.data_ptr(), self.packed.data_ptr(), self.cb.data_ptr(), self.center.data_ptr(),
+                self.scale.data_ptr(), self.code_sum.data_ptr(), self.bias.data_ptr(), y.data_ptr(), ARCQ_F16,
+                m, self.n, self.k, self.bits, 64, stream)
+
+    def act_args(self, x, ws, stream):
+        from arcq_vit_amd._lib import ARCQ_F16
+        m = x.shape[0]
+        return (x.data_ptr(), ARCQ_F16, self.thr.data_ptr(), self.cb.data_ptr(), 0, 0, 0, 0, 0, ws.data_ptr(),
+                ARCQ_F16, m, self.k, self.bits, 64, 1.0e-6, stream)
+
+
+def build_workload(model, bits, batch, dev):
+    import torch
+    from arcq_vit_amd import synth
+    m = batch * synth.TOKENS
+    depth = synth.MODEL_DIMS[model]["depth"]
+    layers = []
+    for blk in range(depth):
+        for i, (name, k, n) in enumerate(synth.block_linear_shapes(model)):
+            layers.append(Layer(f"blocks.{blk}.{name}", k, n, bits, synth.SEED + 16 * blk + i, dev))
+    inputs = {}
+    for i, (name, k, n) in enumerate(synth.block_linear_shapes(model)):
+        kind = "gelu" if name == "fc2" else "ln"
+        inputs[name] = synth.make_activation(m, k, synth.SEED + 1000 + i, kind).to(torch.float16).to(dev)
+    kmax = max(l.k for l in layers)
+    nmax = max(l.n for l in layers)
+    ws = torch.empty(m * kmax, dtype=torch.float16, device=dev)
+    y = torch.empty(m * nmax, dtype=torch.float16, device=dev)
+    return m, layers, inputs, ws, y
+
+
+def time_loop(fn, steps, warmup):
+    """Runs fn() warmup+steps times; returns seconds for exactly `steps`, from HIP events on the
+    current stream, bracketed by synchronize on both sides."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3
+
+
+def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
+    import torch
+    from arcq_vit_amd import _lib, synth
+    lib = _lib.load()
+    m, layers, inputs, ws, y = build_workload(model, bits, batch, dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def short(l):
+        return l.name.rsplit(".", 1)[-1]
+
+    otf = [l.otf_args(inputs[short(l)], ws, y, stream) for l in layers]
+    acts = [l.act_args(inputs[short(l)], ws, stream) for l in layers]
+    gemms = [l.gemm_args(ws, y, m, stream) for l in layers]
+
+    def step_full():
+        for a in otf:
+            rc = lib.arcq_linear_otf(*a)
+            if rc:
+                _lib.check(rc)
+
+    def step_act():
+        for a in acts:
+            rc = lib.arcq_act_quant(*a)
+            if rc:
+                _lib.check(rc)
+
+    def step_gemm():
+        for a in gemms:
+            rc = lib.arcq_linear_fused(*a)
+            if rc:
+                _lib.check(rc)
+
+    if use_graph:
+        # Launch-bound regime (batch 1): replay the whole 48-layer step as one HIP graph, as the
+        # reference does for bs <= 1 (scripts/benchmark_arcq_on_the_fly.py:223-231).
+        def capture(kind):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                sp = torch.cuda.current_stream().cuda_stream   # the capture stream
+                for l in layers:
+                    x = inputs[short(l)]
+                    if kind == "full":
+                        rc = lib.arcq_linear_otf(*l.otf_args(x, ws, y, sp))
+                    elif kind == "act":
+                        rc = lib.arcq_act_quant(*l.act_args(x, ws, sp))
+                    else:
+                        rc = lib.arcq_linear_fused(*l.gemm_args(ws, y, m, sp))
+                    if rc:
+                        _lib.check(rc)
+            return g.replay
+        step_full()
+        torch.cuda.synchronize()
+        step_full, step_act, step_gemm = capture("full"), capture("act"), capture("gemm")
+
+    t_full = time_loop(step_full, steps, warmup)
+    t_gemm = time_loop(step_gemm, steps, warmup)
+    t_act = time_loop(step_act, steps, warmup)
+
+    flops = sum(synth.algorithmic_flops(m, l.n, l.k) for l in layers)
+    gemm_bytes = sum(synth.algorithmic_bytes(m, l.n, l.k, bits) for l in layers)
+    act_bytes = sum(2 * 2 * m * l.k for l in layers)          # fp16 in, fp16 out
+    res = {
+        "batch": batch, "M": m, "layers": len(layers),
+        "ms_per_step": t_full / steps * 1e3,
+        "images_per_s": batch * steps / t_full,
+        "gemm_ms_per_step": t_gemm / steps * 1e3,
+        "gemm_us_per_launch": t_gemm / steps / len(layers) * 1e6,
+        "gemm_tflops": flops * steps / t_gemm / 1e12,
+        "gemm_gbs": gemm_bytes * steps / t_gemm / 1e9,
+        "act_ms_per_step": t_act / steps * 1e3,
+        "act_us_per_launch": t_act / steps / len(layers) * 1e6,
+        "act_gbs": act_bytes * steps / t_act / 1e9,
+        "flops_per_step": flops, "gemm_bytes_per_step": gemm_bytes,
+    }
+    return res, layers, inputs
+
+
+def cpu_baseline(layers, inputs, batch, budget_s=20.0):
+    """Oracle restatement of QuantLinearPCARCQ.forward (FQ/quant_backends.py:312-322) on host cores:
+    the four linears of ONE block at the benchmark's batch, repeated while the time budget lasts
+    (at least once); images/s = batch / (depth * time per block)."""
+    import torch
+    from arcq_vit_amd import synth
+    from oracle import arcq_ref
+    block = layers[:4]
+    depth = len(layers) // 4
+    xs = [inputs[l.name.rsplit(".", 1)[-1]].float().cpu() for l in block]
+    cb = synth.quantile_codebook(block[0].bits)
+    thr = synth.midpoint_thresholds(cb)
+    bs = [l.bias.cpu() for l in block]
+    with torch.no_grad():
+        arcq_ref.fake_quant_linear(xs[1][:256], block[1].w_fp32, bs[1], thr, cb, thr, cb, 64, 1e-6)  # warm up
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            for l, x, b in zip(block, xs, bs):
+                arcq_ref.fake_quant_linear(x, l.w_fp32, b, thr, cb, thr, cb, 64, 1e-6)
+            reps += 1
+            if time.perf_counter() - t0 > budget_s or reps >= 8:
+                break
+        dt = (time.perf_counter() - t0) / reps
+    return {"value": batch / (depth * dt), "unit": "images/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"4 linears of one DeiT block at batch {batch} (M={xs[0].shape[0]}), {reps} repetitions, "
+                      f"scaled by depth {depth}; torch fp32 on {torch.get_num_threads()} threads "
+                      f"(os.cpu_count()={os.cpu_count()})",
+            "ms_per_block": dt * 1e3}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path issues no collectives); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from arcq_vit_amd import _lib
+    _lib.load()
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    res, layers, inputs = run_config(args.model, args.bits, args.batch, args.steps, args.warmup, dev)
+    out = {
+        "metric": "DeiT-S W4A4 images/s at bs1/bs64; packed-linear % of MFMA/HBM roofline",
+        "value": res["images_per_s"], "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"{args.model} 48 packed linears (12 blocks x qkv/proj/fc1/fc2), W{args.bits}A{args.bits}, "
+                               f"g=64, batch {args.batch} (M={res['M']}), fp16 in/out, stage 1 + fused unpack+GEMM",
+                   "model_shapes": args.model, "bits": args.bits, "batch": args.batch, "group_size": 64},
+        "roofline": {"bound": "mfma", "kernel": "gemm_fused_kernel", "achieved": res["gemm_tflops"],
+                     "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": res["gemm_tflops"] / PEAK_FP16_TFLOPS,
+                     "traffic": None, "avg_launch_us": res["gemm_us_per_launch"],
+                     "hbm_frac_of_same_kernel": res["gemm_gbs"] / PEAK_HBM_GBS},
+        "stage1": {"kernel": "act_quant_g64_kernel", "bound": "hbm", "achieved": res["act_gbs"], "peak": PEAK_HBM_GBS,
+                   "unit": "GB/s", "frac": res["act_gbs"] / PEAK_HBM_GBS, "avg_launch_us": res["act_us_per_launch"]},
+        "detail_bs%d" % args.batch: res,
+    }
+    if not args.no_bs1:
+        r1, _, _ = run_config(args.model, args.bits, 1, max(args.steps, 50), max(args.warmup, 10), dev, use_graph=True)
+        out["bs1"] = {"images_per_s": r1["images_per_s"], "ms_per_step": r1["ms_per_step"],
+                      "gemm_us_per_launch": r1["gemm_us_per_launch"], "gemm_gbs_warm": r1["gemm_gbs"],
+                      "gemm_hbm_frac_warm": r1["gemm_gbs"] / PEAK_HBM_GBS, "act_us_per_launch": r1["act_us_per_launch"],
+                      "hip_graph": True}
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(layers, inputs, args.batch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,154 @@
+/*
+ * arcq_hip.h -- C ABI of libarcq_hip.so: ARCQ packed quantized-linear kernels
+ * for AMD MI355X (gfx950 / CDNA4).
+ *
+ * Every entry point is a plain-C replacement for one binding of the
+ * reference's pybind11 extension `arcq_infer_cuda_ext`
+ * (methods/fair_qat_framework/fair_qat/arcq_infer_cuda/arcq_infer_bind.cpp:57-66)
+ * or for one of its Triton launchers
+ * (methods/fair_qat_framework/fair_qat/arcq_packed_triton.py).  Abbreviations
+ * in the citations below: FQ = methods/fair_qat_framework/fair_qat,
+ * EXT = FQ/arcq_infer_cuda.
+ *
+ * Conventions
+ *   - All pointers are DEVICE pointers on the current HIP device unless said
+ *     otherwise.  Tensors are dense row-major.  The library never allocates,
+ *     frees or synchronises; the caller owns every buffer.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Every
+ *     call only enqueues kernels on that stream and returns.
+ *   - Return value: 0 = ok; < 0 = argument error (ARCQ_ERR_*), nothing was
+ *     enqueued; > 0 = the hipError_t of a failed launch.  arcq_last_error()
+ *     returns a message for the calling thread's most recent non-zero return.
+ *   - bits is 2, 3 or 4; a codebook has L = 2^bits fp32 entries and L-1
+ *     non-decreasing fp32 thresholds.  Code j of a row lives at bits
+ *     [j*bits, (j+1)*bits) of the row's little-endian byte stream
+ *     (EXT/arcq_pack_kernel.cu:8-36); a row of n codes takes
+ *     ceil(n*bits/8) bytes.
+ *   - Floating-point contract: fp32 IEEE arithmetic with round-to-nearest,
+ *     correctly rounded divide and sqrt, group sums taken serially left to
+ *     right (the loop order of EXT/arcq_activation_kernel.cu:49-60); fused
+ *     multiply-add only in the two reconstructions x_hat = fma(s, v, mu) and
+ *     w_hat = fma(v, s, mu).
+ */
+#ifndef ARCQ_HIP_H
+#define ARCQ_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ARCQ_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* element types for the void* tensor arguments */
+#define ARCQ_F32 0
+#define ARCQ_F16 1
+
+/* argument errors (negative return values) */
+#define ARCQ_OK 0
+#define ARCQ_ERR_BITS (-1)        /* "bits must be 2, 3, or 4" */
+#define ARCQ_ERR_GROUP (-2)       /* "in_features must be divisible by group_size" */
+#define ARCQ_ERR_NULL (-3)        /* a required pointer is NULL */
+#define ARCQ_ERR_SHAPE (-4)       /* negative or inconsistent sizes */
+#define ARCQ_ERR_DTYPE (-5)       /* dtype code not supported by this entry point */
+#define ARCQ_ERR_UNSUPPORTED (-6) /* valid for the reference, not built here (message says what) */
+#define ARCQ_ERR_ALIGN (-7)       /* pointer not aligned as the kernel requires */
+
+int arcq_version(void);
+const char *arcq_last_error(void);
+
+/* ---- bit packing --------------------------------------------------------
+ * Replaces pack_codes_cuda / unpack_codes_cuda / unpack_codes_u8_cuda,
+ * EXT/arcq_pack_kernel.cu:94-114, :116-136, :138-158.
+ * codes [rows, length]; packed [rows, ceil(length*bits/8)].  `packed` need not
+ * be zeroed beforehand (the reference pre-zeroes and ORs).  Codes are masked
+ * to their low `bits` bits, as set_packed_code_u8 does. */
+int arcq_pack_codes(const int64_t *codes, uint8_t *packed, int64_t rows, int64_t length, int bits, void *stream);
+int arcq_unpack_codes(const uint8_t *packed, int64_t *codes, int64_t rows, int64_t length, int bits, void *stream);
+int arcq_unpack_codes_u8(const uint8_t *packed, uint8_t *codes, int64_t rows, int64_t length, int bits, void *stream);
+
+/* ---- stage 1: activation group-residual quantizer -------------------------
+ * One kernel replaces quantize_activation_cuda, quantize_activation_u8_cuda and
+ * quantize_activation_dequant_cuda (EXT/arcq_activation_kernel.cu:188-237,
+ * :239-285, :287-326) and dequant_activation_triton
+ * (FQ/arcq_packed_triton.py:181-215); which outputs are produced is chosen by
+ * which output pointers are non-NULL:
+ *   packed   [rows, ceil(cols*bits/8)] u8   bit-packed codes
+ *   codes_u8 [rows, cols] u8                one byte per code
+ *   center, scale, code_sum [rows, cols/group_size] f32
+ *   x_hat    [rows, cols] of x_hat_dtype    mu + s*(cb[code] - code_sum/gs)
+ * x is [rows, cols] of x_dtype (ARCQ_F32 or ARCQ_F16; fp16 is widened to fp32
+ * before any arithmetic).  x_hat may alias x when the two dtypes are equal
+ * (the in-place use at FQ/arcq_packed_on_the_fly.py:143-145).
+ * eps is added to the variance inside the square root; the reference kernels
+ * hard-code 1e-6f.  thresholds [L-1], codebook [L], both fp32. */
+int arcq_act_quant(const void *x, int x_dtype, const float *thresholds, const float *codebook,
+                   uint8_t *packed, uint8_t *codes_u8, float *center, float *scale, float *code_sum,
+                   void *x_hat, int x_hat_dtype,
+                   int64_t rows, int64_t cols, int bits, int group_size, float eps, void *stream);
+
+/* ---- stage 2: packed weight -> dense weight -------------------------------
+ * Replaces unpack_weight_triton (FQ/arcq_packed_triton.py:77-120):
+ * out[n,k] = (cb[code] - code_sum[n,g]/gs) * scale[n,g] + center[n,g], g = k/gs,
+ * rounded once to out_dtype (ARCQ_F16 as the reference, or ARCQ_F32).
+ * packed [N, ceil(K*bits/8)]; center/scale/code_sum [N, K/group_size]. */
+int arcq_weight_dequant(const uint8_t *packed, const float *codebook,
+                        const float *center, const float *scale, const float *code_sum,
+                        void *out, int out_dtype,
+                        int64_t N, int64_t K, int bits, int group_size, void *stream);
+
+/* ---- stages 2+3 fused: y = x_hat * w_hat^T + bias --------------------------
+ * Replaces the pair unpack_weight_triton + F.linear at
+ * FQ/arcq_packed_on_the_fly.py:148-160 (and F.linear on weight_dequant at
+ * FQ/arcq_packed_linear.py:175-176) without materialising w_hat in HBM: packed
+ * codes are streamed, reconstructed exactly as arcq_weight_dequant does,
+ * rounded to fp16, and fed to fp16 MFMA with fp32 accumulation.
+ * x_hat [M,K] fp16; y [M,N] of y_dtype (ARCQ_F16 or ARCQ_F32); bias [N] fp32 or
+ * NULL, added in fp32 before the output rounding.  Requires group_size == 64;
+ * x_hat and y must be 16-byte aligned, packed_w 4-byte aligned. */
+int arcq_linear_fused(const void *x_hat,
+                      const uint8_t *packed_w, const float *w_codebook,
+                      const float *w_center, const float *w_scale, const float *w_code_sum,
+                      const float *bias, void *y, int y_dtype,
+                      int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
+
+/* ---- whole packed on-the-fly layer: stage 1 then stages 2+3 ----------------
+ * Replaces ARCQPackedLinearOnTheFly.forward's device work
+ * (FQ/arcq_packed_on_the_fly.py:137-161).  x [M,K] of x_dtype; x_hat_ws is a
+ * caller-owned fp16 [M,K] workspace that receives the reconstructed activation
+ * (it may alias x when x_dtype == ARCQ_F16, as the reference overwrites its
+ * fp16 copy of x). */
+int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const float *a_codebook,
+                    const uint8_t *packed_w, const float *w_codebook,
+                    const float *w_center, const float *w_scale, const float *w_code_sum,
+                    const float *bias, void *x_hat_ws, void *y, int y_dtype,
+                    int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
+
+/* ---- index-space linears (no reconstruction, product-table gather) ---------
+ * Replace arcq_linear_forward_cuda (EXT/arcq_linear_kernel.cu:206-278; fp64
+ * accumulation, kernel :22-78) and arcq_linear_forward_u8_cuda (:280-353; fp32,
+ * 32-lane strided partial sums folded by a shuffle-down tree, kernel :136-202).
+ * Both reproduce the reference's summation order, so results are bit-identical
+ * to a serial CPU evaluation in that order.  product_table [levels, levels]
+ * fp32 = cb_a (x) cb_w; bias [out_features] fp32 or NULL; y [rows, out_features]
+ * fp32. */
+int arcq_linear_forward_packed(const uint8_t *packed_x, const float *x_center, const float *x_scale,
+                               const float *x_code_sum,
+                               const uint8_t *packed_w, const float *w_center, const float *w_scale,
+                               const float *w_code_sum,
+                               const float *product_table, const float *bias, float *y,
+                               int64_t rows, int64_t out_features, int64_t in_features,
+                               int bits, int group_size, int levels, void *stream);
+int arcq_linear_forward_u8(const uint8_t *x_codes, const float *x_center, const float *x_scale,
+                           const float *x_code_sum,
+                           const uint8_t *w_codes, const float *w_center, const float *w_scale,
+                           const float *w_code_sum,
+                           const float *product_table, const float *bias, float *y,
+                           int64_t rows, int64_t out_features, int64_t in_features,
+                           int group_size, int levels, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ARCQ_HIP_H */

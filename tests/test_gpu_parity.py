@@ -1,0 +1,323 @@
+"""GPU parity: every HIP entry point, called through the C ABI (via the ctypes shim in
+``arcq_vit_amd.ops``), against the CPU oracle on the same seeded inputs.
+
+Bars: bit-exact for codes, packed bytes, group metadata and reconstructions (integer work and
+fp32 work with a fixed operation order); for the fp16 MFMA GEMM the fp32-accumulation error bound
+stated in ``_gemm_tol``.
+"""
+import numpy as np
+import pytest
+import torch
+
+from arcq_vit_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _cb(bits):
+    cb = synth.quantile_codebook(bits)
+    return cb, synth.midpoint_thresholds(cb)
+
+
+def _np(t):
+    return t.detach().cpu().numpy()
+
+
+# ------------------------------------------------------------------------------------------------
+# bit packing
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("shape", [(1, 1), (3, 7), (5, 64), (17, 197), (768, 192), (384, 1536)])
+def test_pack_unpack(cuda, oracle, bits, shape):
+    rng = np.random.default_rng(bits * 31 + shape[1])
+    codes = rng.integers(0, 1 << bits, size=shape, dtype=np.int64)
+    packed = ops.pack_codes(torch.from_numpy(codes).to(cuda), bits)
+    assert packed.dtype == torch.uint8 and tuple(packed.shape) == (shape[0], (shape[1] * bits + 7) // 8)
+    assert np.array_equal(_np(packed), oracle.pack_codes_c(codes, bits))
+    assert np.array_equal(_np(ops.unpack_codes(packed, bits, shape[1])), codes)
+    u8 = ops.unpack_codes_u8(packed, bits, shape[1])
+    assert u8.dtype == torch.uint8 and np.array_equal(_np(u8), codes.astype(np.uint8))
+
+
+def test_pack_masks_and_overwrites(cuda, oracle):
+    """High bits are dropped, and the output needs no pre-zeroing."""
+    codes = torch.tensor([[0x1F, 0x23, -1, 7, 9]], dtype=torch.int64)
+    for bits in (2, 3, 4):
+        got = ops.pack_codes(codes.to(cuda), bits)
+        assert np.array_equal(_np(got), oracle.pack_codes_c(codes.numpy(), bits))
+
+
+def test_pack_empty(cuda):
+    assert tuple(ops.pack_codes(torch.zeros((0, 8), dtype=torch.int64, device=cuda), 4).shape) == (0, 4)
+    assert tuple(ops.unpack_codes(torch.zeros((4, 0), dtype=torch.uint8, device=cuda), 3, 0).shape) == (4, 0)
+
+
+# ------------------------------------------------------------------------------------------------
+# stage 1
+# ------------------------------------------------------------------------------------------------
+def _check_stage1(cuda, oracle, x, bits, gs=64):
+    cb, thr = _cb(bits)
+    ref = oracle.act_quant_c(x.numpy(), thr, cb, bits, gs)
+    xd, thrd, cbd = x.to(cuda), thr.to(cuda), cb.to(cuda)
+    packed, center, scale, code_sum = ops.quantize_activation(xd, thrd, cbd, bits, gs)
+    assert np.array_equal(_np(packed), ref["packed"])
+    assert np.array_equal(_np(center), ref["center"])
+    assert np.array_equal(_np(scale), ref["scale"])
+    assert np.array_equal(_np(code_sum), ref["code_sum"])
+    codes, c2, s2, cs2 = ops.quantize_activation_u8(xd, thrd, cbd, bits, gs)
+    assert np.array_equal(_np(codes), ref["codes"])
+    assert torch.equal(c2, center) and torch.equal(s2, scale) and torch.equal(cs2, code_sum)
+    x_hat = ops.quantize_activation_dequant(xd, thrd, cbd, bits, gs)
+    assert x_hat.dtype == torch.float32 and np.array_equal(_np(x_hat), ref["x_hat"])
+    return ref
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("m,k,kind", [(197, 192, "ln"), (197, 384, "ln"), (197, 1536, "gelu"), (1, 64, "ln"),
+                                      (63, 128, "ln"), (65, 64, "gelu"), (1000, 384, "ln")])
+def test_stage1_bitexact_fp32(cuda, oracle, bits, m, k, kind):
+    _check_stage1(cuda, oracle, synth.make_activation(m, k, 100 + bits, kind), bits)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_stage1_fp16_chain_and_inplace(cuda, oracle, bits):
+    """fp16 in -> fp16 out, as the on-the-fly layer runs it; fp16 is widened exactly, statistics are
+    fp32, x_hat is rounded once to fp16.  In-place (out=x) gives the same bytes."""
+    cb, thr = _cb(bits)
+    x16 = synth.make_activation(197, 384, 7).to(torch.float16)
+    ref = oracle.act_quant_c(x16.float().numpy(), thr, cb, bits, 64)
+    want = ref["x_hat"].astype(np.float16)
+    xd = x16.to(cuda)
+    out = ops.dequant_activation_hip(xd, thr.to(cuda), cb.to(cuda), 64)
+    assert out.dtype == torch.float16 and out.data_ptr() != xd.data_ptr()
+    assert np.array_equal(_np(out).view(np.uint16), want.view(np.uint16))
+    assert torch.equal(xd.cpu(), x16)                      # input untouched
+    same = ops.dequant_activation_hip(xd, thr.to(cuda), cb.to(cuda), 64, out=xd)
+    assert same.data_ptr() == xd.data_ptr()
+    assert np.array_equal(_np(xd).view(np.uint16), want.view(np.uint16))
+    # fp32 in place as well
+    x32 = synth.make_activation(130, 192, 8).to(cuda)
+    ref32 = oracle.act_quant_c(_np(x32), thr, cb, bits, 64)
+    ops.dequant_activation_hip(x32, thr.to(cuda), cb.to(cuda), 64, out=x32)
+    assert np.array_equal(_np(x32), ref32["x_hat"])
+
+
+@pytest.mark.parametrize("gs,bits", [(32, 4), (128, 3), (16, 2), (192, 4)])
+def test_stage1_other_group_sizes(cuda, oracle, gs, bits):
+    _check_stage1(cuda, oracle, synth.make_activation(33, 384, gs, "ln"), bits, gs)
+
+
+def test_stage1_ties_constant_and_extremes(cuda, oracle):
+    """Exact ties (thresholds taken from occurring t values), constant groups (s = sqrt(eps)),
+    large magnitudes and zeros."""
+    bits = 4
+    cb, _ = _cb(bits)
+    x = synth.make_activation(16, 128, 3)
+    x[0] = 2.5
+    x[1, :64] = 0.0
+    x[2] *= 3.0e4
+    x[3] *= 1.0e-4
+    ref0 = oracle.act_quant_c(x.numpy(), synth.midpoint_thresholds(cb), cb, bits, 64)
+    t = ((x.numpy().reshape(16, 2, 64) - ref0["center"][..., None]) / ref0["scale"][..., None]).astype(np.float32)
+    thr = torch.from_numpy(np.sort(np.unique(t))[5::137][:15].copy())
+    assert thr.numel() == 15
+    ref = oracle.act_quant_c(x.numpy(), thr, cb, bits, 64)
+    packed, center, scale, code_sum = ops.quantize_activation(x.to(cuda), thr.to(cuda), cb.to(cuda), bits, 64)
+    assert np.array_equal(_np(packed), ref["packed"])
+    assert np.array_equal(_np(scale), ref["scale"]) and np.array_equal(_np(code_sum), ref["code_sum"])
+    assert _np(scale)[0, 0] == np.sqrt(np.float32(1e-6))
+
+
+def test_stage1_empty(cuda):
+    cb, thr = _cb(4)
+    out = ops.quantize_activation(torch.zeros((0, 128), device=cuda), thr.to(cuda), cb.to(cuda), 4, 64)
+    assert tuple(out[0].shape) == (0, 64) and tuple(out[1].shape) == (0, 2)
+
+
+def test_stage1_torch_order_tie_audit(cuda, oracle):
+    """Against the torch restatement (torch's own reduction order) codes may differ only at near-ties."""
+    bits = 4
+    cb, thr = _cb(bits)
+    x = synth.make_activation(197, 384, 55)
+    codes = _np(ops.quantize_activation_u8(x.to(cuda), thr.to(cuda), cb.to(cuda), bits, 64)[0])
+    codes_t, _, _, _, _ = oracle.act_quant_torch(x, thr, cb, 64)
+    diff = np.argwhere(codes != codes_t.numpy())
+    assert len(diff) < 1e-3 * x.numel()
+    x64 = x.double().reshape(197, -1, 64)
+    mu = x64.mean(-1, keepdim=True)
+    t64 = ((x64 - mu) / ((x64 - mu).square().mean(-1, keepdim=True) + 1e-6).sqrt()).reshape(197, 384).numpy()
+    for r, c in diff:
+        assert np.min(np.abs(thr.double().numpy() - t64[r, c])) < 4e-6 * max(1.0, abs(t64[r, c]))
+
+
+# ------------------------------------------------------------------------------------------------
+# stage 2
+# ------------------------------------------------------------------------------------------------
+def _packed_weight(oracle, n, k, bits, seed, gs=64):
+    cb, thr = _cb(bits)
+    w = synth.make_weight(n, k, seed)
+    codes, center, scale, code_sum = oracle.quantize_weight_torch(w, thr, cb, gs, 1e-6)
+    packed = torch.from_numpy(oracle.pack_codes_np(codes.numpy(), bits))
+    return cb, packed, center, scale, code_sum
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("n,k", [(768, 192), (384, 1536), (1152, 384), (5, 64)])
+def test_stage2_bitexact(cuda, oracle, bits, n, k):
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 9)
+    ref = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, bits, 64, fma=True)
+    got = ops.unpack_weight_hip(packed.to(cuda), cb.to(cuda), center.to(cuda), scale.to(cuda), code_sum.to(cuda),
+                                bits, 64)
+    assert got.dtype == torch.float16 and tuple(got.shape) == (n, k)
+    assert np.array_equal(_np(got).view(np.uint16), ref.astype(np.float16).view(np.uint16))
+    out32 = torch.empty((n, k), dtype=torch.float32, device=cuda)
+    ops.unpack_weight_hip(packed.to(cuda), cb.to(cuda), center.to(cuda), scale.to(cuda), code_sum.to(cuda), bits, 64,
+                          out=out32)
+    assert np.array_equal(_np(out32), ref)
+    # against the two-rounding torch formulation: at most one fp16 ulp apart
+    torch_w = oracle.unpack_weight_torch(packed, cb, center, scale, code_sum, bits, 64)
+    d = np.abs(_np(got).view(np.int16).astype(np.int32) - torch_w.numpy().view(np.int16).astype(np.int32))
+    assert d.max() <= 1 and (d != 0).mean() < 1e-3
+
+
+def test_stage2_shared_buffer_and_odd_group(cuda, oracle):
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, 10, 96, 3, 4, gs=12)
+    ref = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, 3, 12, fma=True)
+    buf = torch.zeros(4096, dtype=torch.float16, device=cuda)
+    out = ops.unpack_weight_hip(packed.to(cuda), cb.to(cuda), center.to(cuda), scale.to(cuda), code_sum.to(cuda),
+                                3, 12, out=buf)
+    assert out.data_ptr() == buf.data_ptr()
+    assert np.array_equal(_np(buf[:960]).view(np.uint16), ref.astype(np.float16).ravel().view(np.uint16))
+    assert not buf[960:].any()
+
+
+# ------------------------------------------------------------------------------------------------
+# stages 2+3 fused, whole layer
+# ------------------------------------------------------------------------------------------------
+def _gemm_tol(mag, k):
+    """fp32 accumulation of exact fp16 products in any order: |err| <= (K+1) * 2^-24 * sum|a*w|
+    (standard forward bound, gamma_K with u = 2^-24), plus one rounding of the result."""
+    return (k + 2) * 2.0 ** -24 * mag
+
+
+def _check_fused(cuda, oracle, m, n, k, bits, seed, with_bias=True, out_dtype=torch.float32):
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, seed)
+    kind = "gelu" if k > n else "ln"
+    _, thr = _cb(bits)
+    x = synth.make_activation(m, k, seed, kind)
+    a = oracle.act_quant_c(x.numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)
+    w = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, bits, 64, fma=True).astype(np.float16)
+    bias = synth.make_bias(n, seed) if with_bias else None
+    y64, mag = oracle.linear_f64_c(a, w, None if bias is None else bias.numpy())
+    y = ops.linear_fused(torch.from_numpy(a).to(cuda), packed.to(cuda), cb.to(cuda), center.to(cuda), scale.to(cuda),
+                         code_sum.to(cuda), None if bias is None else bias.to(cuda), bits, 64, out_dtype=out_dtype)
+    assert y.dtype == out_dtype and tuple(y.shape) == (m, n)
+    got = _np(y).astype(np.float64)
+    tol = _gemm_tol(mag, k)
+    if out_dtype == torch.float16:
+        tol = tol + np.abs(y64) * 2.0 ** -11 + 2.0 ** -25          # one fp16 rounding of the result
+    assert np.all(np.abs(got - y64) <= tol), float(np.max(np.abs(got - y64) / tol))
+    return y, y64
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("m,n,k", [(197, 768, 192), (197, 1152, 384), (197, 384, 384), (197, 1536, 384),
+                                   (197, 384, 1536), (1, 128, 64), (130, 200, 128), (64, 128, 64), (129, 129, 192)])
+def test_fused_gemm_vs_fp64(cuda, oracle, bits, m, n, k):
+    _check_fused(cuda, oracle, m, n, k, bits, seed=17)
+
+
+def test_fused_gemm_fp16_out_no_bias_and_large_tile(cuda, oracle):
+    _check_fused(cuda, oracle, 197, 384, 384, 4, seed=3, with_bias=False, out_dtype=torch.float16)
+    _check_fused(cuda, oracle, 2100, 1152, 384, 4, seed=5, out_dtype=torch.float16)   # takes the 128-row tile
+    _check_fused(cuda, oracle, 2100, 1152, 384, 3, seed=6, out_dtype=torch.float32)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_layer_otf_matches_stagewise(cuda, oracle, bits):
+    """arcq_linear_otf == stage 1 then fused GEMM, and its activation matches the oracle bit for bit."""
+    m, n, k = 197, 1152, 384
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 23)
+    _, thr = _cb(bits)
+    bias = synth.make_bias(n, 23)
+    x = synth.make_activation(m, k, 23).to(torch.float16)
+    d = lambda t: t.to(cuda)
+    ws = torch.empty((m, k), dtype=torch.float16, device=cuda)
+    y = ops.linear_otf(d(x), d(thr), d(cb), d(packed), d(cb), d(center), d(scale), d(code_sum), d(bias), bits, 64,
+                       out_dtype=torch.float16, x_hat_ws=ws)
+    want_xhat = oracle.act_quant_c(x.float().numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)
+    assert np.array_equal(_np(ws).view(np.uint16), want_xhat.view(np.uint16))
+    y2 = ops.linear_fused(ws, d(packed), d(cb), d(center), d(scale), d(code_sum), d(bias), bits, 64,
+                          out_dtype=torch.float16)
+    assert torch.equal(y, y2)
+    w = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, bits, 64).astype(np.float16)
+    y64, mag = oracle.linear_f64_c(want_xhat, w, bias.numpy())
+    tol = _gemm_tol(mag, k) + np.abs(y64) * 2.0 ** -11 + 2.0 ** -25
+    assert np.all(np.abs(_np(y).astype(np.float64) - y64) <= tol)
+    # against the fake-quant fp32 reference path (torch order, unrounded operands): fp16-level agreement
+    fq = oracle.fake_quant_linear(x.float(), synth.make_weight(n, k, 23), bias, thr, cb, thr, cb, 64, 1e-6)
+    cos = torch.nn.functional.cosine_similarity(y.float().cpu().flatten(), fq.flatten(), dim=0)
+    assert cos > 0.9999
+    assert (y.float().cpu() - fq).abs().max() < 2e-2 * fq.abs().max()
+
+
+# ------------------------------------------------------------------------------------------------
+# index-space linears
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("m,n,k", [(197, 768, 192), (33, 50, 128), (1, 1, 64)])
+def test_index_linears_bitexact(cuda, oracle, bits, m, n, k):
+    cb, packed_w, wc, ws, wcs = _packed_weight(oracle, n, k, bits, 41)
+    _, thr = _cb(bits)
+    x = synth.make_activation(m, k, 41)
+    bias = synth.make_bias(n, 41)
+    xa = oracle.act_quant_c(x.numpy(), thr, cb, bits, 64)
+    table = (cb.view(-1, 1) * (cb * 1.25).view(1, -1)).float().contiguous()      # asymmetric on purpose
+    wcodes = oracle.unpack_codes_u8_c(packed_w.numpy(), bits, k)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(cuda) if isinstance(a, np.ndarray) else a.to(cuda)
+    for b in (bias, None):
+        bn = None if b is None else b.numpy()
+        want = oracle.linear_forward_packed_c(xa["packed"], xa["center"], xa["scale"], xa["code_sum"], packed_w.numpy(),
+                                              wc, ws, wcs, table.numpy(), bn, bits, 64, k, n)
+        got = ops.arcq_linear_forward(d(xa["packed"]), d(xa["center"]), d(xa["scale"]), d(xa["code_sum"]),
+                                      d(packed_w), d(wc), d(ws), d(wcs), d(table), None if b is None else d(b),
+                                      bits, 64, k, n)
+        assert got.dtype == torch.float32 and np.array_equal(_np(got), want)
+        want8 = oracle.linear_forward_u8_c(xa["codes"], xa["center"], xa["scale"], xa["code_sum"], wcodes, wc, ws,
+                                           wcs, table.numpy(), bn, 64)
+        got8 = ops.arcq_linear_forward_u8(d(xa["codes"]), d(xa["center"]), d(xa["scale"]), d(xa["code_sum"]),
+                                          d(wcodes), d(wc), d(ws), d(wcs), d(table), None if b is None else d(b), 64)
+        assert np.array_equal(_np(got8), want8)
+
+
+# ------------------------------------------------------------------------------------------------
+# argument errors surface as RuntimeError with the reference's wording
+# ------------------------------------------------------------------------------------------------
+def test_error_paths(cuda):
+    cb, thr = _cb(4)
+    x = torch.zeros((4, 128), device=cuda)
+    with pytest.raises(RuntimeError, match="bits must be 2, 3, or 4"):
+        ops.quantize_activation(x, thr.to(cuda), cb.to(cuda), 5, 64)
+    with pytest.raises(RuntimeError, match="divisible by group_size"):
+        ops.quantize_activation(x, thr.to(cuda), cb.to(cuda), 4, 48)
+    with pytest.raises(RuntimeError, match="x must be float32"):
+        ops.quantize_activation(x.half(), thr.to(cuda), cb.to(cuda), 4, 64)
+    with pytest.raises(RuntimeError, match="x must be CUDA tensor"):
+        ops.quantize_activation(x.cpu(), thr.to(cuda), cb.to(cuda), 4, 64)
+    with pytest.raises(RuntimeError, match="codes must have shape"):
+        ops.pack_codes(torch.zeros(8, dtype=torch.int64, device=cuda), 4)
+    with pytest.raises(RuntimeError, match="packed must be uint8"):
+        ops.unpack_codes(torch.zeros((2, 4), dtype=torch.int32, device=cuda), 4, 8)
+    with pytest.raises(RuntimeError, match="only group_size 64"):
+        ops.linear_fused(torch.zeros((4, 128), dtype=torch.float16, device=cuda),
+                         torch.zeros((8, 64), dtype=torch.uint8, device=cuda), cb.to(cuda),
+                         torch.zeros((8, 4), device=cuda), torch.ones((8, 4), device=cuda),
+                         torch.zeros((8, 4), device=cuda), None, 4, 32)
+    # the raw C ABI reports the same conditions as negative codes without launching anything
+    from arcq_vit_amd import _lib
+    lib = _lib.load()
+    assert lib.arcq_pack_codes(0, 0, 4, 4, 7, 0) == -1
+    assert lib.arcq_act_quant(x.data_ptr(), 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 4, 128, 4, 48, 1e-6, 0) == -2
+    assert b"divisible" in lib.arcq_last_error()
+    assert lib.arcq_act_quant(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 4, 128, 4, 64, 1e-6, 0) == -3
+    torch.cuda.synchronize()

@@ -1,0 +1,323 @@
+"""Pins the oracle's arithmetic (stage 1, stage 2, linears) without running the reference.
+
+Every check is chosen so that a plausible slip in oracle/arcq_oracle.c (wrong tie direction, eps
+outside the sqrt, a dropped code-sum correction, a transposed product-table index, wrong tree
+pairing) fails it:
+
+* group statistics against an independently written serial fp32 evaluation
+  (``np.cumsum(dtype=float32)`` accumulates left to right) and against fp64;
+* threshold search against ``np.searchsorted(side="left")`` == ``torch.bucketize(right=False)``,
+  including exact ties built from the t values themselves;
+* reconstruction against exact rational arithmetic rounded once (fma) or twice (mul, add);
+* the two linear formulations against each other and against an fp64 matmul of the
+  reconstructed operands; the 32-lane tree against a vectorised fold.
+"""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from arcq_vit_amd import synth
+
+
+def _serial_sum_f32(a):
+    """Left-to-right fp32 sum along the last axis, written without an explicit loop."""
+    return np.cumsum(a.astype(np.float32), axis=-1, dtype=np.float32)[..., -1]
+
+
+def _stats_np(x, gs, eps):
+    rows, cols = x.shape
+    x3 = x.reshape(rows, cols // gs, gs).astype(np.float32)
+    mu = _serial_sum_f32(x3) / np.float32(gs)
+    d = x3 - mu[..., None]
+    var = _serial_sum_f32(d * d)
+    s = np.sqrt(var / np.float32(gs) + np.float32(eps), dtype=np.float32)
+    t = d / s[..., None]
+    return mu, s, t.reshape(rows, cols)
+
+
+def _round_f32(v: Fraction) -> np.float32:
+    """Nearest float32 to an exact rational, ties to even."""
+    f = np.float32(float(v))
+    cands = {f, np.nextafter(f, np.float32(np.inf)), np.nextafter(f, np.float32(-np.inf))}
+    best = None
+    for c in cands:
+        err = abs(Fraction(float(c)) - v)
+        even = (np.float32(c).view(np.uint32) & 1) == 0
+        key = (err, 0 if even else 1)
+        if best is None or key < best[0]:
+            best = (key, c)
+    return np.float32(best[1])
+
+
+def _inputs(bits, rows=37, cols=192, seed=0, kind="ln"):
+    cb = synth.quantile_codebook(bits)
+    thr = synth.midpoint_thresholds(cb)
+    x = synth.make_activation(rows, cols, seed, kind)
+    return x.numpy(), thr.numpy(), cb.numpy()
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("kind", ["ln", "gelu"])
+def test_stats_and_codes_match_independent_numpy(oracle, bits, kind):
+    x, thr, cb = _inputs(bits, kind=kind, seed=bits)
+    out = oracle.act_quant_c(x, thr, cb, bits, 64)
+    mu, s, t = _stats_np(x, 64, 1e-6)
+    assert np.array_equal(out["center"], mu)
+    assert np.array_equal(out["scale"], s)
+    codes = np.searchsorted(thr, t, side="left")          # number of thresholds strictly below t
+    assert np.array_equal(out["codes"], codes.astype(np.uint8))
+    assert np.array_equal(codes, torch.bucketize(torch.from_numpy(t), torch.from_numpy(thr)).numpy())
+    vals = cb[codes].reshape(x.shape[0], -1, 64)
+    assert np.array_equal(out["code_sum"], _serial_sum_f32(vals))
+    assert np.array_equal(out["packed"], oracle.pack_codes_np(codes, bits))
+    # fp64 agreement: catches eps outside the sqrt, population-vs-sample variance, missing centering
+    x64 = x.astype(np.float64).reshape(x.shape[0], -1, 64)
+    mu64 = x64.mean(-1)
+    s64 = np.sqrt(((x64 - mu64[..., None]) ** 2).mean(-1) + 1e-6)
+    assert np.allclose(out["center"], mu64, rtol=0, atol=2e-6)
+    assert np.allclose(out["scale"], s64, rtol=2e-6, atol=0)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_exact_threshold_ties_take_lower_code(oracle, bits):
+    """t == thr must NOT count that threshold (strict '>', EXT/arcq_activation_kernel.cu:67;
+    bucketize right=False, Q/dcarcq.py:552).  Thresholds are set to t values that occur."""
+    x, _, cb = _inputs(bits, rows=8, cols=128, seed=5)
+    _, _, t = _stats_np(x, 64, 1e-6)
+    levels = 1 << bits
+    picks = np.sort(np.unique(t.ravel()))[:: max(1, t.size // (levels - 1))][: levels - 1].astype(np.float32)
+    assert picks.size == levels - 1
+    out = oracle.act_quant_c(x, picks, cb, bits, 64)
+    want = np.searchsorted(picks, t, side="left")
+    assert np.array_equal(out["codes"], want.astype(np.uint8))
+    on_tie = np.isin(t, picks)
+    assert on_tie.sum() >= levels - 1
+    # with right=True (the wrong rule) every tied element would be one code higher
+    assert np.array_equal(np.searchsorted(picks, t, side="right")[on_tie], want[on_tie] + 1)
+
+
+def test_constant_group_and_eps_inside_sqrt(oracle):
+    cb = synth.quantile_codebook(4).numpy()
+    thr = synth.midpoint_thresholds(torch.from_numpy(cb)).numpy()
+    x = np.full((2, 64), 3.25, dtype=np.float32)
+    out = oracle.act_quant_c(x, thr, cb, 4, 64)
+    assert np.all(out["center"] == np.float32(3.25))
+    assert np.all(out["scale"] == np.sqrt(np.float32(1e-6)))      # sqrt(0 + eps), not sqrt(0) + eps
+    assert np.all(out["codes"] == np.searchsorted(thr, 0.0, side="left"))
+    assert np.allclose(out["x_hat"], 3.25, atol=1e-6)
+    out2 = oracle.act_quant_c(x, thr, cb, 4, 64, eps=1e-2)
+    assert np.all(out2["scale"] == np.sqrt(np.float32(1e-2)))
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_reconstruction_rounding_and_invariants(oracle, bits):
+    x, thr, cb = _inputs(bits, rows=5, cols=128, seed=11)
+    fused = oracle.act_quant_c(x, thr, cb, bits, 64, fma=True)
+    split = oracle.act_quant_c(x, thr, cb, bits, 64, fma=False)
+    codes = fused["codes"].astype(np.int64)
+    mu = np.repeat(fused["center"], 64, axis=1)
+    s = np.repeat(fused["scale"], 64, axis=1)
+    mean = np.repeat(fused["code_sum"] / np.float32(64), 64, axis=1)
+    d = (cb[codes] - mean).astype(np.float32)
+    assert np.array_equal(split["x_hat"], mu + s * d)                  # two roundings
+    want = np.empty_like(d)
+    for idx in np.ndindex(d.shape):                                    # one rounding, exact rational
+        want[idx] = _round_f32(Fraction(float(s[idx])) * Fraction(float(d[idx])) + Fraction(float(mu[idx])))
+    assert np.array_equal(fused["x_hat"], want)
+    # the split form rounds s*d first, so the two differ by at most ulp(s*d) + ulp(result)
+    bound = (np.spacing(np.abs(s * d)) + np.spacing(np.abs(want))).astype(np.float64)
+    assert np.all(np.abs(fused["x_hat"].astype(np.float64) - split["x_hat"]) <= bound)
+    # mean preservation: sum_j (cb[c_j] - S/gs) == 0 up to rounding, so mean(x_hat) == mu
+    g = fused["x_hat"].reshape(5, -1, 64).astype(np.float64)
+    assert np.allclose(g.mean(-1), fused["center"], atol=1e-6)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_serial_order_vs_torch_order_tie_audit(oracle, bits):
+    """The torch restatement reduces in torch's own order; codes may differ from the serial-order
+    oracle only where the exactly computed t sits within a few fp32 ulps of a threshold."""
+    x, thr, cb = _inputs(bits, rows=197, cols=384, seed=21)
+    c_out = oracle.act_quant_c(x, thr, cb, bits, 64)
+    codes_t, center_t, scale_t, _, _ = oracle.act_quant_torch(torch.from_numpy(x), torch.from_numpy(thr),
+                                                             torch.from_numpy(cb), 64)
+    codes_t = codes_t.numpy()
+    assert np.allclose(c_out["center"], center_t.numpy(), atol=1e-6)
+    assert np.allclose(c_out["scale"], scale_t.numpy(), rtol=1e-6)
+    diff = np.argwhere(c_out["codes"] != codes_t)
+    assert len(diff) <= x.size * 1e-3
+    x64 = x.astype(np.float64).reshape(x.shape[0], -1, 64)
+    mu = x64.mean(-1, keepdims=True)
+    t64 = ((x64 - mu) / np.sqrt(((x64 - mu) ** 2).mean(-1, keepdims=True) + 1e-6)).reshape(x.shape)
+    for r, c in diff:
+        assert abs(int(c_out["codes"][r, c]) - int(codes_t[r, c])) == 1
+        assert np.min(np.abs(thr.astype(np.float64) - t64[r, c])) < 4e-6 * max(1.0, abs(t64[r, c]))
+
+
+def test_torch_paths_agree_with_each_other(oracle):
+    """a8 (dequant_activation_torch), a14 (pcarcq_fake_quant) and a4 (quantize_weight_torch) are the
+    same formula; they must agree bit for bit on one host."""
+    cb = synth.quantile_codebook(4)
+    thr = synth.midpoint_thresholds(cb)
+    x = synth.make_activation(50, 192, 3)
+    a = oracle.dequant_activation_torch(x, thr, cb, 64)
+    b = oracle.pcarcq_fake_quant(x, thr, cb, 64, 1e-6)
+    assert torch.allclose(a, b, atol=1e-6)     # b = x + (x_hat - x) rounds differently, values equal to an ulp
+    codes, center, scale, code_sum = oracle.quantize_weight_torch(x, thr, cb, 64, 1e-6)
+    codes2, center2, scale2, code_sum2, _ = oracle.act_quant_torch(x, thr, cb, 64)
+    assert torch.equal(codes, codes2) and torch.equal(center, center2) and torch.equal(scale, scale2)
+    assert torch.equal(code_sum, code_sum2)
+    # padding branch of the quantizer (Q/dcarcq.py:522-527): 100 channels -> padded to 128
+    xp = synth.make_activation(4, 100, 4)
+    yp = oracle.pcarcq_fake_quant(xp, thr, cb, 64, 1e-6)
+    full = oracle.pcarcq_fake_quant(torch.nn.functional.pad(xp, (0, 28)), thr, cb, 64, 1e-6)
+    assert torch.equal(yp, full[:, :100])
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_weight_dequant_closed_form(oracle, bits):
+    cb = synth.quantile_codebook(bits)
+    thr = synth.midpoint_thresholds(cb)
+    w = synth.make_weight(24, 128, 7)
+    codes, center, scale, code_sum = oracle.quantize_weight_torch(w, thr, cb, 64, 1e-6)
+    packed = oracle.pack_codes_np(codes.numpy(), bits)
+    fused = oracle.weight_dequant_c(packed, cb, center, scale, code_sum, bits, 64, fma=True)
+    split = oracle.weight_dequant_c(packed, cb, center, scale, code_sum, bits, 64, fma=False)
+    cbn = cb.numpy()
+    c = np.repeat(center.numpy(), 64, axis=1)
+    s = np.repeat(scale.numpy(), 64, axis=1)
+    m = np.repeat(code_sum.numpy() / np.float32(64), 64, axis=1)
+    d = (cbn[codes.numpy()] - m).astype(np.float32)
+    assert np.array_equal(split, c + s * d)
+    for idx in list(np.ndindex(d.shape))[::7]:
+        assert fused[idx] == _round_f32(Fraction(float(d[idx])) * Fraction(float(s[idx])) + Fraction(float(c[idx])))
+    # torch restatement of a10 == the two-rounding variant, rounded to fp16
+    wt = oracle.unpack_weight_torch(torch.from_numpy(packed), cb, center, scale, code_sum, bits, 64)
+    assert np.array_equal(wt.numpy(), split.astype(np.float16))
+    # the reconstruction approximates the weight it encodes
+    rel_rms = np.sqrt(np.mean((fused - w.numpy()) ** 2)) / np.sqrt(np.mean(w.numpy() ** 2))
+    assert rel_rms < {4: 0.15, 3: 0.25, 2: 0.45}[bits]
+
+
+def _quantized_pair(oracle, bits, m=9, n=11, k=128, seed=31):
+    cb = synth.quantile_codebook(bits)
+    thr = synth.midpoint_thresholds(cb)
+    x = synth.make_activation(m, k, seed)
+    w = synth.make_weight(n, k, seed)
+    b = synth.make_bias(n, seed)
+    xa = oracle.act_quant_c(x.numpy(), thr, cb, bits, 64)
+    wcodes, wc, ws, wcs = oracle.quantize_weight_torch(w, thr, cb, 64, 1e-6)
+    return cb.numpy(), xa, wcodes.numpy(), wc.numpy(), ws.numpy(), wcs.numpy(), b.numpy()
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_linear_formulations_agree(oracle, bits):
+    cb, xa, wcodes, wc, ws, wcs, b = _quantized_pair(oracle, bits)
+    table = np.outer(cb, cb).astype(np.float32)
+    pw = oracle.pack_codes_np(wcodes, bits)
+    y_packed = oracle.linear_forward_packed_c(xa["packed"], xa["center"], xa["scale"], xa["code_sum"], pw, wc, ws,
+                                              wcs, table, b, bits, 64, 128, wcodes.shape[0])
+    y_u8 = oracle.linear_forward_u8_c(xa["codes"], xa["center"], xa["scale"], xa["code_sum"],
+                                      wcodes.astype(np.uint8), wc, ws, wcs, table, b, 64)
+    y_id = oracle.linear_identity_f64_np(xa["codes"], xa["center"], xa["scale"], xa["code_sum"], wcodes, wc, ws,
+                                         wcs, cb, cb, b, 64)
+    # reconstruct both operands in fp64 (no rounding to fp16) and multiply: the identity's left side
+    def recon(codes, c, s, cs):
+        v = cb.astype(np.float64)[codes].reshape(codes.shape[0], -1, 64)
+        return (c[..., None] + s[..., None] * (v - cs[..., None] / 64.0)).reshape(codes.shape[0], -1)
+    y_mm = recon(xa["codes"].astype(np.int64), xa["center"].astype(np.float64), xa["scale"].astype(np.float64),
+                 xa["code_sum"].astype(np.float64)) @ recon(wcodes, wc.astype(np.float64), ws.astype(np.float64),
+                                                           wcs.astype(np.float64)).T + b
+    scale = np.abs(y_mm).max()
+    assert np.abs(y_id - y_mm).max() < 1e-6 * scale        # fp32 product-table entries vs fp64 products
+    assert np.abs(y_packed - y_id).max() < 2e-7 * scale    # fp64 accumulate, rounded once to fp32
+    assert np.abs(y_u8 - y_id).max() < 1e-5 * scale        # fp32 accumulate
+
+
+def test_linear_packed_bitexact_vs_numpy_serial(oracle):
+    """fp64 serial accumulation, statement by statement (EXT/arcq_linear_kernel.cu:55-77)."""
+    bits = 3
+    cb, xa, wcodes, wc, ws, wcs, b = _quantized_pair(oracle, bits, m=4, n=5, k=192)
+    table = np.outer(cb, cb).astype(np.float32)
+    pw = oracle.pack_codes_np(wcodes, bits)
+    y = oracle.linear_forward_packed_c(xa["packed"], xa["center"], xa["scale"], xa["code_sum"], pw, wc, ws, wcs,
+                                       table, b, bits, 64, 192, 5)
+    xc = xa["codes"].astype(np.int64)
+    want = np.empty((4, 5), dtype=np.float32)
+    for r in range(4):
+        for o in range(5):
+            acc = np.float64(b[o])
+            for g in range(3):
+                sl = slice(64 * g, 64 * g + 64)
+                cross = np.cumsum(table[xc[r, sl], wcodes[o, sl]].astype(np.float64))[-1]
+                mu_term = np.float64(64) * np.float64(xa["center"][r, g]) * np.float64(wc[o, g])
+                res = np.float64(xa["scale"][r, g]) * np.float64(ws[o, g]) * (
+                    cross - (np.float64(xa["code_sum"][r, g]) * np.float64(wcs[o, g])) / np.float64(64))
+                acc = acc + (mu_term + res)
+            want[r, o] = np.float32(acc)
+    assert np.array_equal(y, want)
+    # a transposed table index would change the result: use an asymmetric table to prove the test sees it
+    cb2 = (cb * 1.7 + 0.3).astype(np.float32)
+    t_ab = np.outer(cb, cb2).astype(np.float32)
+    y_ab = oracle.linear_forward_packed_c(xa["packed"], xa["center"], xa["scale"], xa["code_sum"], pw, wc, ws, wcs,
+                                          t_ab, b, bits, 64, 192, 5)
+    y_ba = oracle.linear_forward_packed_c(xa["packed"], xa["center"], xa["scale"], xa["code_sum"], pw, wc, ws, wcs,
+                                          np.ascontiguousarray(t_ab.T), b, bits, 64, 192, 5)
+    assert not np.array_equal(y_ab, y_ba)
+    row0 = t_ab[xc[0, :64], wcodes[0, :64]].astype(np.float64).sum()      # table[x_code][w_code]
+    mu0 = 64.0 * xa["center"][0, 0] * wc[0, 0]
+    # first group of output (0,0) alone, recomputed with the documented index order
+    one = oracle.linear_forward_packed_c(xa["packed"][:1, :24], xa["center"][:1, :1], xa["scale"][:1, :1],
+                                         xa["code_sum"][:1, :1], pw[:1, :24], wc[:1, :1], ws[:1, :1], wcs[:1, :1],
+                                         t_ab, None, bits, 64, 64, 1)
+    want_one = mu0 + float(xa["scale"][0, 0]) * float(ws[0, 0]) * (
+        row0 - float(xa["code_sum"][0, 0]) * float(wcs[0, 0]) / 64.0)
+    assert abs(float(one[0, 0]) - want_one) <= 1e-6 * max(1.0, abs(want_one))
+
+
+@pytest.mark.parametrize("gs", [64, 32, 128])
+def test_linear_u8_bitexact_vs_vectorised_tree(oracle, gs):
+    """Lane l sums j = l, l+32, ...; partials fold with offsets 16, 8, 4, 2, 1
+    (EXT/arcq_linear_kernel.cu:176-185); closed form in fp32 (:187-197)."""
+    bits = 4
+    rng = np.random.default_rng(gs)
+    m, n, k = 3, 4, 2 * gs
+    cb = synth.quantile_codebook(bits).numpy()
+    table = np.outer(cb, cb * 1.3).astype(np.float32)
+    xc = rng.integers(0, 16, size=(m, k)).astype(np.uint8)
+    wcod = rng.integers(0, 16, size=(n, k)).astype(np.uint8)
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)
+    xm, xs, xS, wm, ws, wS, b = f(m, 2), np.abs(f(m, 2)), f(m, 2), f(n, 2), np.abs(f(n, 2)), f(n, 2), f(n)
+    y = oracle.linear_forward_u8_c(xc, xm, xs, xS, wcod, wm, ws, wS, table, b, gs)
+    want = np.empty((m, n), dtype=np.float32)
+    for r in range(m):
+        for o in range(n):
+            acc = np.float32(b[o])
+            for g in range(2):
+                p = table[xc[r, g * gs:(g + 1) * gs].astype(np.int64), wcod[o, g * gs:(g + 1) * gs].astype(np.int64)]
+                lanes = np.zeros(32, dtype=np.float32)
+                for start in range(0, gs, 32):                      # lane l: j = l, l+32, ... in order
+                    lanes = lanes + p[start:start + 32]
+                for off in (16, 8, 4, 2, 1):
+                    lanes[:off] = lanes[:off] + lanes[off:2 * off]
+                cross = lanes[0]
+                mu_term = np.float32(gs) * xm[r, g] * wm[o, g]
+                res = xs[r, g] * ws[o, g] * (cross - (xS[r, g] * wS[o, g]) / np.float32(gs))
+                acc = np.float32(acc + np.float32(mu_term + res))
+            want[r, o] = acc
+    assert np.array_equal(y, want)
+
+
+def test_linear_f64_and_error_scale(oracle):
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal((5, 128)).astype(np.float16)
+    w = rng.standard_normal((7, 128)).astype(np.float16)
+    b = rng.standard_normal(7).astype(np.float32)
+    y, mag = oracle.linear_f64_c(a, w, b)
+    ref = a.astype(np.float64) @ w.astype(np.float64).T + b
+    assert np.allclose(y, ref, rtol=1e-13, atol=1e-13)
+    assert np.allclose(mag, np.abs(a.astype(np.float64))[:, None, :].__mul__(np.abs(w.astype(np.float64))[None]).sum(-1)
+                       + np.abs(b), rtol=1e-13)
+    y2, _ = oracle.linear_f64_c(a, w, None)
+    assert np.allclose(y2, ref - b, rtol=1e-13, atol=1e-13)
