@@ -226,7 +226,7 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
     if (x_hat) {
         const float code_mean = sum_codes / 64.0f;
 #pragma unroll
-        for (int j = 0; j < 64; ++j) col[j] = __fmaf_rn(s, xv[j] - code_mean, mu);
+        for (int j = 0; j < 64; ++j) col[j] = fma_f32(s, xv[j] - code_mean, mu);
         __syncthreads();
         store_tile<TOUT>(x_hat, elem0, elem_end, tile, lane);
     }
@@ -294,7 +294,7 @@ act_quant_generic_kernel(const TIN *__restrict__ x, const float *__restrict__ th
             const float t = (to_float(xg[j]) - mu) / s;
             int c = 0;
             while (c < levels - 1 && t > thr[c]) ++c;
-            x_hat[g * gs + j] = from_float<TOUT>(__fmaf_rn(s, cb[c] - code_mean, mu));
+            x_hat[g * gs + j] = from_float<TOUT>(fma_f32(s, cb[c] - code_mean, mu));
         }
     }
 }

@@ -48,6 +48,16 @@ __device__ __forceinline__ uint32_t load_codes8(const uint8_t *__restrict__ p)
     }
 }
 
+// fma with the fp32 rounding made visible.  Without the barrier the compiler fuses a following
+// float->half conversion into v_fma_mixlo_f16, which rounds the exact result once to fp16; the
+// contract here (and what the reference's kernels do) is round to fp32, then round to fp16.
+__device__ __forceinline__ float fma_f32(float a, float b, float c)
+{
+    float v = __fmaf_rn(a, b, c);
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
 __device__ __forceinline__ float to_float(float v) { return v; }
 __device__ __forceinline__ float to_float(__half v) { return __half2float(v); }
 

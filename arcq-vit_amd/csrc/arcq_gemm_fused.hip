@@ -114,7 +114,7 @@ gemm_fused_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, 
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
                 const int code = code_at<BITS>(b_reg, q4 * 8 + q);
-                hv[q] = static_cast<_Float16>(__fmaf_rn(lut[code * 64 + lane] - b_m, b_s, b_c));
+                hv[q] = static_cast<_Float16>(fma_f32(lut[code * 64 + lane] - b_m, b_s, b_c));
             }
             *reinterpret_cast<half8_t *>(dst + q4 * 8) = hv;
         }

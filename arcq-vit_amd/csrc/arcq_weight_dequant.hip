@@ -49,7 +49,7 @@ weight_dequant8_kernel(const uint8_t *__restrict__ packed, const float *__restri
             g_prev = g;
         }
         const int code = (w >> (BITS * q)) & (L - 1);
-        v[q] = __fmaf_rn(lut[code * 64 + lane] - m, s, c);
+        v[q] = fma_f32(lut[code * 64 + lane] - m, s, c);
     }
     TOUT *dst = out + n * K + k0;
     if constexpr (sizeof(TOUT) == 2) {
@@ -80,7 +80,7 @@ weight_dequant_generic_kernel(const uint8_t *__restrict__ packed, const float *_
     const int64_t g = k / gs;
     const int code = get_code(packed + n * packed_cols(K, bits), k, bits);
     const float m = code_sum[n * groups + g] / static_cast<float>(gs);
-    out[idx] = from_float<TOUT>(__fmaf_rn(cb[code] - m, scale[n * groups + g], center[n * groups + g]));
+    out[idx] = from_float<TOUT>(fma_f32(cb[code] - m, scale[n * groups + g], center[n * groups + g]));
 }
 
 template <typename TOUT>

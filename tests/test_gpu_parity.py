@@ -119,8 +119,9 @@ def test_stage1_ties_constant_and_extremes(cuda, oracle):
     x[3] *= 1.0e-4
     ref0 = oracle.act_quant_c(x.numpy(), synth.midpoint_thresholds(cb), cb, bits, 64)
     t = ((x.numpy().reshape(16, 2, 64) - ref0["center"][..., None]) / ref0["scale"][..., None]).astype(np.float32)
-    thr = torch.from_numpy(np.sort(np.unique(t))[5::137][:15].copy())
-    assert thr.numel() == 15
+    u = np.sort(np.unique(t))
+    thr = torch.from_numpy(u[np.linspace(5, u.size - 6, 15).astype(np.int64)].copy())
+    assert thr.numel() == 15 and bool((thr[1:] > thr[:-1]).all())
     ref = oracle.act_quant_c(x.numpy(), thr, cb, bits, 64)
     packed, center, scale, code_sum = ops.quantize_activation(x.to(cuda), thr.to(cuda), cb.to(cuda), bits, 64)
     assert np.array_equal(_np(packed), ref["packed"])
