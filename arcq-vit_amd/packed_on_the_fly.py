@@ -76,21 +76,27 @@ class ARCQPackedLinearOnTheFly(nn.Module):
                    packed_layer.weight_scale, packed_layer.weight_code_sum, packed_layer.activation_codebook,
                    packed_layer.activation_thresholds, packed_layer.bits, packed_layer.group_size, b)
 
+    _FP32_BUFFERS = ("weight_codebook", "weight_center", "weight_scale", "weight_code_sum",
+                     "activation_codebook", "activation_thresholds", "bias_tensor")
+
     def _apply(self, fn, *args, **kwargs):
-        # model.half() must not narrow the fp32 metadata (the reference undoes it afterwards,
-        # scripts/benchmark_arcq_on_the_fly.py:63-85); keep those buffers fp32 through any cast.
+        # model.half() must not narrow the fp32 metadata.  (The reference casts the whole model and
+        # then widens these buffers again, scripts/benchmark_arcq_on_the_fly.py:63-85, which leaves
+        # them rounded to fp16.)  Device moves still apply; dtype changes of these buffers do not.
+        keep = {n: self._buffers[n] for n in self._FP32_BUFFERS if self._buffers.get(n) is not None}
         super()._apply(fn, *args, **kwargs)
-        for name in ("weight_codebook", "weight_center", "weight_scale", "weight_code_sum",
-                     "activation_codebook", "activation_thresholds", "bias_tensor"):
-            buf = self._buffers.get(name)
-            if buf is not None and buf.is_floating_point() and buf.dtype != torch.float32:
-                self._buffers[name] = buf.float()
+        for name, orig in keep.items():
+            new = self._buffers[name]
+            if new.dtype != orig.dtype:
+                self._buffers[name] = orig.to(device=new.device)
         return self
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         original_shape = x.shape
         if original_shape[-1] != self.in_features:
             raise ValueError(f"expected last dim {self.in_features}, got {original_shape[-1]}")
+        if not x.is_cuda or not self.packed_weight_codes.is_cuda:
+            raise RuntimeError("x and the layer's buffers must be CUDA tensors (there is no CPU forward)")
         x2 = x.reshape(-1, self.in_features)
         if x2.dtype not in (torch.float16, torch.float32):
             x2 = x2.to(torch.float16)

@@ -1,0 +1,322 @@
+"""CPU-side tests: golden fixtures vs the oracle, the C-ABI library's exports, the module layer
+(buffer layout, conversion, checkpoint loading, error behaviour) and the synthetic generators.
+Nothing here launches a kernel."""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import arcq_vit_amd as A
+from arcq_vit_amd import synth
+from arcq_vit_amd.vit import build_fakequant_vit
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+# ------------------------------------------------------------------------------------------------
+# golden fixtures
+# ------------------------------------------------------------------------------------------------
+def test_layout_vectors(oracle):
+    vecs = json.load(open(os.path.join(GOLDEN, "layout_vectors.json")))["vectors"]
+    for v in vecs:
+        codes = np.array([v["codes"]], dtype=np.int64)
+        assert oracle.pack_codes_c(codes, v["bits"]).tolist() == [v["bytes"]]
+        assert oracle.pack_codes_np(codes, v["bits"]).tolist() == [v["bytes"]]
+        assert A.pack_codes_py(torch.from_numpy(codes), v["bits"]).tolist() == [v["bytes"]]
+        assert oracle.unpack_codes_c(np.array([v["bytes"]], dtype=np.uint8), v["bits"], len(v["codes"])).tolist() == [v["codes"]]
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_oracle_reproduces_golden(oracle, bits):
+    g = np.load(os.path.join(GOLDEN, f"arcq_w{bits}a{bits}_g64.npz"))
+    a32 = oracle.act_quant_c(g["x"], g["thresholds"], g["codebook"], bits, 64)
+    for k in ("packed", "codes", "center", "scale", "code_sum", "x_hat"):
+        assert np.array_equal(a32[k], g[f"a32_{k}"]), k
+    a16 = oracle.act_quant_c(g["x_f16"].astype(np.float32), g["thresholds"], g["codebook"], bits, 64)
+    assert np.array_equal(a16["packed"], g["a16_packed"])
+    assert np.array_equal(a16["x_hat"].astype(np.float16).view(np.uint16), g["a16_x_hat_f16"].view(np.uint16))
+    wd = oracle.weight_dequant_c(g["w_packed"], g["codebook"], g["w_center"], g["w_scale"], g["w_code_sum"], bits, 64)
+    assert np.array_equal(wd.astype(np.float16).view(np.uint16), g["w_dequant_f16"].view(np.uint16))
+    y64, mag = oracle.linear_f64_c(g["a16_x_hat_f16"], g["w_dequant_f16"], g["bias"])
+    assert np.array_equal(y64, g["y_f64"]) and np.array_equal(mag, g["y_abs_sum"])
+    yp = oracle.linear_forward_packed_c(g["a32_packed"], g["a32_center"], g["a32_scale"], g["a32_code_sum"],
+                                        g["w_packed"], g["w_center"], g["w_scale"], g["w_code_sum"],
+                                        g["product_table"], g["bias"], bits, 64, 128, 16)
+    assert np.array_equal(yp, g["y_index_packed"])
+    yu = oracle.linear_forward_u8_c(g["a32_codes"], g["a32_center"], g["a32_scale"], g["a32_code_sum"], g["w_codes"],
+                                    g["w_center"], g["w_scale"], g["w_code_sum"], g["product_table"], g["bias"], 64)
+    assert np.array_equal(yu, g["y_index_u8"])
+    # the fixture's first group is constant: s = sqrt(eps)
+    assert g["a32_scale"][0, 0] == np.sqrt(np.float32(1e-6))
+
+
+# ------------------------------------------------------------------------------------------------
+# C ABI
+# ------------------------------------------------------------------------------------------------
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "arcq_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(arcq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert len(names) >= 11 and "arcq_linear_fused" in names and "arcq_act_quant" in names
+    lib = A._lib.load()
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in include/arcq_hip.h but not exported"
+    assert sorted(A._lib.EXPORTED_SYMBOLS) == names
+    assert lib.arcq_version() == 100
+    # no torch / pybind types leak into the ABI: the library links against the HIP runtime only
+    deps = os.popen(f"ldd {A._lib.LIB_PATH}").read()
+    assert "libtorch" not in deps and "libc10" not in deps and "python" not in deps.lower()
+
+
+def test_abi_argument_errors_need_no_gpu():
+    """Validation happens before any HIP call, so these are safe on a machine without a GPU."""
+    lib = A._lib.load()
+    assert lib.arcq_pack_codes(0, 0, 4, 4, 7, 0) == -1
+    assert b"bits must be 2, 3, or 4" in lib.arcq_last_error()
+    assert lib.arcq_unpack_codes(0, 0, -1, 4, 4, 0) == -4
+    assert lib.arcq_pack_codes(0, 0, 4, 4, 4, 0) == -3                       # NULL tensors, non-empty shape
+    assert lib.arcq_pack_codes(0, 0, 0, 4, 4, 0) == 0                        # empty is fine
+    assert lib.arcq_act_quant(8, 0, 8, 8, 0, 0, 0, 0, 0, 0, 0, 4, 128, 4, 48, 1e-6, 0) == -2
+    assert b"in_features must be divisible by group_size" in lib.arcq_last_error()
+    assert lib.arcq_act_quant(8, 7, 8, 8, 0, 0, 0, 0, 0, 0, 0, 4, 128, 4, 64, 1e-6, 0) == -5
+    assert lib.arcq_weight_dequant(8, 8, 8, 8, 8, 8, 9, 4, 128, 4, 64, 0) == -5
+    assert lib.arcq_linear_fused(16, 16, 8, 8, 8, 8, 0, 16, 1, 4, 4, 128, 4, 32, 0) == -6
+    assert b"group_size 64" in lib.arcq_last_error()
+    assert lib.arcq_linear_fused(8, 16, 8, 8, 8, 8, 0, 16, 1, 4, 4, 128, 4, 64, 0) == -7  # misaligned x_hat
+    assert lib.arcq_linear_forward_packed(*([8] * 11), 4, 4, 128, 4, 64, 8, 0) == -4      # 8 levels < 2^4
+    assert lib.arcq_linear_otf(8, 0, 8, 8, 8, 8, 8, 8, 8, 0, 8, 16, 1, 4, 4, 128, 4, 64, 0) == -5  # fp32 x aliasing ws
+    with pytest.raises(RuntimeError, match="aliasing|alias"):
+        A._lib.check(-5)
+
+
+# ------------------------------------------------------------------------------------------------
+# module layer
+# ------------------------------------------------------------------------------------------------
+def _source(in_f=128, out_f=24, bias=True, bits=4, gs=64, seed=1):
+    torch.manual_seed(seed)
+    src = A.QuantLinearPCARCQ(in_f, out_f, bias, bits, bits, gs)
+    cb = synth.quantile_codebook(bits)
+    src.act_quant.set_codebook(cb * 1.1)
+    src.weight_quant.set_codebook(cb)
+    with torch.no_grad():
+        src.linear.weight.copy_(synth.make_weight(out_f, in_f, seed))
+        if bias:
+            src.linear.bias.copy_(synth.make_bias(out_f, seed))
+    return src.eval()
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("fmt", ["packed", "u8", "dequant_gemm", "hip_fused"])
+def test_packed_linear_buffers(oracle, bits, fmt):
+    """Buffer names, shapes, dtypes and contents (FQ/arcq_packed_linear.py:106-151)."""
+    src = _source(bits=bits)
+    layer = A.ARCQPackedLinear(src, runtime_code_format=fmt)
+    n, k, g, L = 24, 128, 2, 1 << bits
+    sd = layer.state_dict()
+    assert list(sd) == ["packed_weight_codes", "weight_codes_u8", "weight_dequant", "weight_center", "weight_scale",
+                        "weight_code_sum", "weight_codebook", "activation_codebook", "activation_thresholds",
+                        "product_table", "bias"]
+    want_shapes = {"packed_weight_codes": (n, k * bits // 8), "weight_center": (n, g), "weight_scale": (n, g),
+                   "weight_code_sum": (n, g), "weight_codebook": (L,), "activation_codebook": (L,),
+                   "activation_thresholds": (L - 1,), "product_table": (L, L), "bias": (n,),
+                   "weight_codes_u8": (n, k) if fmt == "u8" else (0,),
+                   "weight_dequant": (n, k) if fmt == "dequant_gemm" else (0,)}
+    for name, shape in want_shapes.items():
+        assert tuple(sd[name].shape) == shape, name
+    assert sd["packed_weight_codes"].dtype == torch.uint8 and sd["weight_codes_u8"].dtype == torch.uint8
+    assert sd["weight_dequant"].dtype == torch.float16
+    assert all(sd[k_].dtype == torch.float32 for k_ in ("weight_center", "weight_scale", "weight_code_sum",
+                                                        "weight_codebook", "product_table", "bias"))
+    # contents: the oracle's restatement of the offline encoder + packer
+    w_thr = src.weight_quant._pc_thresholds
+    codes, center, scale, code_sum = oracle.quantize_weight_torch(src.linear.weight, w_thr, src.weight_quant._pc_cb,
+                                                                 64, 1e-6)
+    assert np.array_equal(sd["packed_weight_codes"].numpy(), oracle.pack_codes_np(codes.numpy(), bits))
+    assert torch.equal(sd["weight_center"], center) and torch.equal(sd["weight_scale"], scale)
+    assert torch.equal(sd["weight_code_sum"], code_sum)
+    assert torch.equal(sd["product_table"], src.act_quant._pc_cb.view(-1, 1) * src.weight_quant._pc_cb.view(1, -1))
+    assert torch.equal(sd["activation_thresholds"], src.act_quant._pc_thresholds)
+    assert torch.equal(sd["bias"], src.linear.bias.detach())
+    if fmt == "u8":
+        assert np.array_equal(sd["weight_codes_u8"].numpy(), codes.numpy().astype(np.uint8))
+    if fmt == "dequant_gemm":
+        want = oracle.unpack_weight_torch(sd["packed_weight_codes"], sd["weight_codebook"], center, scale, code_sum,
+                                          bits, 64)
+        assert torch.equal(sd["weight_dequant"], want)
+    # attributes and accounting (:148-151, :224-241)
+    assert (layer.in_features, layer.out_features, layer.group_size, layer.bits, layer.act_bits) == (k, n, 64, bits, bits)
+    assert layer.packed_weight_bytes == n * k * bits // 8 and layer.weight_meta_floats == 3 * n * g
+    assert layer.estimated_storage_bytes() == n * k * bits // 8 + 4 * (3 * n * g + 3 * L - 1 + L * L + n)
+    assert layer.runtime_cache_bytes() == (n * k if fmt == "u8" else 2 * n * k if fmt == "dequant_gemm" else 0)
+    assert f"bits={bits}" in layer.extra_repr() and f"runtime_code_format={fmt}" in layer.extra_repr()
+
+
+def test_packed_linear_no_bias_and_errors():
+    layer = A.ARCQPackedLinear(_source(bias=False))
+    assert layer.bias.numel() == 0 and layer.bias.dtype == torch.float32
+    with pytest.raises(ValueError, match="runtime_code_format"):
+        A.ARCQPackedLinear(_source(), "int8")
+    with pytest.raises(TypeError, match="source.linear.weight"):
+        A.ARCQPackedLinear(nn.Identity())
+    no_q = nn.Module()
+    no_q.linear = nn.Linear(64, 8)
+    with pytest.raises(TypeError, match="act_quant and weight_quant"):
+        A.ARCQPackedLinear(no_q)
+    mixed = A.QuantLinearPCARCQ(64, 8, True, 4, 3)
+    mixed.act_quant.set_codebook(synth.quantile_codebook(3))
+    mixed.weight_quant.set_codebook(synth.quantile_codebook(4))
+    with pytest.raises(ValueError, match="W bits == A bits"):
+        A.ARCQPackedLinear(mixed)
+    five = A.QuantLinearPCARCQ(64, 8, True, 5, 5)
+    with pytest.raises(ValueError, match="supports bits 2/3/4"):
+        A.ARCQPackedLinear(five)
+    with pytest.raises(ValueError, match="divisible by group_size"):
+        A.ARCQPackedLinear(A.QuantLinearPCARCQ(100, 8, True, 4, 4))
+    empty = A.QuantLinearPCARCQ(64, 8, True, 4, 4)
+    with pytest.raises(ValueError, match="is missing; load a checkpoint"):
+        A.ARCQPackedLinear(empty)
+    wrong = A.QuantLinearPCARCQ(64, 8, True, 4, 4)
+    wrong.act_quant._pc_cb = torch.zeros(8)
+    wrong.act_quant._pc_thresholds = torch.zeros(7)
+    wrong.weight_quant.set_codebook(synth.quantile_codebook(4))
+    with pytest.raises(ValueError, match="codebook size must be 16"):
+        A.ARCQPackedLinear(wrong)
+    with pytest.raises(ValueError, match="expected last dim"):
+        layer(torch.zeros(2, 3))
+
+
+def test_forward_has_no_cpu_fallback():
+    """On CPU tensors every forward must fail loudly rather than compute something else."""
+    x = torch.zeros(2, 128)
+    for fmt in ("packed", "u8", "dequant_gemm", "hip_fused"):
+        with pytest.raises(RuntimeError, match="CUDA tensor"):
+            A.ARCQPackedLinear(_source(), fmt)(x)
+    otf = A.ARCQPackedLinearOnTheFly.from_packed(A.ARCQPackedLinear(_source()))
+    with pytest.raises(RuntimeError, match="CUDA"):
+        otf(x)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        A.pack_codes(torch.zeros(2, 8, dtype=torch.int64), 4)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        A.quantize_activation(x, torch.zeros(15), torch.zeros(16), 4, 64)
+
+
+def test_on_the_fly_module():
+    packed = A.ARCQPackedLinear(_source())
+    otf = A.ARCQPackedLinearOnTheFly.from_packed(packed)
+    assert list(otf.state_dict()) == ["packed_weight_codes", "weight_codebook", "weight_center", "weight_scale",
+                                      "weight_code_sum", "activation_codebook", "activation_thresholds", "bias_tensor"]
+    assert otf.groups == 2 and otf.bits == 4 and otf.group_size == 64
+    assert otf.packed_weight_codes.data_ptr() == packed.packed_weight_codes.data_ptr()     # shared, not copied
+    want_mb = sum(b.numel() * b.element_size() for b in otf.buffers()) / 1024 / 1024
+    assert abs(otf.estimated_persistent_mb() - want_mb) < 1e-12
+    otf.half()                                                                            # half-chain cast
+    assert all(b.dtype == torch.float32 for n, b in otf.named_buffers() if n != "packed_weight_codes")
+    nb = A.ARCQPackedLinearOnTheFly(128, 24, False, packed.packed_weight_codes, packed.weight_codebook,
+                                    packed.weight_center, packed.weight_scale, packed.weight_code_sum,
+                                    packed.activation_codebook, packed.activation_thresholds, 4, 64, None)
+    assert nb.bias_tensor.numel() == 0
+    with pytest.raises(ValueError, match="packed_weight_codes has shape"):
+        A.ARCQPackedLinearOnTheFly(256, 24, False, packed.packed_weight_codes, packed.weight_codebook,
+                                   packed.weight_center, packed.weight_scale, packed.weight_code_sum,
+                                   packed.activation_codebook, packed.activation_thresholds, 4, 64, None)
+
+
+def test_convert_model_and_checkpoint_roundtrip(tmp_path, oracle):
+    vit = build_fakequant_vit("deit_tiny", 4, num_classes=10)
+    assert sum(m.__class__.__name__ == "QuantLinearPCARCQ" for m in vit.modules()) == 48
+    A.convert_arcq_linear_to_packed(vit, "packed")
+    assert A.count_packed_linear(vit) == 48
+    assert A.count_packed_linear(A.convert_arcq_linear_to_packed(vit, "dequant_gemm")) == 48   # 2nd pass: nothing left
+    assert all(m.runtime_code_format == "packed" for m in vit.modules() if isinstance(m, A.ARCQPackedLinear))
+    sd = vit.state_dict()
+    assert "blocks.3.mlp.fc1.packed_weight_codes" in sd and "blocks.0.attn.qkv.product_table" in sd
+    assert tuple(sd["blocks.3.mlp.fc1.packed_weight_codes"].shape) == (768, 96)
+    path = tmp_path / "deit_tiny_w4a4_packed.pt"
+    torch.save({"module." + k: v for k, v in sd.items()}, path)                # DDP-style prefix
+
+    hp = A.infer_packed_hparams(sd["blocks.3.mlp.fc2.packed_weight_codes"], sd["blocks.3.mlp.fc2.weight_center"],
+                                sd["blocks.3.mlp.fc2.weight_codebook"])
+    assert hp == {"in_features": 768, "out_features": 192, "bits": 4, "group_size": 64}
+
+    from arcq_vit_amd.vit import VisionTransformer
+    fresh = VisionTransformer(192, 12, 3, 768, num_classes=10)
+    loaded = torch.load(path, weights_only=True)
+    A.load_packed_state_dict(fresh, loaded, on_the_fly=True)
+    otf = fresh.blocks[3].mlp.fc1
+    assert isinstance(otf, A.ARCQPackedLinearOnTheFly) and (otf.in_features, otf.out_features) == (192, 768)
+    assert torch.equal(otf.packed_weight_codes, sd["blocks.3.mlp.fc1.packed_weight_codes"])
+    assert torch.equal(otf.bias_tensor, sd["blocks.3.mlp.fc1.bias"])
+    assert torch.equal(fresh.pos_embed, vit.pos_embed) and torch.equal(fresh.head.weight, vit.head.weight)
+    # the on-the-fly spelling (bias_tensor) loads too, into either module kind
+    fresh2 = VisionTransformer(192, 12, 3, 768, num_classes=10)
+    A.load_packed_state_dict(fresh2, fresh.state_dict(), on_the_fly=False, runtime_code_format="u8")
+    pl = fresh2.blocks[0].attn.qkv
+    assert isinstance(pl, A.ARCQPackedLinear) and pl.weight_codes_u8.shape == (576, 192)
+    assert torch.equal(pl.bias, sd["blocks.0.attn.qkv.bias"])
+    bad = dict(sd)
+    bad["blocks.99.attn.qkv.packed_weight_codes"] = sd["blocks.0.attn.qkv.packed_weight_codes"]
+    with pytest.raises(KeyError, match="blocks.99"):
+        A.load_packed_state_dict(VisionTransformer(192, 12, 3, 768, num_classes=10), bad)
+
+
+def test_three_bit_conversion_sizes():
+    layer = A.ARCQPackedLinear(_source(in_f=384, out_f=16, bits=3))
+    assert tuple(layer.packed_weight_codes.shape) == (16, 144)
+    hp = A.infer_packed_hparams(layer.packed_weight_codes, layer.weight_center, layer.weight_codebook)
+    assert hp == {"in_features": 384, "out_features": 16, "bits": 3, "group_size": 64}
+    with pytest.raises(ValueError):
+        A.infer_packed_hparams(layer.packed_weight_codes, layer.weight_center, torch.zeros(5))
+
+
+def test_fake_quant_source_matches_oracle(oracle):
+    src = _source(in_f=192, out_f=32, bits=4)
+    x = synth.make_activation(50, 192, 2)
+    want = oracle.fake_quant_linear(x, src.linear.weight.detach(), src.linear.bias.detach(),
+                                    src.act_quant._pc_thresholds, src.act_quant._pc_cb,
+                                    src.weight_quant._pc_thresholds, src.weight_quant._pc_cb, 64, 1e-6)
+    assert torch.equal(src(x), want)
+    x3 = x.reshape(5, 10, 192)
+    assert torch.equal(src(x3).reshape(50, 32), want)            # any leading dims
+    q = A.FrozenARCQQuantizer(4, 64)
+    with pytest.raises(RuntimeError, match="no compiled codebook"):
+        q(x)
+    q8 = A.FrozenARCQQuantizer(8, 64)
+    assert q8(x) is x                                              # bits >= 8 is a pass-through (Q/dcarcq.py:513-514)
+
+
+# ------------------------------------------------------------------------------------------------
+# synthetic generators and work accounting
+# ------------------------------------------------------------------------------------------------
+def test_synth():
+    for bits in (2, 3, 4):
+        cb = synth.quantile_codebook(bits)
+        thr = synth.midpoint_thresholds(cb)
+        assert cb.dtype == torch.float32 and cb.numel() == 1 << bits and bool((cb[1:] > cb[:-1]).all())
+        assert torch.allclose(cb, -cb.flip(0), atol=1e-6) and thr.numel() == cb.numel() - 1
+    assert abs(float(synth.quantile_codebook(4)[-1]) - 1.8627) < 1e-3
+    x = synth.make_activation(2000, 384, 0)
+    frac = float((x.abs() == 8.0).float().mean())
+    assert 0.003 < frac < 0.007 and torch.equal(x, synth.make_activation(2000, 384, 0))
+    g = synth.make_activation(2000, 384, 0, "gelu")
+    assert float(g.min()) > -0.2 and float(g.mean()) > 0.2
+    w = synth.make_weight(256, 256, 0)
+    assert abs(float(w.std()) - 0.02) < 1e-3
+    img = synth.make_images(2, 0)
+    assert tuple(img.shape) == (2, 3, 224, 224) and -2.2 < float(img.min()) and float(img.max()) < 2.7
+    # algorithmic bytes/flops of the DeiT-S qkv shape at batch 1 and batch 64
+    assert synth.algorithmic_bytes(197, 1152, 384, 4) == 914108
+    assert synth.algorithmic_bytes(12608, 1152, 384, 4) == 39040700
+    assert synth.algorithmic_bytes(197, 384, 1536, 4) == 1163708
+    assert synth.algorithmic_bytes(197, 1152, 384, 3) == 858716
+    assert synth.algorithmic_flops(12608, 1536, 384) == 2 * 12608 * 1536 * 384
+    assert [s[1:] for s in synth.block_linear_shapes("deit_small")] == [(384, 1152), (384, 384), (384, 1536), (1536, 384)]
