@@ -5,115 +5,139 @@
 // Per group of gs input channels of one token:
 //   mu = (x0 + x1 + ... ) / gs           serial, left to right
 //   s  = sqrt((sum_j (x_j - mu)^2) / gs + eps)
-//   t_j = (x_j - mu) / s                 IEEE divide
+//   t_j = (x_j - mu) / s                 correctly rounded
 //   code_j = number of leading thresholds with t_j > thr[i]
 //   S = sum_j cb[code_j]                 serial
 //   x_hat_j = fma(s, cb[code_j] - S/gs, mu)
 //
-// Data layout.  x is [rows, cols] with cols = G*gs, so the groups of the whole
-// tensor are consecutive 64-element runs of one flat array and "group index"
-// is simply flat_offset/64.  The gs == 64 kernel gives every lane ONE group (so
-// the serial sums are plain register loops, 64 independent chains per wave) and
-// moves data between the coalesced global layout and that lane-per-group layout
-// through an LDS tile of 64 groups x 64 elements, padded to a row stride of 65
-// floats so that the per-lane column reads hit 64 different banks.
+// gs == 64 kernel.  x is [rows, G*64], so the groups of the whole tensor are consecutive 64-element
+// runs of one flat array.  A wave owns a tile of 64 consecutive groups and gives every lane ONE group,
+// so the serial sums are plain register loops (64 independent chains per wave).  Data moves between
+// the coalesced global layout (16-byte accesses) and the lane-per-group layout through a per-wave LDS
+// tile whose row stride is odd in dwords (33 for fp16, 65 for fp32), which makes both the row-wise
+// 16-byte phase and the per-lane column phase bank-conflict free.
+//
+// Two things keep the per-element VALU work low without changing a single result bit:
+//  * t = d/s is evaluated as three fused corrections of d * RN(1/s) (q0 = d*y; e = fma(-s,q,d);
+//    q = fma(e,y,q), twice).  With y the correctly rounded reciprocal and the second residual exact
+//    this yields the correctly rounded quotient (Markstein); lanes whose s or mu fall outside the
+//    range where no intermediate can under/overflow take the plain divide instead.
+//  * the threshold search is one table lookup plus one compare: t is mapped by a monotone function
+//    to one of 512 buckets over [-8, 8) (|t| < 8 always, since s^2 >= d_j^2/64); a bucket stores how
+//    many thresholds lie in lower buckets and the single threshold inside it.  Monotonicity makes
+//    base + (t > thr_in_bucket) equal to the count of thresholds below t.  If two thresholds share a
+//    bucket, or the thresholds are not sorted, the kernel falls back to the compare chain.
 #include "arcq_common.h"
 
 namespace arcq {
 
-constexpr int kTileGroups = 64;   // groups per wave-sized workgroup
-constexpr int kTileStride = 65;   // floats per group row in LDS (64 + 1 pad)
+constexpr int kWaves = 4;          // waves (tiles in flight) per workgroup
+constexpr int kTileGroups = 64;    // groups per tile = lanes per wave
+constexpr int kBuckets = 512;
+constexpr float kBucketScale = 32.0f;   // buckets per unit of t
+constexpr float kBucketOffset = 256.0f;
 
-template <typename T> struct Vec16B;  // 16-byte global access unit
-template <> struct Vec16B<float> { static constexpr int n = 4; };
-template <> struct Vec16B<__half> { static constexpr int n = 8; };
+template <typename T> struct Tile;
+template <> struct Tile<float> { static constexpr int stride = 65; static constexpr int vec = 4; };
+template <> struct Tile<__half> { static constexpr int stride = 33; static constexpr int vec = 8; };
 
-// Coalesced 16-byte loads of one tile (4096 elements) into the padded LDS tile.
+__device__ __forceinline__ int bucket_of(float t)
+{
+    const float f = __fmaf_rn(t, kBucketScale, kBucketOffset);
+    const int i = __float2int_rz(f);            // NaN -> 0, saturating
+    return min(max(i, 0), kBuckets - 1);
+}
+
+struct Bucket { float thr; int base; };
+
+// Coalesced 16-byte global loads of one tile (64 groups x 64 elements) into the wave's LDS tile.
 template <typename TIN>
 __device__ __forceinline__ void load_tile(const TIN *__restrict__ x, int64_t elem0, int64_t elem_end,
-                                          float *__restrict__ tile, int lane)
+                                          uint32_t *__restrict__ tile, int lane)
 {
-    constexpr int n = Vec16B<TIN>::n;
+    constexpr int n = Tile<TIN>::vec;
     constexpr int iters = kTileGroups * 64 / (64 * n);
+    uint4 raw[iters];
 #pragma unroll
     for (int i = 0; i < iters; ++i) {
-        const int e = (i * 64 + lane) * n;  // element offset inside the tile
-        float v[n];
-        if (elem0 + e < elem_end) {
-            const uint4 raw = *reinterpret_cast<const uint4 *>(x + elem0 + e);
-            if constexpr (n == 4) {
-                v[0] = __uint_as_float(raw.x); v[1] = __uint_as_float(raw.y);
-                v[2] = __uint_as_float(raw.z); v[3] = __uint_as_float(raw.w);
-            } else {
-                const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+        const int e = (i * 64 + lane) * n;
+        raw[i] = (elem0 + e < elem_end) ? *reinterpret_cast<const uint4 *>(x + elem0 + e) : make_uint4(0, 0, 0, 0);
+    }
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float2 f = __half22float2(h[q]);
-                    v[2 * q] = f.x; v[2 * q + 1] = f.y;
-                }
-            }
-        } else {
-#pragma unroll
-            for (int q = 0; q < n; ++q) v[q] = 0.0f;
-        }
-        float *dst = tile + (e >> 6) * kTileStride + (e & 63);
-#pragma unroll
-        for (int q = 0; q < n; ++q) dst[q] = v[q];
+    for (int i = 0; i < iters; ++i) {
+        const int e = (i * 64 + lane) * n;
+        uint32_t *dst = tile + (e >> 6) * Tile<TIN>::stride + (e & 63) * static_cast<int>(sizeof(TIN)) / 4;
+        dst[0] = raw[i].x; dst[1] = raw[i].y; dst[2] = raw[i].z; dst[3] = raw[i].w;
     }
 }
 
 template <typename TOUT>
 __device__ __forceinline__ void store_tile(TOUT *__restrict__ out, int64_t elem0, int64_t elem_end,
-                                           const float *__restrict__ tile, int lane)
+                                           const uint32_t *__restrict__ tile, int lane)
 {
-    constexpr int n = Vec16B<TOUT>::n;
+    constexpr int n = Tile<TOUT>::vec;
     constexpr int iters = kTileGroups * 64 / (64 * n);
 #pragma unroll
     for (int i = 0; i < iters; ++i) {
         const int e = (i * 64 + lane) * n;
         if (elem0 + e >= elem_end) continue;
-        const float *src = tile + (e >> 6) * kTileStride + (e & 63);
-        uint4 raw;
-        if constexpr (n == 4) {
-            raw.x = __float_as_uint(src[0]); raw.y = __float_as_uint(src[1]);
-            raw.z = __float_as_uint(src[2]); raw.w = __float_as_uint(src[3]);
-        } else {
-            __half2 *h = reinterpret_cast<__half2 *>(&raw);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) h[q] = __floats2half2_rn(src[2 * q], src[2 * q + 1]);
-        }
-        *reinterpret_cast<uint4 *>(out + elem0 + e) = raw;
+        const uint32_t *src = tile + (e >> 6) * Tile<TOUT>::stride + (e & 63) * static_cast<int>(sizeof(TOUT)) / 4;
+        *reinterpret_cast<uint4 *>(out + elem0 + e) = make_uint4(src[0], src[1], src[2], src[3]);
     }
 }
 
-// Packs the lane's 64 codes (one byte each in `c`) into 2*BITS dwords, LSB first.
-template <int BITS>
-__device__ __forceinline__ void pack64(const uint8_t (&c)[64], uint32_t (&w)[2 * BITS])
+// The lane's own group (row `lane` of the tile) as 64 floats.
+template <typename TIN>
+__device__ __forceinline__ void read_row(const uint32_t *__restrict__ row, float (&v)[64])
 {
-    if constexpr (BITS == 4) {
+    if constexpr (sizeof(TIN) == 4) {
 #pragma unroll
-        for (int d = 0; d < 8; ++d) {
-            uint32_t v = 0;
+        for (int j = 0; j < 64; ++j) v[j] = __uint_as_float(row[j]);
+    } else {
 #pragma unroll
-            for (int q = 0; q < 8; ++q) v |= static_cast<uint32_t>(c[d * 8 + q]) << (4 * q);
-            w[d] = v;
+        for (int p = 0; p < 32; ++p) {
+            const uint32_t w = row[p];
+            v[2 * p] = __half2float(__ushort_as_half(static_cast<unsigned short>(w & 0xffffu)));
+            v[2 * p + 1] = __half2float(__ushort_as_half(static_cast<unsigned short>(w >> 16)));
         }
-    } else if constexpr (BITS == 2) {
+    }
+}
+
+template <typename TOUT>
+__device__ __forceinline__ void write_row(uint32_t *__restrict__ row, const float (&v)[64])
+{
+    if constexpr (sizeof(TOUT) == 4) {
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
+        for (int j = 0; j < 64; ++j) row[j] = __float_as_uint(v[j]);
+    } else {
+#pragma unroll
+        for (int p = 0; p < 32; ++p) {
+            const __half2 h = __floats2half2_rn(v[2 * p], v[2 * p + 1]);
+            row[p] = *reinterpret_cast<const uint32_t *>(&h);
+        }
+    }
+}
+
+// Appends the 64 codes (one per array slot) to packed dwords, LSB first.
+template <int BITS>
+__device__ __forceinline__ void pack64(const uint32_t (&c)[64], uint32_t (&w)[2 * BITS])
+{
+    if constexpr (BITS == 4 || BITS == 2) {
+        constexpr int per = 32 / BITS;
+#pragma unroll
+        for (int d = 0; d < 2 * BITS; ++d) {
             uint32_t v = 0;
 #pragma unroll
-            for (int q = 0; q < 16; ++q) v |= static_cast<uint32_t>(c[d * 16 + q]) << (2 * q);
+            for (int q = 0; q < per; ++q) v |= c[d * per + q] << (BITS * q);
             w[d] = v;
         }
     } else {
-        // 8 codes -> one 24-bit chunk; 4 chunks -> 3 dwords.
-        uint32_t ch[8];
+        uint32_t ch[8];   // 8 codes -> one 24-bit chunk; 4 chunks -> 3 dwords
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             uint32_t v = 0;
 #pragma unroll
-            for (int q = 0; q < 8; ++q) v |= static_cast<uint32_t>(c[k * 8 + q]) << (3 * q);
+            for (int q = 0; q < 8; ++q) v |= c[k * 8 + q] << (3 * q);
             ch[k] = v;
         }
 #pragma unroll
@@ -125,110 +149,187 @@ __device__ __forceinline__ void pack64(const uint8_t (&c)[64], uint32_t (&w)[2 *
     }
 }
 
-template <typename TIN, typename TOUT, int BITS>
-__global__ void __launch_bounds__(64)
+// CODES = false drops everything only the code outputs need (the on-the-fly layer asks for x_hat alone).
+template <typename TIN, typename TOUT, int BITS, bool CODES>
+__global__ void __launch_bounds__(64 * kWaves)
 act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, const float *__restrict__ cb,
                      uint8_t *__restrict__ packed, uint8_t *__restrict__ codes_u8,
                      float *__restrict__ center, float *__restrict__ scale, float *__restrict__ code_sum,
                      TOUT *__restrict__ x_hat, int64_t total_groups, float eps)
 {
     constexpr int L = 1 << BITS;
-    __shared__ float tile[kTileGroups * kTileStride];
-    __shared__ float lut[L * 64];  // codebook replicated per lane: lut[c*64 + lane], conflict-free
+    constexpr int kStride = (Tile<TIN>::stride > Tile<TOUT>::stride) ? Tile<TIN>::stride : Tile<TOUT>::stride;
+    __shared__ uint32_t tiles[kWaves][kTileGroups * kStride];
+    __shared__ float lut[L * 64];          // codebook replicated per lane: lut[c*64 + lane], conflict-free
+    __shared__ Bucket table[kBuckets];
+    __shared__ float s_thr[16];
+    __shared__ int s_slow;
 
-    const int lane = threadIdx.x;
-    const int64_t group0 = static_cast<int64_t>(blockIdx.x) * kTileGroups;
-    const int64_t elem0 = group0 * 64;
-    const int64_t elem_end = total_groups * 64;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
 
     float th[L - 1];
 #pragma unroll
     for (int i = 0; i < L - 1; ++i) th[i] = thr[i];
-#pragma unroll
-    for (int c = 0; c < L; ++c) lut[c * 64 + lane] = cb[c];
 
-    load_tile<TIN>(x, elem0, elem_end, tile, lane);
+    // ---- per-workgroup setup: codebook copies and the bucket table --------------------------------
+    if (tid == 0) s_slow = 0;
+    if (tid < 64) {
+#pragma unroll
+        for (int c = 0; c < L; ++c) lut[c * 64 + lane] = cb[c];
+    }
+    if (tid < L - 1) s_thr[tid] = thr[tid];
     __syncthreads();
-
-    const int64_t g = group0 + lane;
-    const bool live = g < total_groups;
-    float *col = tile + lane * kTileStride;
-
-    float xv[64];
+    {
+        int tb[L - 1];
+        bool bad = false;
 #pragma unroll
-    for (int j = 0; j < 64; ++j) xv[j] = col[j];
-
-    float mu = 0.0f;
+        for (int i = 0; i < L - 1; ++i) tb[i] = bucket_of(th[i]);
 #pragma unroll
-    for (int j = 0; j < 64; ++j) mu += xv[j];
-    mu /= 64.0f;
-
-    float var = 0.0f;
+        for (int i = 0; i + 1 < L - 1; ++i) bad = bad || !(th[i] <= th[i + 1]);
+        if (L == 2) bad = bad || (th[0] != th[0]);
 #pragma unroll
-    for (int j = 0; j < 64; ++j) {
-        const float d = xv[j] - mu;
-        var += d * d;
-    }
-    const float s = sqrtf(var / 64.0f + eps);
-
-    uint8_t code[64];
-    float sum_codes = 0.0f;
+        for (int q = 0; q < kBuckets / (64 * kWaves); ++q) {
+            const int b = tid * (kBuckets / (64 * kWaves)) + q;
+            int below = 0, upto = 0;   // thresholds in buckets < b, <= b
 #pragma unroll
-    for (int j = 0; j < 64; ++j) {
-        const float t = (xv[j] - mu) / s;
-        int c = 0;
-        bool alive = true;
-#pragma unroll
-        for (int i = 0; i < L - 1; ++i) {
-            alive = alive && (t > th[i]);
-            c += alive ? 1 : 0;
-        }
-        code[j] = static_cast<uint8_t>(c);
-        const float v = lut[c * 64 + lane];
-        xv[j] = v;  // the input value is not needed any more
-        sum_codes += v;
-    }
-
-    if (live) {
-        if (center) center[g] = mu;
-        if (scale) scale[g] = s;
-        if (code_sum) code_sum[g] = sum_codes;
-        if (packed) {
-            uint32_t w[2 * BITS];
-            pack64<BITS>(code, w);
-            uint32_t *dst = reinterpret_cast<uint32_t *>(packed + g * (8 * BITS));
-            if constexpr (BITS == 4) {
-                reinterpret_cast<uint4 *>(dst)[0] = make_uint4(w[0], w[1], w[2], w[3]);
-                reinterpret_cast<uint4 *>(dst)[1] = make_uint4(w[4], w[5], w[6], w[7]);
-            } else if constexpr (BITS == 2) {
-                reinterpret_cast<uint4 *>(dst)[0] = make_uint4(w[0], w[1], w[2], w[3]);
-            } else {
-#pragma unroll
-                for (int q = 0; q < 3; ++q) reinterpret_cast<uint2 *>(dst)[q] = make_uint2(w[2 * q], w[2 * q + 1]);
+            for (int i = 0; i < L - 1; ++i) {
+                below += (tb[i] < b) ? 1 : 0;
+                upto += (tb[i] <= b) ? 1 : 0;
             }
+            const int inside = upto - below;
+            bad = bad || inside > 1;
+            Bucket e;
+            e.base = below;
+            e.thr = (inside == 1) ? s_thr[below] : __int_as_float(0x7f800000);   // +inf: never exceeded
+            table[b] = e;
         }
-        if (codes_u8) {
-            uint4 *dst = reinterpret_cast<uint4 *>(codes_u8 + g * 64);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t d[4];
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int b = q * 16 + k * 4;
-                    d[k] = static_cast<uint32_t>(code[b]) | (static_cast<uint32_t>(code[b + 1]) << 8) |
-                           (static_cast<uint32_t>(code[b + 2]) << 16) | (static_cast<uint32_t>(code[b + 3]) << 24);
-                }
-                dst[q] = make_uint4(d[0], d[1], d[2], d[3]);
-            }
-        }
+        if (bad) s_slow = 1;
     }
+    __syncthreads();
+    const bool table_ok = (s_slow == 0);
 
-    if (x_hat) {
-        const float code_mean = sum_codes / 64.0f;
-#pragma unroll
-        for (int j = 0; j < 64; ++j) col[j] = fma_f32(s, xv[j] - code_mean, mu);
+    uint32_t *tile = tiles[wave];
+    const int64_t ntiles = (total_groups + kTileGroups - 1) / kTileGroups;
+    const int64_t elem_end = total_groups * 64;
+
+    // All four waves run the same number of iterations so that the barriers below are uniform.
+    for (int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kWaves; tile0 < ntiles;
+         tile0 += static_cast<int64_t>(gridDim.x) * kWaves) {
+        const int64_t group0 = (tile0 + wave) * kTileGroups;
+        const int64_t elem0 = group0 * 64;
+        load_tile<TIN>(x, elem0, elem_end, tile, lane);
         __syncthreads();
-        store_tile<TOUT>(x_hat, elem0, elem_end, tile, lane);
+
+        float xv[64];
+        read_row<TIN>(tile + lane * Tile<TIN>::stride, xv);
+
+        float mu = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 64; ++j) mu += xv[j];
+        mu *= 0.015625f;                       // exact: /64
+        float var = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 64; ++j) {
+            xv[j] -= mu;                       // d_j
+            var += xv[j] * xv[j];
+        }
+        const float s = sqrtf(var * 0.015625f + eps);
+
+        // Range in which d*y, the residuals and the corrections are exact or harmlessly rounded:
+        // s normal and far from the ends, and no non-zero d_j small enough to push a residual
+        // into the subnormals (|d_j| >= 2^-90 whenever |mu| >= 2^-66, or all d_j are zero).
+        const bool lane_fast = (s >= 0x1p-60f) && (s <= 0x1p60f) && !(fabsf(mu) < 0x1p-66f && var > 0.0f);
+        const bool fast = table_ok && __all(lane_fast);
+
+        uint32_t code[CODES ? 64 : 1];
+        float sum_codes = 0.0f;
+        if (fast) {
+            const float y = 1.0f / s;
+            const float ns = -s;
+            const uint32_t lane4 = static_cast<uint32_t>(lane) * 4u;
+#pragma unroll
+            for (int j = 0; j < 64; ++j) {
+                const float d = xv[j];
+                float q = d * y;
+                float e = __fmaf_rn(ns, q, d);
+                q = __fmaf_rn(e, y, q);
+                e = __fmaf_rn(ns, q, d);
+                q = __fmaf_rn(e, y, q);        // == RN(d / s)
+                const Bucket bk = table[bucket_of(q)];
+                const uint32_t c = static_cast<uint32_t>(bk.base) + ((q > bk.thr) ? 1u : 0u);
+                if constexpr (CODES) code[j] = c;
+                const float v = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(lut) + ((c << 8) | lane4));
+                xv[j] = v;
+                sum_codes += v;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 64; ++j) {
+                const float t = xv[j] / s;
+                uint32_t c = 0;
+                bool alive = true;
+#pragma unroll
+                for (int i = 0; i < L - 1; ++i) {   // while (c < L-1 && t > thr[c]) ++c
+                    alive = alive && (t > th[i]);
+                    c += alive ? 1u : 0u;
+                }
+                if constexpr (CODES) code[j] = c;
+                const float v = lut[c * 64 + lane];
+                xv[j] = v;
+                sum_codes += v;
+            }
+        }
+
+        const int64_t g = group0 + lane;
+        if (g < total_groups) {
+            if (center) center[g] = mu;
+            if (scale) scale[g] = s;
+            if (code_sum) code_sum[g] = sum_codes;
+            if constexpr (CODES) {
+                if (packed) {
+                    uint32_t w[2 * BITS];
+                    pack64<BITS>(code, w);
+                    uint32_t *dst = reinterpret_cast<uint32_t *>(packed + g * (8 * BITS));
+                    if constexpr (BITS == 4) {
+                        reinterpret_cast<uint4 *>(dst)[0] = make_uint4(w[0], w[1], w[2], w[3]);
+                        reinterpret_cast<uint4 *>(dst)[1] = make_uint4(w[4], w[5], w[6], w[7]);
+                    } else if constexpr (BITS == 2) {
+                        reinterpret_cast<uint4 *>(dst)[0] = make_uint4(w[0], w[1], w[2], w[3]);
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 3; ++q)
+                            reinterpret_cast<uint2 *>(dst)[q] = make_uint2(w[2 * q], w[2 * q + 1]);
+                    }
+                }
+                if (codes_u8) {
+                    uint4 *dst = reinterpret_cast<uint4 *>(codes_u8 + g * 64);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        uint32_t d[4];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const int b = q * 16 + k * 4;
+                            d[k] = code[b] | (code[b + 1] << 8) | (code[b + 2] << 16) | (code[b + 3] << 24);
+                        }
+                        dst[q] = make_uint4(d[0], d[1], d[2], d[3]);
+                    }
+                }
+            }
+        }
+
+        if (x_hat) {
+            const float code_mean = sum_codes * 0.015625f;
+#pragma unroll
+            for (int j = 0; j < 64; ++j) xv[j] = fma_f32(s, xv[j] - code_mean, mu);
+            // Every lane has consumed its input row (program order within the wave), so rows may be
+            // rewritten now, possibly with a different stride.
+            write_row<TOUT>(tile + lane * Tile<TOUT>::stride, xv);
+            __syncthreads();
+            store_tile<TOUT>(x_hat, elem0, elem_end, tile, lane);
+        }
+        __syncthreads();   // the tile is reloaded in the next iteration
     }
 }
 
@@ -310,13 +411,17 @@ static int launch(const void *x, const float *thr, const float *cb, uint8_t *pac
     TOUT *xo = static_cast<TOUT *>(x_hat);
     const bool fast = gs == 64 && aligned(x, 16) && aligned(x_hat, 16) && aligned(packed, 16) && aligned(codes_u8, 16);
     if (fast) {
-        const unsigned blocks = static_cast<unsigned>((total_groups + kTileGroups - 1) / kTileGroups);
-#define ARCQ_LAUNCH_G64(B)                                                                                   \
-    hipLaunchKernelGGL((act_quant_g64_kernel<TIN, TOUT, B>), dim3(blocks), dim3(64), 0, stream, xin, thr, cb, \
-                       packed, codes_u8, center, scale, code_sum, xo, total_groups, eps)
-        if (bits == 4) ARCQ_LAUNCH_G64(4);
-        else if (bits == 3) ARCQ_LAUNCH_G64(3);
-        else ARCQ_LAUNCH_G64(2);
+        const int64_t ntiles = (total_groups + kTileGroups - 1) / kTileGroups;
+        // Up to 3 workgroups fit a CU (LDS); more tiles than that are walked by the grid-stride loop.
+        const int64_t want = (ntiles + kWaves - 1) / kWaves;
+        const unsigned blocks = static_cast<unsigned>(want < 4096 ? want : 4096);
+        const bool codes = packed || codes_u8;
+#define ARCQ_LAUNCH_G64(B, C)                                                                                     \
+    hipLaunchKernelGGL((act_quant_g64_kernel<TIN, TOUT, B, C>), dim3(blocks), dim3(64 * kWaves), 0, stream, xin, \
+                       thr, cb, packed, codes_u8, center, scale, code_sum, xo, total_groups, eps)
+        if (bits == 4) { if (codes) ARCQ_LAUNCH_G64(4, true); else ARCQ_LAUNCH_G64(4, false); }
+        else if (bits == 3) { if (codes) ARCQ_LAUNCH_G64(3, true); else ARCQ_LAUNCH_G64(3, false); }
+        else { if (codes) ARCQ_LAUNCH_G64(2, true); else ARCQ_LAUNCH_G64(2, false); }
 #undef ARCQ_LAUNCH_G64
     } else {
         if (packed && (static_cast<int64_t>(gs) * bits) % 8 != 0)
