@@ -54,7 +54,7 @@ __device__ __forceinline__ uint32_t load_codes8(const uint8_t *__restrict__ p)
 __device__ __forceinline__ float fma_f32(float a, float b, float c)
 {
     float v = __fmaf_rn(a, b, c);
-    asm volatile("" : "+v"(v));
+    asm("" : "+v"(v));   // not volatile: opaque to instruction selection, free for the scheduler to move
     return v;
 }
 

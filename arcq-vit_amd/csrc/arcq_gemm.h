@@ -1,0 +1,23 @@
+// Internal interface between the fused-GEMM entry point and its kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace arcq {
+
+struct GemmArgs {
+    const void *x_hat;       // [M,K] fp16
+    const uint8_t *pw;       // [N, K*bits/8]
+    const float *cb;         // [2^bits]
+    const float *wc, *ws, *wcs;   // [N, K/64]
+    const float *bias;       // [N] or nullptr
+    void *y;                 // [M,N]
+    bool y_f16;
+    int M, N, K, bits;
+};
+
+// Large-M kernel (256-column x up-to-256-row workgroup tiles); requires K >= 64.
+void launch_gemm_stream(const GemmArgs &g, hipStream_t stream);
+
+}  // namespace arcq

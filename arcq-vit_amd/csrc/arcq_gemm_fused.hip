@@ -11,11 +11,14 @@
 // operands are K-contiguous, which is the layout v_mfma_f32_32x32x16_f16 wants:
 // lane l supplies 8 consecutive k for row (l % 32), k offset 8*(l / 32).
 #include "arcq_common.h"
+#include "arcq_gemm.h"
 
 namespace arcq {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));   // native vectors keep staging arrays in registers
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int BK = 64;            // one quantization group per main-loop step
 constexpr int LDS_STRIDE = 72;    // halves per tile row: 64 + 8 pad (144 B) -> conflict-free b128 reads
@@ -26,11 +29,11 @@ __device__ __forceinline__ void load_codes32(const uint8_t *__restrict__ row_g, 
 {
     const uint32_t *p = reinterpret_cast<const uint32_t *>(row_g + h * (4 * BITS));
     if constexpr (BITS == 4) {
-        const uint4 v = *reinterpret_cast<const uint4 *>(p);
-        w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(p);
+        w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
     } else if constexpr (BITS == 2) {
-        const uint2 v = *reinterpret_cast<const uint2 *>(p);
-        w[0] = v.x; w[1] = v.y;
+        const u32x2_t v = *reinterpret_cast<const u32x2_t *>(p);
+        w[0] = v[0]; w[1] = v[1];
     } else {
         w[0] = p[0]; w[1] = p[1]; w[2] = p[2];
     }
@@ -87,7 +90,7 @@ gemm_fused_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, 
     const float *ws_row = ws + static_cast<int64_t>(bn) * G;
     const float *wcs_row = wcs + static_cast<int64_t>(bn) * G;
 
-    uint4 a_reg[A_PASSES];
+    u32x4_t a_reg[A_PASSES];
     uint32_t b_reg[BITS];
     float b_c, b_s, b_m;
 
@@ -95,7 +98,7 @@ gemm_fused_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, 
 #pragma unroll
         for (int p = 0; p < A_PASSES; ++p) {
             const int r = min(m0 + p * 32 + a_row, M - 1);
-            a_reg[p] = *reinterpret_cast<const uint4 *>(a + static_cast<int64_t>(r) * K + g * BK + a_col);
+            a_reg[p] = *reinterpret_cast<const u32x4_t *>(a + static_cast<int64_t>(r) * K + g * BK + a_col);
         }
         load_codes32<BITS>(pw_row + g * (8 * BITS), b_h, b_reg);
         b_c = wc_row[g];
@@ -106,7 +109,7 @@ gemm_fused_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, 
     auto stage = [&]() {
 #pragma unroll
         for (int p = 0; p < A_PASSES; ++p)
-            *reinterpret_cast<uint4 *>(&sa[(p * 32 + a_row) * LDS_STRIDE + a_col]) = a_reg[p];
+            *reinterpret_cast<u32x4_t *>(&sa[(p * 32 + a_row) * LDS_STRIDE + a_col]) = a_reg[p];
         _Float16 *dst = &sb[b_row * LDS_STRIDE + b_h * 32];
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
@@ -227,9 +230,13 @@ ARCQ_API int arcq_linear_fused(const void *x_hat,
         return fail(ARCQ_ERR_ALIGN, "arcq_linear_fused: x_hat, y and packed_w must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
-    if (y_dtype == ARCQ_F16)
+    if (m >= 512 && k >= 64) {
+        GemmArgs g{x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype == ARCQ_F16, m, n, k, bits};
+        launch_gemm_stream(g, st);
+    } else if (y_dtype == ARCQ_F16) {
         launch_out<__half>(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, m, n, k, bits, st);
-    else
+    } else {
         launch_out<float>(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, m, n, k, bits, st);
+    }
     return launch_status("arcq_linear_fused");
 }
