@@ -1,8 +1,11 @@
 // Stages 2+3 fused, large-M kernel: y[M,N] = x_hat[M,K] * w_hat[N,K]^T + bias.
 //
-// Workgroup = 4 waves, tile = (32*TI) rows x 256 columns; wave w owns columns [64w, 64w+64) of the
-// tile for all rows, i.e. TI x 2 MFMA 32x32x16 accumulator blocks (256 accumulator registers at
-// TI = 8).  The K loop advances one quantization group (64) at a time.
+// Workgroup = 4*WM waves laid out WM (rows) x 4 (columns), tile = (32*TI*WM) rows x 256 columns; a
+// wave owns 32*TI rows x 64 columns, i.e. TI x 2 MFMA 32x32x16 accumulator blocks.  The shipped
+// configuration is WM = 1, TI = 8 (four waves, one per SIMD, 256 accumulator registers each): every
+// dequantized weight fragment then feeds 8 MFMAs.  WM = 2, TI = 4 (two waves per SIMD) is kept
+// instantiable; it measured slower because the dequantization work per MFMA doubles.  The K loop
+// advances one quantization group (64) at a time.
 //
 //  * x_hat (fp16) goes global -> registers -> LDS (double buffered, row stride 144 B so that the
 //    16-byte fragment reads are bank-conflict free) and is read by all four waves.
@@ -61,46 +64,43 @@ __device__ __forceinline__ uint32_t pair_at(const uint32_t (&w)[BITS], int p)
     return v & ((1u << PB) - 1u);
 }
 
-template <int BITS, typename TOUT, int TI>
-__global__ void __launch_bounds__(256)
+template <int BITS, typename TOUT, int TI, int WM>
+__global__ void __launch_bounds__(256 * WM)
 gemm_stream_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, const float *__restrict__ cb,
                    const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
                    const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K)
 {
-    constexpr int BM = 32 * TI;
+    constexpr int THREADS = 256 * WM;
+    constexpr int BM = 32 * TI * WM;
     constexpr int L = 1 << BITS;
     constexpr int PAIRS = 1 << (2 * BITS);
-    constexpr int A_PASSES = BM / 32;            // 256 threads x 16 B cover 32 rows of 64 halves
+    constexpr int ROWS_PER_PASS = THREADS / 8;   // 8 threads x 16 B cover one row of 64 halves
+    constexpr int A_PASSES = BM / ROWS_PER_PASS;
 
+    // LDS map: [2 x_hat buffers: BM rows x 144 B][pair LUT: PAIRS entries x 32 copies x 8 B][bias: 256 floats]
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    _Float16 *sa = reinterpret_cast<_Float16 *>(smem);                       // [2][BM][kAStride]
-    float2 *pair_lut = reinterpret_cast<float2 *>(smem + 2 * BM * kAStride * 2);   // [PAIRS][32 copies]
-    __shared__ float s_cb[L];
+    _Float16 *sa = reinterpret_cast<_Float16 *>(smem);
+    float2 *pair_lut = reinterpret_cast<float2 *>(smem + 2 * BM * kAStride * 2);
+    float *s_bias = reinterpret_cast<float *>(smem + 2 * BM * kAStride * 2 + PAIRS * 256);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    const int wn = wave & 3;          // column block of 64
+    const int wm = wave >> 2;         // row block of 32*TI
     const int lr = lane & 31;         // row inside a 32-row / 32-column block
     const int lh = lane >> 5;         // k half
     const int m0 = blockIdx.y * BM;
-    const int n0 = blockIdx.x * kBN + wave * 64;
+    const int n0 = blockIdx.x * kBN + wn * 64;
     const int G = K / kBK;
     const int64_t pcols = static_cast<int64_t>(K) * BITS / 8;
-
-    if (tid < L) s_cb[tid] = cb[tid];
-    __syncthreads();
-    for (int idx = tid; idx < PAIRS * 16; idx += 256) {      // 16 x 16-byte writes cover the 32 copies of an entry
-        const int e = idx >> 4;
-        const float lo = s_cb[e & (L - 1)], hi = s_cb[e >> BITS];
-        reinterpret_cast<float4 *>(pair_lut)[idx] = make_float4(lo, hi, lo, hi);
-    }
 
     // ---- global -> register staging of the next group -------------------------------------------
     const int a_row = tid >> 3, a_col = (tid & 7) * 8;
     const __half *a_src[A_PASSES];
 #pragma unroll
     for (int p = 0; p < A_PASSES; ++p)
-        a_src[p] = a + static_cast<int64_t>(min(m0 + p * 32 + a_row, M - 1)) * K + a_col;
+        a_src[p] = a + static_cast<int64_t>(min(m0 + p * ROWS_PER_PASS + a_row, M - 1)) * K + a_col;
 
     const uint8_t *w_src[2];
     const float *wc_src[2], *ws_src[2], *wcs_src[2];
@@ -132,7 +132,7 @@ gemm_stream_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
         _Float16 *dst = sa + buf * (BM * kAStride);
 #pragma unroll
         for (int p = 0; p < A_PASSES; ++p)
-            *reinterpret_cast<u32x4_t *>(dst + (p * 32 + a_row) * kAStride + a_col) = a_reg[p];
+            *reinterpret_cast<u32x4_t *>(dst + (p * ROWS_PER_PASS + a_row) * kAStride + a_col) = a_reg[p];
     };
     auto take_b = [&]() {
 #pragma unroll
@@ -154,7 +154,7 @@ gemm_stream_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
     const char *lut_lane = reinterpret_cast<const char *>(pair_lut) + lr * 8;
-    const int lane_off = lr * kAStride + lh * 32;        // this lane's row / k-half inside an A buffer
+    const int lane_off = (wm * TI * 32 + lr) * kAStride + lh * 32;   // this lane's row / k-half inside an A buffer
 
     // Fragments are double buffered in registers: while the MFMAs of k-step s run on buffer s%2, the
     // x_hat fragments of step s+1 are read from LDS and the w_hat fragments of step s+1 are rebuilt.
@@ -196,8 +196,18 @@ gemm_stream_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
         }
     };
 
+    if (G > 0) fetch(0);
+    // While the first group's loads are in flight: codebook pairs and bias into LDS.
+    if (tid < 256) {
+        const int col = blockIdx.x * kBN + tid;
+        s_bias[tid] = (bias && col < N) ? bias[col] : 0.0f;
+    }
+    for (int idx = tid; idx < PAIRS * 16; idx += THREADS) {   // 16 x 16-byte writes cover the 32 copies of an entry
+        const int e = idx >> 4;
+        const float lo = cb[e & (L - 1)], hi = cb[e >> BITS];
+        reinterpret_cast<float4 *>(pair_lut)[idx] = make_float4(lo, hi, lo, hi);
+    }
     if (G > 0) {
-        fetch(0);
         commit_a(0);
         take_b();
     }
@@ -231,26 +241,24 @@ gemm_stream_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     if (G > 0) group_step(G - 1, std::true_type{});
 
     // ---- epilogue ----------------------------------------------------------------------------------
-    // All LDS reads of the main loop precede its last barrier, so the whole dynamic LDS block is free.
-    // Each wave stages 128 rows x 64 columns of its tile (bias added, rounded to TOUT) in its own LDS
+    // Each wave stages 32*CH rows x 64 columns of its tile (bias added, rounded to TOUT) in its own LDS
     // region, row-major with a 16-byte pad, and writes it out as 16-byte row-contiguous stores.
-    constexpr int CH = 4;                                            // 32-row blocks per pass
+    constexpr int CH = 4 / WM;                                       // 32-row blocks per pass
     constexpr int kOutStride = 64 * static_cast<int>(sizeof(TOUT)) + 16;   // bytes per staged row
     constexpr int kVec = 16 / static_cast<int>(sizeof(TOUT));        // elements per 16-byte store
     constexpr int kLanesPerRow = 64 / kVec;
-    unsigned char *stage = smem + wave * (CH * 32 * kOutStride);
+    constexpr int kRowsPerIter = 64 / kLanesPerRow;
     const bool vec_ok = (N % kVec) == 0;
 
-    float bv[2][4][4];
+    float bv[2][4][4];   // bias of this lane's 32 columns, read before the staging writes reuse the block
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int col = n0 + j * 32 + 8 * q + 4 * lh + r;
-                bv[j][q][r] = (bias && col < N) ? bias[col] : 0.0f;
-            }
+            for (int r = 0; r < 4; ++r) bv[j][q][r] = s_bias[wn * 64 + j * 32 + 8 * q + 4 * lh + r];
+    __syncthreads();     // every wave is done with the x_hat buffers, the LUT and the bias
+    unsigned char *stage = smem + wave * (CH * 32 * kOutStride);
 
 #pragma unroll
     for (int pass = 0; pass < TI / CH; ++pass) {
@@ -282,10 +290,10 @@ gemm_stream_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
         }
         __syncthreads();
 #pragma unroll
-        for (int t = 0; t < CH * 32 / (64 / kLanesPerRow); ++t) {
-            const int r = t * (64 / kLanesPerRow) + lane / kLanesPerRow;     // staged row
+        for (int t = 0; t < CH * 32 / kRowsPerIter; ++t) {
+            const int r = t * kRowsPerIter + lane / kLanesPerRow;     // staged row
             const int cseg = lane % kLanesPerRow;
-            const int row = m0 + pass * (CH * 32) + r;
+            const int row = m0 + (wm * TI + pass * CH) * 32 + r;
             const int col = n0 + cseg * kVec;
             if (row < M && col < N) {
                 const u32x4_t v = *reinterpret_cast<const u32x4_t *>(stage + r * kOutStride + cseg * 16);
@@ -304,14 +312,14 @@ gemm_stream_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     }
 }
 
-template <int BITS, typename TOUT, int TI>
+template <int BITS, typename TOUT, int TI, int WM>
 static void launch_ti(const GemmArgs &g, hipStream_t stream)
 {
-    constexpr int BM = 32 * TI;
-    const size_t main_bytes = 2 * BM * kAStride * 2 + (size_t(1) << (2 * BITS)) * 256;   // A buffers + pair LUT
-    const size_t stage_bytes = 4 * 128 * (64 * sizeof(TOUT) + 16);                       // epilogue staging
+    constexpr int BM = 32 * TI * WM;
+    const size_t main_bytes = 2 * BM * kAStride * 2 + (size_t(1) << (2 * BITS)) * 256 + 1024;   // x_hat buffers + pair LUT + bias
+    const size_t stage_bytes = size_t(4 * WM) * (4 / WM) * 32 * (64 * sizeof(TOUT) + 16);       // epilogue staging
     const size_t smem = main_bytes > stage_bytes ? main_bytes : stage_bytes;
-    auto kernel = gemm_stream_kernel<BITS, TOUT, TI>;
+    auto kernel = gemm_stream_kernel<BITS, TOUT, TI, WM>;
     static bool configured = false;   // per instantiation; the attribute is sticky for the process
     if (!configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -319,15 +327,16 @@ static void launch_ti(const GemmArgs &g, hipStream_t stream)
         configured = true;
     }
     dim3 grid((g.N + kBN - 1) / kBN, (g.M + BM - 1) / BM);
-    hipLaunchKernelGGL(kernel, grid, dim3(256), smem, stream, static_cast<const __half *>(g.x_hat), g.pw, g.cb, g.wc,
-                       g.ws, g.wcs, g.bias, static_cast<TOUT *>(g.y), g.M, g.N, g.K);
+    hipLaunchKernelGGL(kernel, grid, dim3(256 * WM), smem, stream, static_cast<const __half *>(g.x_hat), g.pw, g.cb,
+                       g.wc, g.ws, g.wcs, g.bias, static_cast<TOUT *>(g.y), g.M, g.N, g.K);
 }
 
 template <int BITS, typename TOUT>
 static void launch_bits(const GemmArgs &g, hipStream_t stream)
 {
-    if (g.M > 1024) launch_ti<BITS, TOUT, 8>(g, stream);
-    else launch_ti<BITS, TOUT, 4>(g, stream);
+    // One wave per SIMD with 256-row x 64-column wave tiles measured faster than two waves per SIMD
+    // with 128-row tiles (the dequantization work per MFMA doubles with the smaller tile).
+    launch_ti<BITS, TOUT, 8, 1>(g, stream);
 }
 
 void launch_gemm_stream(const GemmArgs &g, hipStream_t stream)
