@@ -90,8 +90,18 @@ gemm_stream_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     const int wm = wave >> 2;         // row block of 32*TI
     const int lr = lane & 31;         // row inside a 32-row / 32-column block
     const int lh = lane >> 5;         // k half
-    const int m0 = blockIdx.y * BM;
-    const int n0 = blockIdx.x * kBN + wn * 64;
+    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  Tiles are numbered with
+    // the column tile fastest and XCD x takes the contiguous range [x*per, (x+1)*per), so the column
+    // tiles that share a row tile of x_hat (and neighbouring row tiles, which share the weights) run on
+    // one XCD at about the same time and re-read their operands from that L2 instead of from HBM.
+    const int n_tiles = (N + kBN - 1) / kBN;
+    const int tiles = n_tiles * ((M + BM - 1) / BM);
+    const int per_xcd = (tiles + 7) / 8;
+    const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (tile >= tiles) return;
+    const int tile_n = tile % n_tiles;
+    const int m0 = (tile / n_tiles) * BM;
+    const int n0 = tile_n * kBN + wn * 64;
     const int G = K / kBK;
     const int64_t pcols = static_cast<int64_t>(K) * BITS / 8;
 
@@ -199,7 +209,7 @@ gemm_stream_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     if (G > 0) fetch(0);
     // While the first group's loads are in flight: codebook pairs and bias into LDS.
     if (tid < 256) {
-        const int col = blockIdx.x * kBN + tid;
+        const int col = tile_n * kBN + tid;
         s_bias[tid] = (bias && col < N) ? bias[col] : 0.0f;
     }
     for (int idx = tid; idx < PAIRS * 16; idx += THREADS) {   // 16 x 16-byte writes cover the 32 copies of an entry
@@ -326,7 +336,8 @@ static void launch_ti(const GemmArgs &g, hipStream_t stream)
                                   static_cast<int>(smem));
         configured = true;
     }
-    dim3 grid((g.N + kBN - 1) / kBN, (g.M + BM - 1) / BM);
+    const int tiles = ((g.N + kBN - 1) / kBN) * ((g.M + BM - 1) / BM);
+    dim3 grid(8 * ((tiles + 7) / 8));
     hipLaunchKernelGGL(kernel, grid, dim3(256 * WM), smem, stream, static_cast<const __half *>(g.x_hat), g.pw, g.cb,
                        g.wc, g.ws, g.wcs, g.bias, static_cast<TOUT *>(g.y), g.M, g.N, g.K);
 }
