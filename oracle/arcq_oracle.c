@@ -328,3 +328,55 @@ ORACLE_API void oracle_linear_forward_u8(
         }
     }
 }
+
+/* ------------------------------------------------------------------------- */
+/* Checker for the GPU stage-1 kernel's divide: t = d/s evaluated as          */
+/*   y = 1/s;  q = d*y;  e = fma(-s,q,d);  q = fma(e,y,q);  (twice)           */
+/* must equal the IEEE quotient d/s for every input its guard admits          */
+/* (2^-60 <= s <= 2^60, |d| <= 8s, and d == 0 or |d| >= 2^-90).  Draws n      */
+/* pseudo-random (d, s) pairs in that range, mantissa extremes included, and  */
+/* returns how many disagree (0 expected).  Not part of the reference; it     */
+/* exists so that the equivalence is tested on the CPU as well as on the GPU. */
+/* ------------------------------------------------------------------------- */
+static inline float u32_as_float(uint32_t b)
+{
+    float f;
+    memcpy(&f, &b, 4);
+    return f;
+}
+
+ORACLE_API float oracle_div_sequence(float d, float s)
+{
+    const float y = 1.0f / s;
+    float q = d * y;
+    float e = fmaf(-s, q, d);
+    q = fmaf(e, y, q);
+    e = fmaf(-s, q, d);
+    return fmaf(e, y, q);
+}
+
+ORACLE_API int64_t oracle_check_div_sequence(int64_t n, uint64_t seed)
+{
+    uint64_t rng = seed ? seed : 88172645463325252ull;
+    int64_t bad = 0;
+    for (int64_t i = 0; i < n; ++i) {
+        rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
+        const uint64_t a = rng;
+        rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
+        const uint64_t b = rng;
+        const int es = (int)(a % 121) - 60;
+        uint32_t ms = (uint32_t)(a >> 20) & 0x7fffffu;
+        if ((i & 15) == 0) ms = (i & 16) ? 0x7fffffu : 0u;
+        float s = u32_as_float(((uint32_t)(es + 127) << 23) | ms);
+        if (s > 0x1p60f) s = 0x1p60f;
+        int er = es + 3 - (int)((b >> 8) % 44);
+        if (er < -90) er = -90;
+        uint32_t mr = (uint32_t)(b >> 24) & 0x7fffffu;
+        if ((i & 31) == 1) mr = 0u;
+        float d = u32_as_float(((uint32_t)(b & 1u) << 31) | ((uint32_t)(er + 127) << 23) | mr);
+        if (fabsf(d) > 8.0f * s) d = ((b & 1u) ? -7.9f : 7.9f) * s;
+        const float want = d / s, got = oracle_div_sequence(d, s);
+        if (memcmp(&want, &got, 4) != 0) ++bad;
+    }
+    return bad;
+}

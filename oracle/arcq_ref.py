@@ -34,7 +34,9 @@ _lib = None
 
 def build_c_oracle(force: bool = False) -> str:
     """Compile ``arcq_oracle.c`` with gcc (see ``oracle/Makefile``)."""
-    if force or not os.path.exists(_LIB_PATH):
+    src = os.path.join(_HERE, "arcq_oracle.c")
+    stale = (not os.path.exists(_LIB_PATH)) or (os.path.exists(src) and os.path.getmtime(src) > os.path.getmtime(_LIB_PATH))
+    if force or stale:
         subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s", "libarcq_oracle.so"])
     return _LIB_PATH
 
@@ -48,6 +50,13 @@ def _c():
         lib.oracle_packed_cols.argtypes = [ctypes.c_int64, ctypes.c_int]
         _lib = lib
     return _lib
+
+
+def check_div_sequence(n: int, seed: int = 1) -> int:
+    """Mismatches between the GPU kernel's fma-based divide and IEEE division on ``n`` random inputs."""
+    lib = _c()
+    lib.oracle_check_div_sequence.restype = ctypes.c_int64
+    return int(lib.oracle_check_div_sequence(ctypes.c_int64(n), ctypes.c_uint64(seed)))
 
 
 def _p(a: Optional[np.ndarray]):

@@ -129,6 +129,44 @@ def test_stage1_ties_constant_and_extremes(cuda, oracle):
     assert _np(scale)[0, 0] == np.sqrt(np.float32(1e-6))
 
 
+def test_stage1_fallback_paths(cuda, oracle):
+    """The gs=64 kernel leaves its fast path (bucket-table search, fma-based divide) when two thresholds
+    share a bucket, when thresholds are unsorted, or when a group's scale / mean is out of the guarded
+    range; every fallback must give the same bits as the oracle."""
+    bits = 4
+    cb, thr = _cb(bits)
+    x = synth.make_activation(70, 128, 9)
+    d = lambda t: t.to(cuda)
+
+    def check(xx, tt, eps=1e-6):
+        ref = oracle.act_quant_c(xx.numpy(), tt, cb, bits, 64, eps=eps)
+        out = ops._act_quant(d(xx), d(tt), d(cb), bits, 64, want_packed=True, want_meta=True, eps=eps)
+        assert np.array_equal(_np(out[0]), ref["packed"])
+        assert np.array_equal(_np(out[3]), ref["scale"]) and np.array_equal(_np(out[4]), ref["code_sum"])
+
+    close = thr.clone()
+    close[7] = close[6] + 1e-4                       # two thresholds inside one 1/32-wide bucket
+    check(x, close)
+    dup = thr.clone()
+    dup[3] = dup[2]                                  # equal thresholds
+    check(x, dup)
+    unsorted = thr.clone()
+    unsorted[[4, 9]] = unsorted[[9, 4]]              # while-loop semantics: stops at the first failing threshold
+    check(x, unsorted)
+    far = thr.clone()
+    far[-1] = 9.5                                    # beyond the reachable range of t
+    check(x, far)
+    tiny = x.clone()
+    tiny[3] *= 1e-30                                 # |mu| < 2^-66 with non-zero residuals
+    tiny[5] = 0.0
+    check(tiny, thr)
+    huge = x.clone()
+    huge[7] *= 3e18                                  # variance overflows to inf: s = inf, t = 0 or nan
+    check(huge, thr)
+    check(x * 1e-12, thr, eps=0.0)                   # eps = 0: s far below 2^-60... still exact
+    check(x, thr, eps=1e-2)
+
+
 def test_stage1_empty(cuda):
     cb, thr = _cb(4)
     out = ops.quantize_activation(torch.zeros((0, 128), device=cuda), thr.to(cuda), cb.to(cuda), 4, 64)

@@ -321,3 +321,10 @@ def test_linear_f64_and_error_scale(oracle):
                        + np.abs(b), rtol=1e-13)
     y2, _ = oracle.linear_f64_c(a, w, None)
     assert np.allclose(y2, ref - b, rtol=1e-13, atol=1e-13)
+
+
+def test_fma_division_sequence_is_ieee_division(oracle):
+    """The stage-1 kernel computes t = d/s as d*RN(1/s) plus two fused residual corrections; within its
+    guard range that is the correctly rounded quotient.  20 million random pairs incl. mantissa extremes."""
+    for seed in (1, 2, 3, 4):
+        assert oracle.check_div_sequence(5_000_000, seed) == 0
