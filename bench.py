@@ -28,6 +28,10 @@ if ROOT not in sys.path:
 
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+# HBM bytes per gemm_stream_kernel launch at the default workload (average over the four layer shapes), from two
+# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a plain 256 MiB copy
+# (factors 2.00 and 1.00): 22.3 MB read + 21.8 MB written.  Summary: profiles/deit_small_w4a4_bs64_packed_linears.md.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): 44.1e6}
 
 
 def parse_args():
@@ -265,7 +269,10 @@ def main():
                    "model_shapes": args.model, "bits": args.bits, "batch": args.batch, "group_size": 64},
         "roofline": {"bound": "mfma", "kernel": "gemm_stream_kernel", "achieved": res["gemm_tflops"],
                      "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": res["gemm_tflops"] / PEAK_FP16_TFLOPS,
-                     "traffic": None, "avg_launch_us": res["gemm_us_per_launch"],
+                     "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH.get((args.model, args.bits, args.batch)),
+                     "algorithmic_flops_per_launch": res["flops_per_step"] / res["layers"],
+                     "algorithmic_bytes_per_launch": res["gemm_bytes_per_step"] / res["layers"],
+                     "avg_launch_us": res["gemm_us_per_launch"],
                      "hbm_frac_of_same_kernel": res["gemm_gbs"] / PEAK_HBM_GBS},
         "stage1": {"kernel": "act_quant_g64_kernel", "bound": "hbm", "achieved": res["act_gbs"], "peak": PEAK_HBM_GBS,
                    "unit": "GB/s", "frac": res["act_gbs"] / PEAK_HBM_GBS, "avg_launch_us": res["act_us_per_launch"]},
