@@ -20,4 +20,7 @@ struct GemmArgs {
 // Large-M kernel (256-column x up-to-256-row workgroup tiles); requires K >= 64.
 void launch_gemm_stream(const GemmArgs &g, hipStream_t stream);
 
+// Large-M weight-stationary kernel (128-column slabs dequantized once per workgroup into LDS); requires K >= 64.
+void launch_gemm_slab(const GemmArgs &g, hipStream_t stream);
+
 }  // namespace arcq

@@ -12,6 +12,8 @@
 // lane l supplies 8 consecutive k for row (l % 32), k offset 8*(l / 32).
 #include "arcq_common.h"
 #include "arcq_gemm.h"
+#include <stdlib.h>
+#include <string.h>
 
 namespace arcq {
 
@@ -205,6 +207,44 @@ static void launch_out(const void *x_hat, const uint8_t *pw, const float *cb, co
 
 using namespace arcq;
 
+// Tuning aid: ARCQ_GEMM_KERNEL=stream|slab|small pins the kernel choice (looked up on every call).
+static int forced_kernel()
+{
+    const char *e = getenv("ARCQ_GEMM_KERNEL");
+    if (!e) return 0;
+    if (!strcmp(e, "stream")) return 1;
+    if (!strcmp(e, "slab")) return 2;
+    if (!strcmp(e, "small")) return 3;
+    return 0;
+}
+
+// Picks between the two large-M kernels with a cost model fitted to measured launch durations (microseconds,
+// output write-out excluded since both pay it alike):
+//   streaming kernel: waves of 256 workgroup tiles (256 x 256), each 5 + 2.0 per quantization group;
+//   weight-stationary kernel: 5.5 + 0.85 per (64-row x group) unit of a wave + 3.5 per slab slice rebuilt
+//   (5.5 when K spans several slices, which adds two barriers per slice).
+// The weight-stationary kernel wins when K fits one slice or N is small (few slabs, many row ranges); the
+// streaming kernel wins for wide N and long K.
+static bool prefer_slab(int64_t M, int64_t N, int64_t K)
+{
+    if (M * K * 2 >= (int64_t(1) << 32)) return false;      // the slab kernel addresses x_hat with 32-bit byte offsets
+    const int64_t G = K / 64;
+    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    const double stream = static_cast<double>((tiles + 255) / 256) * (5.0 + 2.0 * static_cast<double>(G));
+    const int64_t n_slabs = (N + 127) / 128, blocks = (M + 31) / 32;
+    int64_t ranges = 256 / n_slabs;
+    if (ranges < 1) ranges = 1;
+    if (ranges > blocks) ranges = blocks;
+    const int64_t per_range = (blocks + ranges - 1) / ranges;
+    ranges = (blocks + per_range - 1) / per_range;
+    const int64_t rounds = (n_slabs * ranges + 255) / 256;
+    const int64_t passes = ((per_range + 3) / 4 + 1) / 2;
+    const int64_t slices = (G + 5) / 6;
+    const double rebuilds = slices == 1 ? 3.5 : 5.5 * static_cast<double>(passes * slices);
+    const double slab = static_cast<double>(rounds) * (5.5 + rebuilds + 0.85 * static_cast<double>(passes * G));
+    return slab < stream;
+}
+
 ARCQ_API int arcq_linear_fused(const void *x_hat,
                                const uint8_t *packed_w, const float *w_codebook,
                                const float *w_center, const float *w_scale, const float *w_code_sum,
@@ -230,9 +270,12 @@ ARCQ_API int arcq_linear_fused(const void *x_hat,
         return fail(ARCQ_ERR_ALIGN, "arcq_linear_fused: x_hat, y and packed_w must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
-    if (m >= 512 && k >= 64) {
+    const int forced = forced_kernel();
+    if (k >= 64 && (forced == 1 || forced == 2 || (forced == 0 && m >= 512))) {
         GemmArgs g{x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype == ARCQ_F16, m, n, k, bits};
-        launch_gemm_stream(g, st);
+        const bool slab = forced == 2 ? M * K * 2 < (int64_t(1) << 32) : (forced == 0 && prefer_slab(M, N, K));
+        if (slab) launch_gemm_slab(g, st);
+        else launch_gemm_stream(g, st);
     } else if (y_dtype == ARCQ_F16) {
         launch_out<__half>(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, m, n, k, bits, st);
     } else {

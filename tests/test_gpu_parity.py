@@ -272,6 +272,25 @@ def test_fused_gemm_fp16_out_no_bias_and_large_tile(cuda, oracle):
     _check_fused(cuda, oracle, 2100, 1152, 384, 3, seed=6, out_dtype=torch.float32)
 
 
+@pytest.mark.parametrize("bits,out_dtype", [(4, torch.float16), (3, torch.float32), (2, torch.float16)])
+@pytest.mark.parametrize("m,n,k", [(2100, 1152, 384),     # several passes per wave, K in one slab slice
+                                   (1000, 200, 448),      # ragged N, 7 groups: a full slice plus a one-group slice
+                                   (700, 130, 64),        # one group, last slab two columns wide
+                                   (1500, 384, 1536),     # four slab slices
+                                   (515, 520, 832)])      # 13 groups, ragged M and N
+def test_fused_gemm_kernel_variants(cuda, oracle, monkeypatch, bits, out_dtype, m, n, k):
+    """Every kernel behind arcq_linear_fused (pinned through ARCQ_GEMM_KERNEL) meets the fp64 bound, and the two
+    large-M kernels, which accumulate in the same k order, agree bit for bit."""
+    outs = {}
+    for kern in ("stream", "slab", "small"):
+        monkeypatch.setenv("ARCQ_GEMM_KERNEL", kern)
+        outs[kern], _ = _check_fused(cuda, oracle, m, n, k, bits, seed=29, out_dtype=out_dtype)
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL")
+    assert torch.equal(outs["stream"], outs["slab"])
+    auto, _ = _check_fused(cuda, oracle, m, n, k, bits, seed=29, out_dtype=out_dtype)
+    assert torch.equal(auto, outs["slab"])
+
+
 @pytest.mark.parametrize("bits", [3, 4])
 def test_layer_otf_matches_stagewise(cuda, oracle, bits):
     """arcq_linear_otf == stage 1 then fused GEMM, and its activation matches the oracle bit for bit."""
