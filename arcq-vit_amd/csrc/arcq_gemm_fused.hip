@@ -207,7 +207,7 @@ static void launch_out(const void *x_hat, const uint8_t *pw, const float *cb, co
 
 using namespace arcq;
 
-// Tuning aid: ARCQ_GEMM_KERNEL=stream|slab|small pins the kernel choice (looked up on every call).
+// Tuning aid: ARCQ_GEMM_KERNEL=stream|slab|small|splitk pins the kernel choice (looked up on every call).
 static int forced_kernel()
 {
     const char *e = getenv("ARCQ_GEMM_KERNEL");
@@ -215,6 +215,7 @@ static int forced_kernel()
     if (!strcmp(e, "stream")) return 1;
     if (!strcmp(e, "slab")) return 2;
     if (!strcmp(e, "small")) return 3;
+    if (!strcmp(e, "splitk")) return 4;
     return 0;
 }
 
@@ -271,7 +272,10 @@ ARCQ_API int arcq_linear_fused(const void *x_hat,
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
     const int forced = forced_kernel();
-    if (k >= 64 && (forced == 1 || forced == 2 || (forced == 0 && m >= 512))) {
+    if (k >= 64 && (forced == 4 || (forced == 0 && m < 512))) {
+        GemmArgs g{x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype == ARCQ_F16, m, n, k, bits};
+        launch_gemm_splitk(g, st);
+    } else if (k >= 64 && (forced == 1 || forced == 2 || (forced == 0 && m >= 512))) {
         GemmArgs g{x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype == ARCQ_F16, m, n, k, bits};
         const bool slab = forced == 2 ? M * K * 2 < (int64_t(1) << 32) : (forced == 0 && prefer_slab(M, N, K));
         if (slab) launch_gemm_slab(g, st);

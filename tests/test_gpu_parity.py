@@ -282,13 +282,27 @@ def test_fused_gemm_kernel_variants(cuda, oracle, monkeypatch, bits, out_dtype, 
     """Every kernel behind arcq_linear_fused (pinned through ARCQ_GEMM_KERNEL) meets the fp64 bound, and the two
     large-M kernels, which accumulate in the same k order, agree bit for bit."""
     outs = {}
-    for kern in ("stream", "slab", "small"):
+    for kern in ("stream", "slab", "small", "splitk"):
         monkeypatch.setenv("ARCQ_GEMM_KERNEL", kern)
         outs[kern], _ = _check_fused(cuda, oracle, m, n, k, bits, seed=29, out_dtype=out_dtype)
     monkeypatch.delenv("ARCQ_GEMM_KERNEL")
     assert torch.equal(outs["stream"], outs["slab"])
     auto, _ = _check_fused(cuda, oracle, m, n, k, bits, seed=29, out_dtype=out_dtype)
     assert torch.equal(auto, outs["slab"])
+
+
+@pytest.mark.parametrize("bits,out_dtype", [(4, torch.float16), (3, torch.float32), (2, torch.float32)])
+@pytest.mark.parametrize("m,n,k", [(197, 1152, 384), (197, 384, 1536), (1, 70, 64), (65, 130, 1088), (300, 64, 4096)])
+def test_fused_gemm_small_m_kernels(cuda, oracle, monkeypatch, bits, out_dtype, m, n, k):
+    """Small-M shapes through the split-K kernel (the default below 512 rows) and the tiled small kernel; the split-K
+    reduction order is fixed, so two launches agree bit for bit."""
+    monkeypatch.setenv("ARCQ_GEMM_KERNEL", "small")
+    _check_fused(cuda, oracle, m, n, k, bits, seed=31, out_dtype=out_dtype)
+    monkeypatch.setenv("ARCQ_GEMM_KERNEL", "splitk")
+    a, _ = _check_fused(cuda, oracle, m, n, k, bits, seed=31, out_dtype=out_dtype)
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL")
+    b, _ = _check_fused(cuda, oracle, m, n, k, bits, seed=31, out_dtype=out_dtype)
+    assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("bits", [3, 4])
