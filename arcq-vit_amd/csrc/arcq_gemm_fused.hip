@@ -223,7 +223,7 @@ static int forced_kernel()
 // output write-out excluded since both pay it alike):
 //   streaming kernel: waves of 256 workgroup tiles (256 x 256), each 5 + 2.0 per quantization group;
 //   weight-stationary kernel: 5.5 + 0.85 per (64-row x group) unit of a wave + 3.5 per slab slice rebuilt
-//   (5.5 when K spans several slices, which adds two barriers per slice).
+//   (4.2 when K spans several slices, which adds two barriers per slice).
 // The weight-stationary kernel wins when K fits one slice or N is small (few slabs, many row ranges); the
 // streaming kernel wins for wide N and long K.
 static bool prefer_slab(int64_t M, int64_t N, int64_t K)
@@ -241,9 +241,35 @@ static bool prefer_slab(int64_t M, int64_t N, int64_t K)
     const int64_t rounds = (n_slabs * ranges + 255) / 256;
     const int64_t passes = ((per_range + 3) / 4 + 1) / 2;
     const int64_t slices = (G + 5) / 6;
-    const double rebuilds = slices == 1 ? 3.5 : 5.5 * static_cast<double>(passes * slices);
+    const double rebuilds = slices == 1 ? 3.5 : 4.2 * static_cast<double>(passes * slices);
     const double slab = static_cast<double>(rounds) * (5.5 + rebuilds + 0.85 * static_cast<double>(passes * G));
     return slab < stream;
+}
+
+enum GemmKernel { kTiled = 0, kStream = 1, kSlab = 2, kSplitK = 4 };
+
+// Kernel that arcq_linear_fused runs for this shape: K below one group goes to the tiled kernel (it handles K = 0),
+// fewer than 512 rows to the split-K kernel, larger M to whichever of the two large-M kernels the cost model favours.
+static GemmKernel pick_kernel(int64_t M, int64_t N, int64_t K)
+{
+    const int forced = forced_kernel();
+    if (K < 64 || forced == 3) return kTiled;
+    const bool slab_ok = M * K * 2 < (int64_t(1) << 32);
+    if (forced == 4) return kSplitK;
+    if (forced == 2) return slab_ok ? kSlab : kStream;
+    if (forced == 1) return kStream;
+    if (M < 512) return kSplitK;
+    return prefer_slab(M, N, K) ? kSlab : kStream;
+}
+
+ARCQ_API const char *arcq_linear_fused_kernel(int64_t M, int64_t N, int64_t K)
+{
+    switch (pick_kernel(M, N, K)) {
+    case kSplitK: return "gemm_splitk_kernel";
+    case kSlab: return "gemm_slab_kernel";
+    case kStream: return "gemm_stream_kernel";
+    default: return "gemm_fused_kernel";
+    }
 }
 
 ARCQ_API int arcq_linear_fused(const void *x_hat,
@@ -271,19 +297,16 @@ ARCQ_API int arcq_linear_fused(const void *x_hat,
         return fail(ARCQ_ERR_ALIGN, "arcq_linear_fused: x_hat, y and packed_w must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
-    const int forced = forced_kernel();
-    if (k >= 64 && (forced == 4 || (forced == 0 && m < 512))) {
-        GemmArgs g{x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype == ARCQ_F16, m, n, k, bits};
-        launch_gemm_splitk(g, st);
-    } else if (k >= 64 && (forced == 1 || forced == 2 || (forced == 0 && m >= 512))) {
-        GemmArgs g{x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype == ARCQ_F16, m, n, k, bits};
-        const bool slab = forced == 2 ? M * K * 2 < (int64_t(1) << 32) : (forced == 0 && prefer_slab(M, N, K));
-        if (slab) launch_gemm_slab(g, st);
-        else launch_gemm_stream(g, st);
-    } else if (y_dtype == ARCQ_F16) {
-        launch_out<__half>(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, m, n, k, bits, st);
-    } else {
-        launch_out<float>(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, m, n, k, bits, st);
+    GemmArgs g{x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype == ARCQ_F16, m, n, k, bits};
+    switch (pick_kernel(M, N, K)) {
+    case kSplitK: launch_gemm_splitk(g, st); break;
+    case kSlab: launch_gemm_slab(g, st); break;
+    case kStream: launch_gemm_stream(g, st); break;
+    default:
+        if (y_dtype == ARCQ_F16)
+            launch_out<__half>(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, m, n, k, bits, st);
+        else
+            launch_out<float>(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, m, n, k, bits, st);
     }
     return launch_status("arcq_linear_fused");
 }

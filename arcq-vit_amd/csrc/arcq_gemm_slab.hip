@@ -117,14 +117,10 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
     }
     if (tid < kSlabN) s_bias[tid] = (bias && n_base + tid < N) ? bias[n_base + tid] : 0.0f;
 
-    // Dequantization role of this thread: weight row d_row of the slab, 32-code half d_h of every group.
-    const int d_row = tid >> 1, d_h = tid & 1;
-    const int d_n = min(n_base + d_row, N - 1);
-    const uint8_t *d_codes = pw + static_cast<int64_t>(d_n) * pcols + d_h * (4 * BITS);
-    const float *d_wc = wc + static_cast<int64_t>(d_n) * G;
-    const float *d_ws = ws + static_cast<int64_t>(d_n) * G;
-    const float *d_wcs = wcs + static_cast<int64_t>(d_n) * G;
-    unsigned char *d_dst = slab + d_row * kPitch + d_h * 64;
+    // Dequantization roles: a slab slice is 128 rows x 12 half groups (32 codes = 4*BITS bytes each, the 12 of a row
+    // contiguous in memory); half group number p = round * 256 + tid, so that consecutive lanes read consecutive
+    // pieces of a row and a wave's load touches about six rows instead of thirty-two.
+    constexpr int kHalves = 2 * kSliceGroups;
 
     const unsigned char *slab_lane = slab + lr * kPitch + lh * 64;
     unsigned char *a_tile = stage_all + wave * kATile;
@@ -138,31 +134,39 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
         uint32_t codes[kSliceGroups][BITS];
         float c[kSliceGroups], s[kSliceGroups], m[kSliceGroups];
 #pragma unroll
-        for (int gl = 0; gl < kSliceGroups; ++gl) {
-            const int g = min(g0 + gl, G - 1);
-            slab_load_codes<BITS>(d_codes + g * (8 * BITS), codes[gl]);
-            c[gl] = d_wc[g];
-            s[gl] = d_ws[g];
-            m[gl] = d_wcs[g] * 0.015625f;          // S/64, exact
+        for (int r = 0; r < kSliceGroups; ++r) {
+            const int p = r * 256 + tid;
+            const int row = p / kHalves, q = p % kHalves;
+            const int n = min(n_base + row, N - 1);
+            const int g = min(g0 + (q >> 1), G - 1);
+            slab_load_codes<BITS>(pw + static_cast<int64_t>(n) * pcols + g * (8 * BITS) + (q & 1) * (4 * BITS), codes[r]);
+            const int64_t mi = static_cast<int64_t>(n) * G + g;
+            c[r] = wc[mi];
+            s[r] = ws[mi];
+            m[r] = wcs[mi];
         }
 #pragma unroll
-        for (int gl = 0; gl < kSliceGroups; ++gl) {
-            if (gl < ng) {
-                // All 32 table lookups of this thread's half group are issued before the first is used.
+        for (int r = 0; r < kSliceGroups; ++r) {
+            const int p = r * 256 + tid;
+            const int row = p / kHalves, q = p % kHalves;
+            if ((q >> 1) < ng) {
+                // All 32 table lookups of this half group are issued before the first is used.
+                const float mg = m[r] * 0.015625f;          // S/64, exact
                 float v[32];
 #pragma unroll
-                for (int q = 0; q < 32; ++q) {
-                    const uint32_t code = slab_code_at<BITS>(codes[gl], q);
-                    v[q] = *reinterpret_cast<const float *>(
+                for (int e = 0; e < 32; ++e) {
+                    const uint32_t code = slab_code_at<BITS>(codes[r], e);
+                    v[e] = *reinterpret_cast<const float *>(
                         reinterpret_cast<const char *>(lut) + ((code << 8) | (static_cast<uint32_t>(lane) << 2)));
                 }
+                unsigned char *dst = slab + row * kPitch + q * 64;
 #pragma unroll
                 for (int q8 = 0; q8 < 4; ++q8) {
                     half8_t hv;
 #pragma unroll
-                    for (int q = 0; q < 8; ++q)
-                        hv[q] = static_cast<_Float16>(fma_f32(v[q8 * 8 + q] - m[gl], s[gl], c[gl]));
-                    *reinterpret_cast<half8_t *>(d_dst + gl * 128 + q8 * 16) = hv;
+                    for (int e = 0; e < 8; ++e)
+                        hv[e] = static_cast<_Float16>(fma_f32(v[q8 * 8 + e] - mg, s[r], c[r]));
+                    *reinterpret_cast<half8_t *>(dst + q8 * 16) = hv;
                 }
             }
         }

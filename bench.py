@@ -28,10 +28,10 @@ if ROOT not in sys.path:
 
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
-# HBM bytes per gemm_stream_kernel launch at the default workload (average over the four layer shapes), from two
-# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a plain 256 MiB copy
-# (factors 2.00 and 1.00): 22.3 MB read + 21.8 MB written.  Summary: profiles/deit_small_w4a4_bs64_packed_linears.md.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): 44.1e6}
+# HBM bytes per launch of each fused-GEMM kernel at the default workload (average over the layer shapes it serves),
+# from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a plain 256 MiB
+# copy (factors 2.00 and 1.00).  Summary: profiles/deit_small_w4a4_bs64_packed_linears.md.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): {}}
 
 
 def parse_args():
@@ -163,11 +163,11 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
         # One HIP graph per step (the reference does this for bs <= 1,
         # scripts/benchmark_arcq_on_the_fly.py:223-231).  A launch through ctypes costs ~10 us of host
         # time, more than several of these kernels run, so eager timing would measure Python.
-        def capture(kind):
+        def capture(kind, subset=None):
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
                 sp = torch.cuda.current_stream().cuda_stream   # the capture stream
-                for l in layers:
+                for l in (layers if subset is None else subset):
                     x = inputs[short(l)]
                     if kind == "full":
                         rc = lib.arcq_linear_otf(*l.otf_args(x, ws, y, sp))
@@ -186,6 +186,30 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
     t_gemm = time_loop(step_gemm, steps, warmup)
     t_act = time_loop(step_act, steps, warmup)
 
+    # The fused entry point picks one of several kernels per shape; time each kernel's launches on their own so that
+    # the roofline figure belongs to one kernel (the one with the largest share of the step).
+    per_kernel = {}
+    by_kernel = {}
+    for l in layers:
+        by_kernel.setdefault(lib.arcq_linear_fused_kernel(m, l.n, l.k).decode(), []).append(l)
+    for name, sub in by_kernel.items():
+        if use_graph:
+            fn = capture("gemm", sub)
+        else:
+            sub_args = [l.gemm_args(ws, y, m, stream) for l in sub]
+
+            def fn(sub_args=sub_args):
+                for a in sub_args:
+                    lib.arcq_linear_fused(*a)
+        t = time_loop(fn, steps, warmup)
+        kf = sum(synth.algorithmic_flops(m, l.n, l.k) for l in sub)
+        kb = sum(synth.algorithmic_bytes(m, l.n, l.k, bits) for l in sub)
+        per_kernel[name] = {"launches_per_step": len(sub), "us_per_launch": t / steps / len(sub) * 1e6,
+                            "ms_per_step": t / steps * 1e3, "tflops": kf * steps / t / 1e12,
+                            "gbs": kb * steps / t / 1e9, "flops_per_launch": kf / len(sub),
+                            "bytes_per_launch": kb / len(sub),
+                            "shapes_nk": sorted({(l.n, l.k) for l in sub})}
+
     flops = sum(synth.algorithmic_flops(m, l.n, l.k) for l in layers)
     gemm_bytes = sum(synth.algorithmic_bytes(m, l.n, l.k, bits) for l in layers)
     act_bytes = sum(2 * 2 * m * l.k for l in layers)          # fp16 in, fp16 out
@@ -200,7 +224,7 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
         "act_ms_per_step": t_act / steps * 1e3,
         "act_us_per_launch": t_act / steps / len(layers) * 1e6,
         "act_gbs": act_bytes * steps / t_act / 1e9,
-        "flops_per_step": flops, "gemm_bytes_per_step": gemm_bytes,
+        "flops_per_step": flops, "gemm_bytes_per_step": gemm_bytes, "gemm_kernels": per_kernel,
     }
     return res, layers, inputs
 
@@ -259,6 +283,8 @@ def main():
         del src, dst
     res, layers, inputs = run_config(args.model, args.bits, args.batch, args.steps, args.warmup, dev,
                                      use_graph=not args.eager)
+    dom = max(res["gemm_kernels"], key=lambda k: res["gemm_kernels"][k]["ms_per_step"])
+    dk = res["gemm_kernels"][dom]
     out = {
         "metric": "DeiT-S W4A4 images/s at bs1/bs64; packed-linear % of MFMA/HBM roofline",
         "value": res["images_per_s"], "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -267,13 +293,15 @@ def main():
         "config": {"workload": f"{args.model} 48 packed linears (12 blocks x qkv/proj/fc1/fc2), W{args.bits}A{args.bits}, "
                                f"g=64, batch {args.batch} (M={res['M']}), fp16 in/out, stage 1 + fused unpack+GEMM",
                    "model_shapes": args.model, "bits": args.bits, "batch": args.batch, "group_size": 64},
-        "roofline": {"bound": "mfma", "kernel": "gemm_stream_kernel", "achieved": res["gemm_tflops"],
-                     "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": res["gemm_tflops"] / PEAK_FP16_TFLOPS,
-                     "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH.get((args.model, args.bits, args.batch)),
-                     "algorithmic_flops_per_launch": res["flops_per_step"] / res["layers"],
-                     "algorithmic_bytes_per_launch": res["gemm_bytes_per_step"] / res["layers"],
-                     "avg_launch_us": res["gemm_us_per_launch"],
-                     "hbm_frac_of_same_kernel": res["gemm_gbs"] / PEAK_HBM_GBS},
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": dk["tflops"],
+                     "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": dk["tflops"] / PEAK_FP16_TFLOPS,
+                     "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH.get((args.model, args.bits, args.batch), {}).get(dom),
+                     "algorithmic_flops_per_launch": dk["flops_per_launch"],
+                     "algorithmic_bytes_per_launch": dk["bytes_per_launch"],
+                     "avg_launch_us": dk["us_per_launch"], "launches_per_step": dk["launches_per_step"],
+                     "hbm_frac_of_same_kernel": dk["gbs"] / PEAK_HBM_GBS,
+                     "all_fused_gemm_launches": {"tflops": res["gemm_tflops"], "avg_launch_us": res["gemm_us_per_launch"],
+                                                 "frac": res["gemm_tflops"] / PEAK_FP16_TFLOPS}},
         "stage1": {"kernel": "act_quant_g64_kernel", "bound": "hbm", "achieved": res["act_gbs"], "peak": PEAK_HBM_GBS,
                    "unit": "GB/s", "frac": res["act_gbs"] / PEAK_HBM_GBS, "avg_launch_us": res["act_us_per_launch"]},
         "detail_bs%d" % args.batch: res,

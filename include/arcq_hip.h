@@ -113,6 +113,11 @@ int arcq_linear_fused(const void *x_hat,
                       const float *bias, void *y, int y_dtype,
                       int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
 
+/* Name of the kernel arcq_linear_fused launches for an [M,K] x [N,K] problem ("gemm_splitk_kernel",
+ * "gemm_slab_kernel", "gemm_stream_kernel" or "gemm_fused_kernel"), as it appears in a kernel trace.  A profiling
+ * aid with no counterpart in the reference; the returned string is static. */
+const char *arcq_linear_fused_kernel(int64_t M, int64_t N, int64_t K);
+
 /* ---- whole packed on-the-fly layer: stage 1 then stages 2+3 ----------------
  * Replaces ARCQPackedLinearOnTheFly.forward's device work
  * (FQ/arcq_packed_on_the_fly.py:137-161).  x [M,K] of x_dtype; x_hat_ws is a
