@@ -23,51 +23,52 @@
 //    this yields the correctly rounded quotient (Markstein); lanes whose s or mu fall outside the
 //    range where no intermediate can under/overflow take the plain divide instead.
 //  * the threshold search is one table lookup plus one compare: t is mapped by a monotone function
-//    to one of 512 buckets over [-8, 8) (|t| < 8 always, since s^2 >= d_j^2/64); a bucket stores how
+//    to one of 513 buckets over [-8, 8] (|t| <= 8 always, since s^2 >= d_j^2/64); a bucket stores how
 //    many thresholds lie in lower buckets and the single threshold inside it.  Monotonicity makes
-//    base + (t > thr_in_bucket) equal to the count of thresholds below t.  If two thresholds share a
-//    bucket, or the thresholds are not sorted, the kernel falls back to the compare chain.
-#include "arcq_common.h"
+//    base + (t > thr_in_bucket) equal to the count of thresholds below t.  (Keeping the two candidate
+//    codebook values in the bucket as well saves instructions but measured slower: the wider reads at
+//    data-dependent addresses collide in LDS, while the per-lane codebook copy never does.)  If two
+//    thresholds share a bucket, a threshold lies outside [-8, 8), or the thresholds are not sorted,
+//    the kernel falls back to the compare chain.
+// The arithmetic itself lives in arcq_act_quant_core.h (shared with the fused small-M layer kernel).
+#include "arcq_act_quant_core.h"
 
 namespace arcq {
 
 constexpr int kWaves = 4;          // waves (tiles in flight) per workgroup
 constexpr int kTileGroups = 64;    // groups per tile = lanes per wave
-constexpr int kBuckets = 512;
-constexpr float kBucketScale = 32.0f;   // buckets per unit of t
-constexpr float kBucketOffset = 256.0f;
-
 template <typename T> struct Tile;
 template <> struct Tile<float> { static constexpr int stride = 65; static constexpr int vec = 4; };
 template <> struct Tile<__half> { static constexpr int stride = 33; static constexpr int vec = 8; };
 
-__device__ __forceinline__ int bucket_of(float t)
-{
-    const float f = __fmaf_rn(t, kBucketScale, kBucketOffset);
-    const int i = __float2int_rz(f);            // NaN -> 0, saturating
-    return min(max(i, 0), kBuckets - 1);
-}
+// Coalesced 16-byte global loads of one tile (64 groups x 64 elements) into registers, and from there
+// into the wave's LDS tile.  Two steps so that the first tile's loads can be in flight during the
+// per-workgroup setup.
+template <typename TIN> struct TileRegs { uint4 raw[kTileGroups * 64 / (64 * Tile<TIN>::vec)]; };
 
-struct Bucket { float thr; int base; };
-
-// Coalesced 16-byte global loads of one tile (64 groups x 64 elements) into the wave's LDS tile.
 template <typename TIN>
-__device__ __forceinline__ void load_tile(const TIN *__restrict__ x, int64_t elem0, int64_t elem_end,
-                                          uint32_t *__restrict__ tile, int lane)
+__device__ __forceinline__ void fetch_tile(const TIN *__restrict__ x, int64_t elem0, int64_t elem_end,
+                                           TileRegs<TIN> &r, int lane)
 {
     constexpr int n = Tile<TIN>::vec;
     constexpr int iters = kTileGroups * 64 / (64 * n);
-    uint4 raw[iters];
 #pragma unroll
     for (int i = 0; i < iters; ++i) {
         const int e = (i * 64 + lane) * n;
-        raw[i] = (elem0 + e < elem_end) ? *reinterpret_cast<const uint4 *>(x + elem0 + e) : make_uint4(0, 0, 0, 0);
+        r.raw[i] = (elem0 + e < elem_end) ? *reinterpret_cast<const uint4 *>(x + elem0 + e) : make_uint4(0, 0, 0, 0);
     }
+}
+
+template <typename TIN>
+__device__ __forceinline__ void commit_tile(const TileRegs<TIN> &r, uint32_t *__restrict__ tile, int lane)
+{
+    constexpr int n = Tile<TIN>::vec;
+    constexpr int iters = kTileGroups * 64 / (64 * n);
 #pragma unroll
     for (int i = 0; i < iters; ++i) {
         const int e = (i * 64 + lane) * n;
         uint32_t *dst = tile + (e >> 6) * Tile<TIN>::stride + (e & 63) * static_cast<int>(sizeof(TIN)) / 4;
-        dst[0] = raw[i].x; dst[1] = raw[i].y; dst[2] = raw[i].z; dst[3] = raw[i].w;
+        dst[0] = r.raw[i].x; dst[1] = r.raw[i].y; dst[2] = r.raw[i].z; dst[3] = r.raw[i].w;
     }
 }
 
@@ -161,7 +162,7 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
     constexpr int kStride = (Tile<TIN>::stride > Tile<TOUT>::stride) ? Tile<TIN>::stride : Tile<TOUT>::stride;
     __shared__ uint32_t tiles[kWaves][kTileGroups * kStride];
     __shared__ float lut[L * 64];          // codebook replicated per lane: lut[c*64 + lane], conflict-free
-    __shared__ Bucket table[kBuckets];
+    __shared__ Bucket table[kBuckets + 64];     // one entry per thread and round below; entries past kBuckets repeat the last state
     __shared__ float s_thr[16];
     __shared__ int s_slow;
 
@@ -169,118 +170,36 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
     const int lane = tid & 63;
     const int wave = tid >> 6;
 
-    float th[L - 1];
-#pragma unroll
-    for (int i = 0; i < L - 1; ++i) th[i] = thr[i];
-
-    // ---- per-workgroup setup: codebook copies and the bucket table --------------------------------
-    if (tid == 0) s_slow = 0;
-    if (tid < 64) {
-#pragma unroll
-        for (int c = 0; c < L; ++c) lut[c * 64 + lane] = cb[c];
-    }
-    if (tid < L - 1) s_thr[tid] = thr[tid];
-    __syncthreads();
+    // The first tile of this wave is requested before anything else: its latency overlaps the setup below.
+    const int64_t ntiles = (total_groups + kTileGroups - 1) / kTileGroups;
+    const int64_t elem_end = total_groups * 64;
+    TileRegs<TIN> regs;
     {
-        int tb[L - 1];
-        bool bad = false;
-#pragma unroll
-        for (int i = 0; i < L - 1; ++i) tb[i] = bucket_of(th[i]);
-#pragma unroll
-        for (int i = 0; i + 1 < L - 1; ++i) bad = bad || !(th[i] <= th[i + 1]);
-        if (L == 2) bad = bad || (th[0] != th[0]);
-#pragma unroll
-        for (int q = 0; q < kBuckets / (64 * kWaves); ++q) {
-            const int b = tid * (kBuckets / (64 * kWaves)) + q;
-            int below = 0, upto = 0;   // thresholds in buckets < b, <= b
-#pragma unroll
-            for (int i = 0; i < L - 1; ++i) {
-                below += (tb[i] < b) ? 1 : 0;
-                upto += (tb[i] <= b) ? 1 : 0;
-            }
-            const int inside = upto - below;
-            bad = bad || inside > 1;
-            Bucket e;
-            e.base = below;
-            e.thr = (inside == 1) ? s_thr[below] : __int_as_float(0x7f800000);   // +inf: never exceeded
-            table[b] = e;
-        }
-        if (bad) s_slow = 1;
+        const int64_t first = static_cast<int64_t>(blockIdx.x) * kWaves + wave;
+        fetch_tile<TIN>(x, first * kTileGroups * 64, elem_end, regs, lane);      // zero-fills past the end
     }
-    __syncthreads();
+
+    float th[L - 1];
+    build_quant_tables<BITS>(thr, cb, th, lut, table, s_thr, &s_slow, tid, 64 * kWaves);
     const bool table_ok = (s_slow == 0);
 
     uint32_t *tile = tiles[wave];
-    const int64_t ntiles = (total_groups + kTileGroups - 1) / kTileGroups;
-    const int64_t elem_end = total_groups * 64;
 
     // All four waves run the same number of iterations so that the barriers below are uniform.
     for (int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kWaves; tile0 < ntiles;
          tile0 += static_cast<int64_t>(gridDim.x) * kWaves) {
         const int64_t group0 = (tile0 + wave) * kTileGroups;
         const int64_t elem0 = group0 * 64;
-        load_tile<TIN>(x, elem0, elem_end, tile, lane);
+        if (tile0 != static_cast<int64_t>(blockIdx.x) * kWaves) fetch_tile<TIN>(x, elem0, elem_end, regs, lane);
+        commit_tile<TIN>(regs, tile, lane);
         __syncthreads();
 
         float xv[64];
         read_row<TIN>(tile + lane * Tile<TIN>::stride, xv);
 
-        float mu = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 64; ++j) mu += xv[j];
-        mu *= 0.015625f;                       // exact: /64
-        float var = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 64; ++j) {
-            xv[j] -= mu;                       // d_j
-            var += xv[j] * xv[j];
-        }
-        const float s = sqrtf(var * 0.015625f + eps);
-
-        // Range in which d*y, the residuals and the corrections are exact or harmlessly rounded:
-        // s normal and far from the ends, and no non-zero d_j small enough to push a residual
-        // into the subnormals (|d_j| >= 2^-90 whenever |mu| >= 2^-66, or all d_j are zero).
-        const bool lane_fast = (s >= 0x1p-60f) && (s <= 0x1p60f) && !(fabsf(mu) < 0x1p-66f && var > 0.0f);
-        const bool fast = table_ok && __all(lane_fast);
-
+        float mu, s, sum_codes;
         uint32_t code[CODES ? 64 : 1];
-        float sum_codes = 0.0f;
-        if (fast) {
-            const float y = 1.0f / s;
-            const float ns = -s;
-            const uint32_t lane4 = static_cast<uint32_t>(lane) * 4u;
-#pragma unroll
-            for (int j = 0; j < 64; ++j) {
-                const float d = xv[j];
-                float q = d * y;
-                float e = __fmaf_rn(ns, q, d);
-                q = __fmaf_rn(e, y, q);
-                e = __fmaf_rn(ns, q, d);
-                q = __fmaf_rn(e, y, q);        // == RN(d / s)
-                const Bucket bk = table[bucket_of(q)];
-                const uint32_t c = static_cast<uint32_t>(bk.base) + ((q > bk.thr) ? 1u : 0u);
-                if constexpr (CODES) code[j] = c;
-                const float v = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(lut) + ((c << 8) | lane4));
-                xv[j] = v;
-                sum_codes += v;
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < 64; ++j) {
-                const float t = xv[j] / s;
-                uint32_t c = 0;
-                bool alive = true;
-#pragma unroll
-                for (int i = 0; i < L - 1; ++i) {   // while (c < L-1 && t > thr[c]) ++c
-                    alive = alive && (t > th[i]);
-                    c += alive ? 1u : 0u;
-                }
-                if constexpr (CODES) code[j] = c;
-                const float v = lut[c * 64 + lane];
-                xv[j] = v;
-                sum_codes += v;
-            }
-        }
+        quantize_group64<BITS, CODES>(xv, th, table, lut, table_ok, lane, eps, mu, s, sum_codes, code);
 
         const int64_t g = group0 + lane;
         if (g < total_groups) {

@@ -1,0 +1,209 @@
+// Stage-1 arithmetic shared by the stand-alone activation quantizer and the fused small-M layer kernel
+// (semantics: EXT/arcq_activation_kernel.cu:24-184): per-workgroup lookup tables and the per-group routine
+// that turns 64 inputs held in one lane's registers into mu, s, the codes and the reconstructed values.
+#pragma once
+
+#include "arcq_common.h"
+
+namespace arcq {
+
+constexpr int kBuckets = 512;      // buckets that can hold a threshold; index 512 is reached by t == 8 only
+constexpr float kBucketScale = 32.0f;   // buckets per unit of t
+constexpr float kBucketOffset = 256.0f;
+
+// Bucket of a threshold: any float, clamped; -1 / kBuckets flag a threshold outside [-8, 8).
+__device__ __forceinline__ int bucket_of_threshold(float t)
+{
+    const float f = __fmaf_rn(t, kBucketScale, kBucketOffset);
+    if (!(f >= 0.0f)) return -1;                // below the table, or NaN
+    if (f >= static_cast<float>(kBuckets)) return kBuckets;
+    return __float2int_rz(f);
+}
+
+// Bucket of t = d/s on the fast path: |t| <= 8, so f lies in [0, 512] and one saturating conversion
+// (negative zero and tiny negatives give 0) is the whole index computation.
+__device__ __forceinline__ uint32_t bucket_of(float t)
+{
+    return static_cast<uint32_t>(__fmaf_rn(t, kBucketScale, kBucketOffset));
+}
+
+struct Bucket { float thr; int base; };     // the threshold inside the bucket (+inf if none); thresholds in lower buckets
+
+
+// LDS tables of one workgroup: `lut` = codebook replicated per lane (lut[c*64 + lane], conflict-free),
+// `table` = the threshold buckets, `slow` = 1 when the buckets cannot be used (two thresholds in one bucket, a
+// threshold outside [-8, 8), unsorted thresholds).  Contains two workgroup barriers; every thread must call it.
+template <int BITS>
+__device__ __forceinline__ void build_quant_tables(const float *__restrict__ thr, const float *__restrict__ cb,
+                                                   float (&th)[(1 << BITS) - 1], float *lut, Bucket *table, float *s_thr,
+                                                   int *s_slow, int tid, int nthreads)
+{
+    constexpr int L = 1 << BITS;
+#pragma unroll
+    for (int i = 0; i < L - 1; ++i) th[i] = thr[i];
+    if (tid == 0) *s_slow = 0;
+    if (tid < 64) {
+#pragma unroll
+        for (int c = 0; c < L; ++c) lut[c * 64 + tid] = cb[c];
+    }
+    if (tid < L - 1) s_thr[tid] = thr[tid];
+    __syncthreads();
+    {
+        int tb[L - 1];
+        bool bad = false;
+#pragma unroll
+        for (int i = 0; i < L - 1; ++i) {
+            tb[i] = bucket_of_threshold(th[i]);
+            bad = bad || tb[i] < 0 || tb[i] >= kBuckets;
+        }
+#pragma unroll
+        for (int i = 0; i + 1 < L - 1; ++i) bad = bad || !(th[i] <= th[i + 1]);
+        for (int b = tid; b < kBuckets + 64; b += nthreads) {
+            int below = 0, upto = 0;   // thresholds in buckets < b, <= b
+#pragma unroll
+            for (int i = 0; i < L - 1; ++i) {
+                below += (tb[i] < b) ? 1 : 0;
+                upto += (tb[i] <= b) ? 1 : 0;
+            }
+            const int inside = upto - below;
+            bad = bad || inside > 1;
+            Bucket e;
+            e.base = below;
+            e.thr = (inside == 1) ? s_thr[below] : __int_as_float(0x7f800000);   // +inf: never exceeded
+            table[b] = e;
+        }
+        if (bad) *s_slow = 1;
+    }
+    __syncthreads();
+}
+
+// One group per lane, first half: xv holds the 64 inputs on entry and the residuals d_j = x_j - mu on exit.
+// Needs no table, so it can run while other waves are still building them.
+__device__ __forceinline__ void group_stats64(float (&xv)[64], float eps, float &mu_out, float &var_out, float &s_out)
+{
+    float mu = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 64; ++j) mu += xv[j];
+    mu *= 0.015625f;                       // exact: /64
+    float var = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 64; ++j) {
+        xv[j] -= mu;                       // d_j
+        var += xv[j] * xv[j];
+    }
+    mu_out = mu;
+    var_out = var;
+    s_out = sqrtf(var * 0.015625f + eps);
+}
+
+// Second half: xv holds the residuals on entry and cb[code_j] on exit.  The whole wave must call it (the fast/slow
+// decision is wave-uniform).
+template <int BITS, bool CODES>
+__device__ __forceinline__ void group_codes64(float (&xv)[64], float mu, float var, float s,
+                                              const float (&th)[(1 << BITS) - 1], const Bucket *table, const float *lut,
+                                              bool table_ok, int lane, float &sum_out, uint32_t (&code)[CODES ? 64 : 1])
+{
+    constexpr int L = 1 << BITS;
+    // Range in which d*y, the residuals and the corrections are exact or harmlessly rounded:
+    // s normal and far from the ends, and no non-zero d_j small enough to push a residual
+    // into the subnormals (|d_j| >= 2^-90 whenever |mu| >= 2^-66, or all d_j are zero).
+    const bool lane_fast = (s >= 0x1p-60f) && (s <= 0x1p60f) && !(fabsf(mu) < 0x1p-66f && var > 0.0f);
+    const bool fast = table_ok && __all(lane_fast);
+
+    float sum_codes = 0.0f;
+    if (fast) {
+        const float y = 1.0f / s;
+        const float ns = -s;
+        const uint32_t lane4 = static_cast<uint32_t>(lane) * 4u;
+#pragma unroll
+        for (int j = 0; j < 64; ++j) {
+            const float d = xv[j];
+            float q = d * y;
+            float e = __fmaf_rn(ns, q, d);
+            q = __fmaf_rn(e, y, q);
+            e = __fmaf_rn(ns, q, d);
+            q = __fmaf_rn(e, y, q);        // == RN(d / s)
+            const Bucket bk = table[bucket_of(q)];
+            const uint32_t c = static_cast<uint32_t>(bk.base) + ((q > bk.thr) ? 1u : 0u);
+            if constexpr (CODES) code[j] = c;
+            const float v = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(lut) + ((c << 8) | lane4));
+            xv[j] = v;
+            sum_codes += v;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 64; ++j) {
+            const float t = xv[j] / s;
+            uint32_t c = 0;
+            bool alive = true;
+#pragma unroll
+            for (int i = 0; i < L - 1; ++i) {   // while (c < L-1 && t > thr[c]) ++c
+                alive = alive && (t > th[i]);
+                c += alive ? 1u : 0u;
+            }
+            if constexpr (CODES) code[j] = c;
+            const float v = lut[c * 64 + lane];
+            xv[j] = v;
+            sum_codes += v;
+        }
+    }
+    sum_out = sum_codes;
+}
+
+// Both halves: xv holds the 64 inputs on entry and cb[code_j] on exit.
+template <int BITS, bool CODES>
+__device__ __forceinline__ void quantize_group64(float (&xv)[64], const float (&th)[(1 << BITS) - 1],
+                                                 const Bucket *table, const float *lut, bool table_ok, int lane,
+                                                 float eps, float &mu_out, float &s_out, float &sum_out,
+                                                 uint32_t (&code)[CODES ? 64 : 1])
+{
+    float var;
+    group_stats64(xv, eps, mu_out, var, s_out);
+    group_codes64<BITS, CODES>(xv, mu_out, var, s_out, th, table, lut, table_ok, lane, sum_out, code);
+}
+
+// Table construction without barriers, by the `nt` threads numbered t = 0 .. nt-1 (nt a multiple of 64; other
+// threads pass t < 0 and only load the thresholds).  Each participating wave reports through its own slot
+// slow_slots[t / 64] whether the buckets are unusable; the caller synchronizes and ORs the slots.
+template <int BITS>
+__device__ __forceinline__ void build_quant_tables_by(const float *__restrict__ thr, const float *__restrict__ cb,
+                                                      float (&th)[(1 << BITS) - 1], float *lut, Bucket *table,
+                                                      int *slow_slots, int t, int nt)
+{
+    constexpr int L = 1 << BITS;
+#pragma unroll
+    for (int i = 0; i < L - 1; ++i) th[i] = thr[i];
+    if (t < 0) return;
+    if (t < 64) {
+#pragma unroll
+        for (int c = 0; c < L; ++c) lut[c * 64 + t] = cb[c];
+    }
+    int tb[L - 1];
+    bool bad = false;
+#pragma unroll
+    for (int i = 0; i < L - 1; ++i) {
+        tb[i] = bucket_of_threshold(th[i]);
+        bad = bad || tb[i] < 0 || tb[i] >= kBuckets;
+    }
+#pragma unroll
+    for (int i = 0; i + 1 < L - 1; ++i) bad = bad || !(th[i] <= th[i + 1]);
+    for (int b = t; b < kBuckets + 64; b += nt) {
+        int below = 0, upto = 0;   // thresholds in buckets < b, <= b
+        float inside_thr = __int_as_float(0x7f800000);   // +inf: never exceeded
+#pragma unroll
+        for (int i = 0; i < L - 1; ++i) {
+            below += (tb[i] < b) ? 1 : 0;
+            upto += (tb[i] <= b) ? 1 : 0;
+            inside_thr = (tb[i] == b) ? th[i] : inside_thr;
+        }
+        bad = bad || (upto - below) > 1;
+        Bucket e;
+        e.base = below;
+        e.thr = inside_thr;
+        table[b] = e;
+    }
+    const bool any_bad = __any(bad);
+    if ((t & 63) == 0) slow_slots[t >> 6] = any_bad ? 1 : 0;
+}
+
+}  // namespace arcq

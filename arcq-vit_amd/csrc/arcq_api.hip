@@ -3,7 +3,10 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <stdlib.h>
+
 #include "arcq_common.h"
+#include "arcq_gemm.h"
 
 namespace arcq {
 
@@ -42,6 +45,24 @@ ARCQ_API int arcq_linear_otf(const void *x, int x_dtype, const float *a_threshol
     if (!x_hat_ws) return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf: x_hat_ws must not be NULL");
     if (x_hat_ws == x && x_dtype != ARCQ_F16)
         return arcq::fail(ARCQ_ERR_DTYPE, "arcq_linear_otf: x_hat_ws may alias x only when x is fp16");
+    // A few hundred rows: one launch for the whole layer (same results bit for bit).  Taken only when every argument
+    // is plainly valid; anything else goes through the two entry points below, which report what is wrong.
+    // ARCQ_OTF_FUSED=0 switches the single-launch path off (tuning aid).
+    {
+        const char *e = getenv("ARCQ_OTF_FUSED");
+        const bool enabled = !(e && e[0] == '0');
+        if (enabled && group_size == 64 && arcq::bits_ok(bits) && M > 0 && N > 0 && N < (int64_t(1) << 30) &&
+            arcq::otf_small_supported(M, K) && x && x != x_hat_ws && a_thresholds && a_codebook && packed_w &&
+            w_codebook && w_center && w_scale && w_code_sum && y && (x_dtype == ARCQ_F16 || x_dtype == ARCQ_F32) &&
+            (y_dtype == ARCQ_F16 || y_dtype == ARCQ_F32) && arcq::aligned(x, 16) && arcq::aligned(x_hat_ws, 16) &&
+            arcq::aligned(y, 16) && arcq::aligned(packed_w, 16)) {
+            arcq::OtfSmallArgs a{x, x_dtype == ARCQ_F16, a_thresholds, a_codebook, packed_w, w_codebook, w_center, w_scale,
+                                 w_code_sum, bias, x_hat_ws, y, y_dtype == ARCQ_F16, static_cast<int>(M),
+                                 static_cast<int>(N), static_cast<int>(K), bits, 1.0e-6f};
+            arcq::launch_otf_small(a, static_cast<hipStream_t>(stream));
+            return arcq::launch_status("arcq_linear_otf");
+        }
+    }
     int rc = arcq_act_quant(x, x_dtype, a_thresholds, a_codebook, nullptr, nullptr, nullptr, nullptr, nullptr,
                             x_hat_ws, ARCQ_F16, M, K, bits, group_size, 1.0e-6f, stream);
     if (rc != ARCQ_OK) return rc;

@@ -26,4 +26,20 @@ void launch_gemm_slab(const GemmArgs &g, hipStream_t stream);
 // Small-M kernel (64 x 64 tiles, K split across the waves of a workgroup); requires K >= 64.
 void launch_gemm_splitk(const GemmArgs &g, hipStream_t stream);
 
+// Whole on-the-fly layer in one launch (activation quantizer + split-K product) for M < 512.
+struct OtfSmallArgs {
+    const void *x;           // [M,K] fp16 or fp32
+    bool x_f16;
+    const float *a_thr, *a_cb;
+    const uint8_t *pw;
+    const float *w_cb, *wc, *ws, *wcs, *bias;
+    void *x_hat_ws;          // [M,K] fp16, must not alias x; may be nullptr
+    void *y;
+    bool y_f16;
+    int M, N, K, bits;
+    float eps;
+};
+bool otf_small_supported(int64_t M, int64_t K);
+void launch_otf_small(const OtfSmallArgs &a, hipStream_t stream);
+
 }  // namespace arcq

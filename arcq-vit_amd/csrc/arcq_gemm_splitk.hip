@@ -2,7 +2,8 @@
 //
 // With so few rows a launch cannot fill the chip and its duration is the length of one workgroup's dependent
 // chain: (global load -> dequantize -> MFMA) once per quantization group.  This kernel shortens that chain by
-// splitting K across the waves of a workgroup: a workgroup owns a 64 x 64 output tile, wave w of NW handles the
+// splitting K across the waves of a workgroup: a workgroup owns a 32 x 64 or 64 x 64 output tile (32 rows when that
+// still leaves idle compute units), wave w of NW handles the
 // groups g = w, w + NW, w + 2 NW, ... entirely on its own (operands straight from global memory into registers, no
 // barrier inside the loop), and the NW partial tiles are added in LDS in the fixed order w = 0, 1, ..., NW-1, so
 // results do not depend on timing.  Weight reconstruction is the stand-alone stage-2 arithmetic
@@ -24,7 +25,7 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
-constexpr int kSkTile = 64;                    // rows and columns per workgroup
+constexpr int kSkTile = 64;                    // columns per workgroup (rows: 32 * RB)
 constexpr int kSkPitch = kSkTile * 4 + 16;     // bytes per row of a partial tile in LDS
 
 template <int BITS>
@@ -52,14 +53,14 @@ __device__ __forceinline__ uint32_t sk_code_at(const uint32_t (&w)[BITS], int q)
     return v & ((1u << BITS) - 1u);
 }
 
-template <int BITS>
+template <int BITS, int RB>
 struct SkOperands {                 // everything one wave needs for one group
-    u32x4_t a[2][4];                // x_hat: 2 row blocks x 4 k-steps, 8 halves each
+    u32x4_t a[RB][4];               // x_hat: RB row blocks x 4 k-steps, 8 halves each
     uint32_t codes[2][BITS];        // 32 codes of this lane's weight row, per column block
     float c[2], s[2], m[2];
 };
 
-template <int BITS, typename TOUT, int NW>
+template <int BITS, typename TOUT, int NW, int RB>
 __global__ void __launch_bounds__(NW * 64)
 gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, const float *__restrict__ cb,
                    const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
@@ -68,34 +69,38 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     constexpr int L = 1 << BITS;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *lut = reinterpret_cast<float *>(smem);                              // [L][64], one copy per lane
-    unsigned char *partial = smem + L * 64 * sizeof(float);                    // [NW][64 rows][kSkPitch]
+    unsigned char *partial = smem + L * 64 * sizeof(float);                    // [NW][RT rows][kSkPitch]
+    constexpr int RT = 32 * RB;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int lr = lane & 31;
     const int lh = lane >> 5;
-    const int m0 = blockIdx.y * kSkTile, n0 = blockIdx.x * kSkTile;
+    const int m0 = blockIdx.y * RT, n0 = blockIdx.x * kSkTile;
     const int G = K / 64;
     const int64_t pcols = static_cast<int64_t>(K) * BITS / 8;
 
-    const __half *a_src[2];
+    const __half *a_src[RB];
     const uint8_t *w_src[2];
     const float *wc_src[2], *ws_src[2], *wcs_src[2];
 #pragma unroll
+    for (int i = 0; i < RB; ++i) a_src[i] = a + static_cast<int64_t>(min(m0 + i * 32 + lr, M - 1)) * K + lh * 32;
+#pragma unroll
     for (int i = 0; i < 2; ++i) {
-        a_src[i] = a + static_cast<int64_t>(min(m0 + i * 32 + lr, M - 1)) * K + lh * 32;
         const int n = min(n0 + i * 32 + lr, N - 1);
         w_src[i] = pw + static_cast<int64_t>(n) * pcols + lh * (4 * BITS);
         wc_src[i] = wc + static_cast<int64_t>(n) * G;
         ws_src[i] = ws + static_cast<int64_t>(n) * G;
         wcs_src[i] = wcs + static_cast<int64_t>(n) * G;
     }
-    auto fetch = [&](int g, SkOperands<BITS> &o) {
+    auto fetch = [&](int g, SkOperands<BITS, RB> &o) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < RB; ++i)
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) o.a[i][kk] = *reinterpret_cast<const u32x4_t *>(a_src[i] + g * 64 + kk * 8);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
             sk_load_codes<BITS>(w_src[i] + g * (8 * BITS), o.codes[i]);
             o.c[i] = wc_src[i][g];
             o.s[i] = ws_src[i][g];
@@ -103,7 +108,7 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
         }
     };
 
-    SkOperands<BITS> o0, o1;
+    SkOperands<BITS, RB> o0, o1;
     if (wave < G) fetch(wave, o0);             // in flight while the codebook is staged
     if (tid < 64) {
 #pragma unroll
@@ -111,32 +116,35 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     }
     __syncthreads();
 
-    float16_t acc[2][2];
+    float16_t acc[RB][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < RB; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
     const char *lut_lane = reinterpret_cast<const char *>(lut) + lane * 4;
-    auto compute = [&](const SkOperands<BITS> &o) {
+    auto compute = [&](const SkOperands<BITS, RB> &o) {
         float mg[2];
 #pragma unroll
         for (int j = 0; j < 2; ++j) mg[j] = o.m[j] * 0.015625f;        // S/64, exact
+        float wv[2][32];          // all 64 table lookups are issued before the first is used
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 32; ++q)
+                wv[j][q] = *reinterpret_cast<const float *>(lut_lane + (sk_code_at<BITS>(o.codes[j], q) << 8));
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
             half8_t bf[2];
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int q = 0; q < 8; ++q) {
-                    const uint32_t code = sk_code_at<BITS>(o.codes[j], kk * 8 + q);
-                    const float v = *reinterpret_cast<const float *>(lut_lane + (code << 8));
-                    bf[j][q] = static_cast<_Float16>(fma_f32(v - mg[j], o.s[j], o.c[j]));
-                }
+                for (int q = 0; q < 8; ++q)
+                    bf[j][q] = static_cast<_Float16>(fma_f32(wv[j][kk * 8 + q] - mg[j], o.s[j], o.c[j]));
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < RB; ++i) {
                 half8_t af;
                 __builtin_memcpy(&af, &o.a[i][kk], 16);
 #pragma unroll
@@ -158,9 +166,9 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     }
 
     // ---- reduction over the waves, bias, output ----------------------------------------------------------
-    unsigned char *mine = partial + wave * (kSkTile * kSkPitch);
+    unsigned char *mine = partial + wave * (RT * kSkPitch);
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < RB; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -170,7 +178,7 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
                 *reinterpret_cast<f32x4_t *>(mine + (i * 32 + lr) * kSkPitch + (j * 32 + 8 * q + 4 * lh) * 4) = v;
             }
     __syncthreads();
-    constexpr int E = kSkTile * kSkTile / (NW * 64);       // outputs per thread, consecutive in a row
+    constexpr int E = RT * kSkTile / (NW * 64);            // outputs per thread, consecutive in a row
     constexpr int TPR = kSkTile / E;                       // threads per row
     const int row = tid / TPR, col = (tid % TPR) * E;
     float sum[E];
@@ -178,7 +186,7 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     for (int e = 0; e < E; ++e) sum[e] = 0.0f;
     const int waves_used = min(NW, G);                     // the others hold zeros; skipping them changes nothing
     for (int w = 0; w < waves_used; ++w) {
-        const unsigned char *src = partial + w * (kSkTile * kSkPitch) + row * kSkPitch + col * 4;
+        const unsigned char *src = partial + w * (RT * kSkPitch) + row * kSkPitch + col * 4;
 #pragma unroll
         for (int e = 0; e < E; e += 4) {
             const f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + e * 4);
@@ -193,10 +201,14 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
 #pragma unroll
             for (int e = 0; e < E; ++e) out[e] = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
             constexpr int BYTES = E * static_cast<int>(sizeof(TOUT));
+            if constexpr (BYTES % 16 == 0) {
 #pragma unroll
-            for (int b = 0; b < BYTES; b += 16)
-                *reinterpret_cast<u32x4_t *>(reinterpret_cast<char *>(dst) + b) =
-                    *reinterpret_cast<const u32x4_t *>(reinterpret_cast<const char *>(out) + b);
+                for (int b = 0; b < BYTES; b += 16)
+                    *reinterpret_cast<u32x4_t *>(reinterpret_cast<char *>(dst) + b) =
+                        *reinterpret_cast<const u32x4_t *>(reinterpret_cast<const char *>(out) + b);
+            } else {
+                *reinterpret_cast<u32x2_t *>(dst) = *reinterpret_cast<const u32x2_t *>(out);
+            }
         } else {
 #pragma unroll
             for (int e = 0; e < E; ++e)
@@ -205,22 +217,33 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     }
 }
 
-template <int BITS, typename TOUT>
-static void launch_splitk_t(const GemmArgs &g, hipStream_t stream)
+template <int BITS, typename TOUT, int RB>
+static void launch_splitk_rb(const GemmArgs &g, hipStream_t stream)
 {
     constexpr int NW = 8;
     constexpr int L = 1 << BITS;
-    const size_t smem = L * 64 * sizeof(float) + static_cast<size_t>(NW) * kSkTile * kSkPitch;
-    auto kernel = gemm_splitk_kernel<BITS, TOUT, NW>;
+    constexpr int RT = 32 * RB;
+    const size_t smem = L * 64 * sizeof(float) + static_cast<size_t>(NW) * RT * kSkPitch;
+    auto kernel = gemm_splitk_kernel<BITS, TOUT, NW, RB>;
     static bool configured = false;   // per instantiation; the attribute is sticky for the process
     if (!configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   static_cast<int>(smem));
         configured = true;
     }
-    const dim3 grid((g.N + kSkTile - 1) / kSkTile, (g.M + kSkTile - 1) / kSkTile);
+    const dim3 grid((g.N + kSkTile - 1) / kSkTile, (g.M + RT - 1) / RT);
     hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), smem, stream, static_cast<const __half *>(g.x_hat), g.pw, g.cb, g.wc,
                        g.ws, g.wcs, g.bias, static_cast<TOUT *>(g.y), g.M, g.N, g.K);
+}
+
+template <int BITS, typename TOUT>
+static void launch_splitk_t(const GemmArgs &g, hipStream_t stream)
+{
+    // 32-row tiles while the grid still fits the chip: more workgroups in flight and half the row-strided x_hat
+    // loads per wave; 64-row tiles otherwise (the weights are then rebuilt half as often).
+    const int64_t tiles32 = static_cast<int64_t>((g.N + kSkTile - 1) / kSkTile) * ((g.M + 31) / 32);
+    if (tiles32 <= 256) launch_splitk_rb<BITS, TOUT, 1>(g, stream);
+    else launch_splitk_rb<BITS, TOUT, 2>(g, stream);
 }
 
 void launch_gemm_splitk(const GemmArgs &g, hipStream_t stream)

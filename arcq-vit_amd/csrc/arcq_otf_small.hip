@@ -1,0 +1,362 @@
+// Whole on-the-fly layer (stage 1 + stages 2+3) in ONE launch, for a few hundred rows
+// (FQ/arcq_packed_on_the_fly.py:137-161 end to end).
+//
+// At batch 1 every kernel of the layer costs about as much as an empty launch, so the number of launches is
+// what matters.  A workgroup owns a tile of RT rows x 64 output columns.  It first quantizes the activations
+// of its RT rows (all K/64 groups; one group per lane, the same arithmetic as the stand-alone stage-1 kernel,
+// arcq_act_quant_core.h) and keeps x_hat as fp16 in LDS; the column tiles of a row tile repeat that work, on
+// compute units that would otherwise idle.  Then it runs the split-K product of gemm_splitk_kernel: wave w
+// multiplies groups w, w+8, ... against weights rebuilt from the packed codes, and the eight partial tiles are
+// added in LDS in a fixed order.  Results are bit-identical to arcq_act_quant followed by arcq_linear_fused.
+// The workgroups of column tile 0 also write x_hat to the caller's workspace, which keeps the entry point's contract.
+#include "arcq_act_quant_core.h"
+#include "arcq_gemm.h"
+
+namespace arcq {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kOsWaves = 8;
+constexpr int kOsCols = 64;                    // output columns per workgroup
+constexpr int kOsRedPitch = kOsCols * 4 + 16;  // bytes per row of a partial tile
+constexpr int kOsGroupPitch = 144;             // bytes per group of an x_hat row in LDS (128 + 16 pad)
+
+__host__ __device__ inline int os_row_pitch(int G) { return G * kOsGroupPitch + 16; }
+
+template <int BITS>
+__device__ __forceinline__ void os_load_codes(const uint8_t *__restrict__ p, uint32_t (&w)[BITS])
+{
+    if constexpr (BITS == 4) {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(p);
+        w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
+    } else if constexpr (BITS == 2) {
+        const u32x2_t v = *reinterpret_cast<const u32x2_t *>(p);
+        w[0] = v[0]; w[1] = v[1];
+    } else {
+        const uint32_t *q = reinterpret_cast<const uint32_t *>(p);
+        w[0] = q[0]; w[1] = q[1]; w[2] = q[2];
+    }
+}
+
+template <int BITS>
+__device__ __forceinline__ uint32_t os_code_at(const uint32_t (&w)[BITS], int q)
+{
+    const int bit = q * BITS;
+    const int d = bit >> 5, sh = bit & 31;
+    uint32_t v = w[d] >> sh;
+    if (sh + BITS > 32) v |= w[d + 1] << (32 - sh);
+    return v & ((1u << BITS) - 1u);
+}
+
+template <int BITS>
+struct OsWeights {                  // what one wave needs of the weights for one group
+    uint32_t codes[2][BITS];        // 32 codes of this lane's weight row, per 32-column block
+    float c[2], s[2], m[2];
+};
+
+// The lane's group (64 consecutive inputs): raw 16-byte loads (zeros when `valid` is false), converted later so
+// that the loads can be in flight during the table setup.
+template <typename TIN> struct OsGroupRegs { u32x4_t raw[sizeof(TIN) == 2 ? 8 : 16]; };
+
+template <typename TIN>
+__device__ __forceinline__ void os_fetch_group(const TIN *__restrict__ src, bool valid, OsGroupRegs<TIN> &r)
+{
+    constexpr int n = sizeof(TIN) == 2 ? 8 : 16;
+#pragma unroll
+    for (int i = 0; i < n; ++i)
+        r.raw[i] = valid ? reinterpret_cast<const u32x4_t *>(src)[i] : u32x4_t{0u, 0u, 0u, 0u};
+}
+
+template <typename TIN>
+__device__ __forceinline__ void os_convert_group(const OsGroupRegs<TIN> &r, float (&xv)[64])
+{
+    if constexpr (sizeof(TIN) == 2) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const uint32_t w = r.raw[i][d];
+                xv[i * 8 + 2 * d] = __half2float(__ushort_as_half(static_cast<unsigned short>(w & 0xffffu)));
+                xv[i * 8 + 2 * d + 1] = __half2float(__ushort_as_half(static_cast<unsigned short>(w >> 16)));
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) xv[4 * i + d] = __uint_as_float(r.raw[i][d]);
+    }
+}
+
+template <typename TIN, int BITS, typename TOUT, int RB>   // RB = 32-row blocks per workgroup tile (1 or 2)
+__global__ void __launch_bounds__(kOsWaves * 64)
+otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, const float *__restrict__ a_cb,
+                 const uint8_t *__restrict__ pw, const float *__restrict__ w_cb,
+                 const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
+                 const float *__restrict__ bias, __half *__restrict__ x_hat_ws, TOUT *__restrict__ y,
+                 int M, int N, int K, float eps, int tile_bytes)
+{
+    constexpr int L = 1 << BITS;
+    constexpr int RT = 32 * RB;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    // [x_hat tile] [partial tiles] [activation LUT] [weight LUT] [buckets] [per-wave flags]
+    unsigned char *xt = smem;
+    unsigned char *partial = smem + tile_bytes;
+    float *a_lut = reinterpret_cast<float *>(partial + kOsWaves * RT * kOsRedPitch);
+    float *w_lut = a_lut + L * 64;
+    Bucket *table = reinterpret_cast<Bucket *>(w_lut + L * 64);
+    int *slow_slots = reinterpret_cast<int *>(table + kBuckets + 64);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int lr = lane & 31;
+    const int lh = lane >> 5;
+    const int m0 = blockIdx.y * RT, n0 = blockIdx.x * kOsCols;
+    const int G = K / 64;
+    const int row_pitch = os_row_pitch(G);
+    const int64_t pcols = static_cast<int64_t>(K) * BITS / 8;
+
+    // ---- weights of this wave's first group: requested now, used after stage 1 ---------------------------
+    const uint8_t *w_src[2];
+    const float *wc_src[2], *ws_src[2], *wcs_src[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int n = min(n0 + j * 32 + lr, N - 1);
+        w_src[j] = pw + static_cast<int64_t>(n) * pcols + lh * (4 * BITS);
+        wc_src[j] = wc + static_cast<int64_t>(n) * G;
+        ws_src[j] = ws + static_cast<int64_t>(n) * G;
+        wcs_src[j] = wcs + static_cast<int64_t>(n) * G;
+    }
+    auto fetch_w = [&](int g, OsWeights<BITS> &o) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            os_load_codes<BITS>(w_src[j] + g * (8 * BITS), o.codes[j]);
+            o.c[j] = wc_src[j][g];
+            o.s[j] = ws_src[j][g];
+            o.m[j] = wcs_src[j][g];
+        }
+    };
+    OsWeights<BITS> o0, o1;
+    if (wave < G) fetch_w(wave, o0);
+
+    // ---- stage 1: x_hat of the RT rows into LDS -----------------------------------------------------------
+    // Group f = t0 + lane of the row tile (row f / G, group f % G).  The first round's inputs are requested before
+    // the table setup so that one memory latency hides behind it.
+    const int groups = RT * G;
+    OsGroupRegs<TIN> in;
+    auto fetch_x = [&](int t0) {
+        const int f = t0 + lane;
+        const int row = f / G, g = f - row * G;
+        os_fetch_group<TIN>(x + static_cast<int64_t>(min(m0 + row, M - 1)) * K + g * 64, f < groups && m0 + row < M, in);
+    };
+    // Waves 0 .. tile_waves-1 own one 64-group tile each (32 rows x K <= 512 is at most four tiles); the other
+    // waves build the lookup tables meanwhile.  One barrier joins the two halves.
+    const int tile_waves = (groups + 63) / 64;
+    const bool has_tile = wave < tile_waves;
+    if (has_tile) fetch_x(wave * 64);
+    float th[L - 1];
+    build_quant_tables_by<BITS>(a_thr, a_cb, th, a_lut, table, slow_slots, has_tile ? -1 : tid - tile_waves * 64,
+                                (kOsWaves - tile_waves) * 64);
+    if (wave == kOsWaves - 1) {
+#pragma unroll
+        for (int c = 0; c < L; ++c) w_lut[c * 64 + lane] = w_cb[c];
+    }
+    float xv[64];
+    float mu = 0.0f, var = 0.0f, s = 0.0f;
+    if (has_tile) {
+        os_convert_group<TIN>(in, xv);
+        group_stats64(xv, eps, mu, var, s);
+    }
+    __syncthreads();
+    const bool write_ws = (x_hat_ws != nullptr) && blockIdx.x == 0;
+    if (has_tile) {
+        bool table_ok = true;
+        for (int w = tile_waves; w < kOsWaves; ++w) table_ok = table_ok && (slow_slots[w - tile_waves] == 0);
+        const int f = wave * 64 + lane;
+        const int row = f / G, g = f - row * G;
+        const bool valid = f < groups && m0 + row < M;
+        float sum_codes;
+        uint32_t code[1];
+        group_codes64<BITS, false>(xv, mu, var, s, th, table, a_lut, table_ok, lane, sum_codes, code);
+        const float code_mean = sum_codes * 0.015625f;
+        u32x4_t out[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const int j = i * 8 + 2 * d;
+                const __half2 h = __floats2half2_rn(fma_f32(s, xv[j] - code_mean, mu), fma_f32(s, xv[j + 1] - code_mean, mu));
+                out[i][d] = *reinterpret_cast<const uint32_t *>(&h);
+            }
+        if (f < groups) {
+            unsigned char *dst = xt + row * row_pitch + g * kOsGroupPitch;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) reinterpret_cast<u32x4_t *>(dst)[i] = out[i];
+        }
+        if (write_ws && valid) {
+            u32x4_t *dst = reinterpret_cast<u32x4_t *>(x_hat_ws + static_cast<int64_t>(m0 + row) * K + g * 64);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dst[i] = out[i];
+        }
+    }
+    __syncthreads();
+
+    // ---- stages 2+3: split-K product, wave w takes groups w, w+8, ... --------------------------------------
+    float16_t acc[RB][2];
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    const char *lut_lane = reinterpret_cast<const char *>(w_lut) + lane * 4;
+    const unsigned char *a_lane = xt + lr * row_pitch + lh * 64;
+    auto compute = [&](int g, const OsWeights<BITS> &o) {
+        float mg[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) mg[j] = o.m[j] * 0.015625f;        // S/64, exact
+        const unsigned char *a_g = a_lane + g * kOsGroupPitch;
+        float wv[2][32];          // all 64 table lookups are issued before the first is used
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 32; ++q)
+                wv[j][q] = *reinterpret_cast<const float *>(lut_lane + (os_code_at<BITS>(o.codes[j], q) << 8));
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            half8_t bf[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int q = 0; q < 8; ++q)
+                    bf[j][q] = static_cast<_Float16>(fma_f32(wv[j][kk * 8 + q] - mg[j], o.s[j], o.c[j]));
+#pragma unroll
+            for (int i = 0; i < RB; ++i) {
+                const half8_t af = *reinterpret_cast<const half8_t *>(a_g + i * 32 * row_pitch + kk * 16);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af, acc[i][j], 0, 0, 0);
+            }
+        }
+    };
+    for (int g = wave; g < G; g += 2 * kOsWaves) {
+        if (g + kOsWaves < G) fetch_w(g + kOsWaves, o1);
+        compute(g, o0);
+        if (g + kOsWaves < G) {
+            if (g + 2 * kOsWaves < G) fetch_w(g + 2 * kOsWaves, o0);
+            compute(g + kOsWaves, o1);
+        }
+    }
+    // ---- reduction over the waves in a fixed order, bias, output -------------------------------------------
+    unsigned char *mine = partial + wave * (RT * kOsRedPitch);
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                f32x4_t v;
+                v[0] = acc[i][j][4 * q]; v[1] = acc[i][j][4 * q + 1]; v[2] = acc[i][j][4 * q + 2]; v[3] = acc[i][j][4 * q + 3];
+                *reinterpret_cast<f32x4_t *>(mine + (i * 32 + lr) * kOsRedPitch + (j * 32 + 8 * q + 4 * lh) * 4) = v;
+            }
+    __syncthreads();
+    constexpr int E = RT * kOsCols / (kOsWaves * 64);      // outputs per thread, consecutive in a row (8 or 4)
+    constexpr int TPR = kOsCols / E;
+    const int row = tid / TPR, col = (tid % TPR) * E;
+    float sum[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) sum[e] = 0.0f;
+    const int waves_used = min(kOsWaves, G);
+    for (int w = 0; w < waves_used; ++w) {
+        const unsigned char *src = partial + w * (RT * kOsRedPitch) + row * kOsRedPitch + col * 4;
+#pragma unroll
+        for (int e = 0; e < E; e += 4) {
+            const f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + e * 4);
+            sum[e] += v[0]; sum[e + 1] += v[1]; sum[e + 2] += v[2]; sum[e + 3] += v[3];
+        }
+    }
+    const int gr = m0 + row, gc = n0 + col;
+    if (gr < M && gc < N) {
+        TOUT *dst = y + static_cast<int64_t>(gr) * N + gc;
+        constexpr int BYTES = E * static_cast<int>(sizeof(TOUT));
+        if (gc + E <= N && (N % E) == 0 && BYTES % 8 == 0) {
+            TOUT out[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) out[e] = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
+            if constexpr (BYTES % 16 == 0) {
+#pragma unroll
+                for (int b = 0; b < BYTES; b += 16)
+                    *reinterpret_cast<u32x4_t *>(reinterpret_cast<char *>(dst) + b) =
+                        *reinterpret_cast<const u32x4_t *>(reinterpret_cast<const char *>(out) + b);
+            } else {
+                *reinterpret_cast<u32x2_t *>(dst) = *reinterpret_cast<const u32x2_t *>(out);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                if (gc + e < N) dst[e] = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
+        }
+    }
+}
+
+template <typename TIN, int BITS, typename TOUT, int RB>
+static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
+{
+    constexpr int L = 1 << BITS;
+    constexpr int RT = 32 * RB;
+    const int G = a.K / 64;
+    const int xhat_bytes = RT * os_row_pitch(G);
+    const int partial_bytes = kOsWaves * RT * kOsRedPitch;
+    const int tile_bytes = xhat_bytes;
+    const size_t smem = tile_bytes + partial_bytes + 2 * L * 64 * sizeof(float) + (kBuckets + 64) * sizeof(Bucket) + 64;
+    auto kernel = otf_small_kernel<TIN, BITS, TOUT, RB>;
+    static int configured = 0;        // per instantiation: largest dynamic LDS size requested so far
+    if (static_cast<int>(smem) > configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  static_cast<int>(smem));
+        configured = static_cast<int>(smem);
+    }
+    const dim3 grid((a.N + kOsCols - 1) / kOsCols, (a.M + RT - 1) / RT);
+    hipLaunchKernelGGL(kernel, grid, dim3(kOsWaves * 64), smem, stream, static_cast<const TIN *>(a.x), a.a_thr, a.a_cb,
+                       a.pw, a.w_cb, a.wc, a.ws, a.wcs, a.bias, static_cast<__half *>(a.x_hat_ws),
+                       static_cast<TOUT *>(a.y), a.M, a.N, a.K, a.eps, tile_bytes);
+}
+
+template <typename TIN, int BITS, typename TOUT>
+static void launch_os_rb(const OtfSmallArgs &a, hipStream_t stream)
+{
+    launch_os<TIN, BITS, TOUT, 1>(a, stream);
+}
+
+template <typename TIN, typename TOUT>
+static void launch_os_bits(const OtfSmallArgs &a, hipStream_t stream)
+{
+    if (a.bits == 4) launch_os_rb<TIN, 4, TOUT>(a, stream);
+    else if (a.bits == 3) launch_os_rb<TIN, 3, TOUT>(a, stream);
+    else launch_os_rb<TIN, 2, TOUT>(a, stream);
+}
+
+// One launch pays off while the activation quantizer of a 32-row tile is at most one 64-group tile per SIMD
+// (K <= 512): every column tile repeats that work, and beyond it the repeated work is longer than a second launch.
+bool otf_small_supported(int64_t M, int64_t K)
+{
+    return M < 512 && K >= 64 && K % 64 == 0 && K <= 512;
+}
+
+void launch_otf_small(const OtfSmallArgs &a, hipStream_t stream)
+{
+    if (a.x_f16) {
+        if (a.y_f16) launch_os_bits<__half, __half>(a, stream);
+        else launch_os_bits<__half, float>(a, stream);
+    } else {
+        if (a.y_f16) launch_os_bits<float, __half>(a, stream);
+        else launch_os_bits<float, float>(a, stream);
+    }
+}
+
+}  // namespace arcq

@@ -333,6 +333,49 @@ def test_layer_otf_matches_stagewise(cuda, oracle, bits):
     assert (y.float().cpu() - fq).abs().max() < 2e-2 * fq.abs().max()
 
 
+@pytest.mark.parametrize("bits,x_dtype,out_dtype", [(4, torch.float16, torch.float16), (3, torch.float32, torch.float32),
+                                                    (2, torch.float16, torch.float32), (4, torch.float32, torch.float16)])
+@pytest.mark.parametrize("m,n,k", [(197, 1152, 384), (197, 384, 1536), (1, 70, 64), (65, 130, 1088), (500, 64, 2048),
+                                   (33, 200, 2112)])
+def test_layer_otf_single_launch(cuda, oracle, monkeypatch, bits, x_dtype, out_dtype, m, n, k):
+    """Below 512 rows arcq_linear_otf runs the whole layer in one launch (when K fits LDS); it must equal the
+    two-launch path bit for bit, in y and in the x_hat workspace, and x_hat must equal the oracle's."""
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 37)
+    _, thr = _cb(bits)
+    bias = synth.make_bias(n, 37)
+    x = synth.make_activation(m, k, 37, "gelu" if k > n else "ln").to(x_dtype)
+    d = lambda t: t.to(cuda)
+    args = (d(x), d(thr), d(cb), d(packed), d(cb), d(center), d(scale), d(code_sum), d(bias), bits, 64)
+    outs = []
+    for flag in ("1", "0"):
+        monkeypatch.setenv("ARCQ_OTF_FUSED", flag)
+        ws = torch.full((m, k), float("nan"), dtype=torch.float16, device=cuda)
+        y = ops.linear_otf(*args, out_dtype=out_dtype, x_hat_ws=ws)
+        outs.append((y, ws))
+    assert torch.equal(outs[0][0], outs[1][0])
+    assert torch.equal(outs[0][1], outs[1][1])
+    want_xhat = oracle.act_quant_c(x.float().numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)
+    assert np.array_equal(_np(outs[0][1]).view(np.uint16), want_xhat.view(np.uint16))
+    w = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, bits, 64).astype(np.float16)
+    y64, mag = oracle.linear_f64_c(want_xhat, w, bias.numpy())
+    tol = _gemm_tol(mag, k) + (np.abs(y64) * 2.0 ** -11 + 2.0 ** -25 if out_dtype == torch.float16 else 0.0)
+    assert np.all(np.abs(_np(outs[0][0]).astype(np.float64) - y64) <= tol)
+
+
+def test_layer_otf_single_launch_fallback_thresholds(cuda, oracle):
+    """Thresholds the bucket table cannot hold (two within one bucket) take the compare chain inside the fused kernel."""
+    bits, m, n, k = 3, 130, 128, 256
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 39)
+    thr = torch.tensor([-1.0, -0.5, -0.49, 0.0, 0.3, 0.31, 1.2], dtype=torch.float32)
+    x = synth.make_activation(m, k, 39).to(torch.float16)
+    d = lambda t: t.to(cuda)
+    ws = torch.empty((m, k), dtype=torch.float16, device=cuda)
+    ops.linear_otf(d(x), d(thr), d(cb), d(packed), d(cb), d(center), d(scale), d(code_sum), None, bits, 64,
+                   out_dtype=torch.float16, x_hat_ws=ws)
+    want = oracle.act_quant_c(x.float().numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)
+    assert np.array_equal(_np(ws).view(np.uint16), want.view(np.uint16))
+
+
 # ------------------------------------------------------------------------------------------------
 # index-space linears
 # ------------------------------------------------------------------------------------------------
