@@ -23,7 +23,8 @@
 //    this yields the correctly rounded quotient (Markstein); lanes whose s or mu fall outside the
 //    range where no intermediate can under/overflow take the plain divide instead.
 //  * the threshold search is one table lookup plus one compare: t is mapped by a monotone function
-//    to one of 513 buckets over [-8, 8] (|t| <= 8 always, since s^2 >= d_j^2/64); a bucket stores how
+//    to one of up to 513 buckets over [-8, 8] (|t| <= 8 always, since s^2 >= d_j^2/64; the bucket width
+//    adapts to the smallest gap between thresholds); a bucket stores how
 //    many thresholds lie in lower buckets and the single threshold inside it.  Monotonicity makes
 //    base + (t > thr_in_bucket) equal to the count of thresholds below t.  (Keeping the two candidate
 //    codebook values in the bucket as well saves instructions but measured slower: the wider reads at
@@ -162,9 +163,8 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
     constexpr int kStride = (Tile<TIN>::stride > Tile<TOUT>::stride) ? Tile<TIN>::stride : Tile<TOUT>::stride;
     __shared__ uint32_t tiles[kWaves][kTileGroups * kStride];
     __shared__ float lut[L * 64];          // codebook replicated per lane: lut[c*64 + lane], conflict-free
-    __shared__ Bucket table[kBuckets + 64];     // one entry per thread and round below; entries past kBuckets repeat the last state
-    __shared__ float s_thr[16];
-    __shared__ int s_slow;
+    __shared__ Bucket table[kMaxBuckets + 1];
+    __shared__ int slow_slots[kWaves];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -179,9 +179,14 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
         fetch_tile<TIN>(x, first * kTileGroups * 64, elem_end, regs, lane);      // zero-fills past the end
     }
 
-    float th[L - 1];
-    build_quant_tables<BITS>(thr, cb, th, lut, table, s_thr, &s_slow, tid, 64 * kWaves);
-    const bool table_ok = (s_slow == 0);
+    // Thresholds and codebook are requested now and first used after the first tile's statistics: the lookup
+    // tables are built once per workgroup, between the two halves of the first tile, so that their load latency
+    // and the tile's hide behind each other.
+    float th[L - 1], cbv[L];
+    load_quant_params<BITS>(thr, cb, th, cbv);
+    bool table_ok = false;
+    bool tables_built = false;
+    BucketScale bq;
 
     uint32_t *tile = tiles[wave];
 
@@ -197,9 +202,19 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
         float xv[64];
         read_row<TIN>(tile + lane * Tile<TIN>::stride, xv);
 
-        float mu, s, sum_codes;
+        float mu, var, s, sum_codes;
         uint32_t code[CODES ? 64 : 1];
-        quantize_group64<BITS, CODES>(xv, th, table, lut, table_ok, lane, eps, mu, s, sum_codes, code);
+        group_stats64(xv, eps, mu, var, s);
+        if (!tables_built) {
+            bq = pick_bucket_scale<BITS>(th);
+            build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * kWaves);
+            __syncthreads();
+            table_ok = true;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) table_ok = table_ok && (slow_slots[w] == 0);
+            tables_built = true;
+        }
+        group_codes64<BITS, CODES>(xv, mu, var, s, th, bq, table, lut, table_ok, lane, sum_codes, code);
 
         const int64_t g = group0 + lane;
         if (g < total_groups) {

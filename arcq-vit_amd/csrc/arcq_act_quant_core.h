@@ -7,74 +7,101 @@
 
 namespace arcq {
 
-constexpr int kBuckets = 512;      // buckets that can hold a threshold; index 512 is reached by t == 8 only
-constexpr float kBucketScale = 32.0f;   // buckets per unit of t
-constexpr float kBucketOffset = 256.0f;
+constexpr int kMaxBuckets = 512;   // table entries 0 .. nb (nb <= 512); entry nb is reached by t == 8 only
 
-// Bucket of a threshold: any float, clamped; -1 / kBuckets flag a threshold outside [-8, 8).
-__device__ __forceinline__ int bucket_of_threshold(float t)
+// Bucket geometry: t in [-8, 8] maps to floor(t * scale + 8 * scale); nb = 16 * scale buckets can hold a threshold.
+// The scale is the smallest of 4, 8, 16, 32 buckets per unit of t that separates every pair of thresholds
+// (scale * smallest gap > 1), so the usual codebooks need a 65- or 129-entry table instead of 513.
+struct BucketScale { float scale, offset; int nb; };
+
+template <int BITS>
+__device__ __forceinline__ BucketScale pick_bucket_scale(const float (&th)[(1 << BITS) - 1])
 {
-    const float f = __fmaf_rn(t, kBucketScale, kBucketOffset);
+    constexpr int L = 1 << BITS;
+    float gap = 16.0f;
+#pragma unroll
+    for (int i = 0; i + 1 < L - 1; ++i) gap = fminf(gap, th[i + 1] - th[i]);      // NaN gaps are ignored; checked later
+    float scale = 32.0f;
+    if (gap * 16.0f > 1.0f) scale = 16.0f;
+    if (gap * 8.0f > 1.0f) scale = 8.0f;
+    if (gap * 4.0f > 1.0f) scale = 4.0f;
+    BucketScale q;
+    q.scale = scale;
+    q.offset = 8.0f * scale;
+    q.nb = static_cast<int>(16.0f * scale);
+    return q;
+}
+
+// Bucket of a threshold: any float; -1 / nb flag a threshold outside [-8, 8).
+__device__ __forceinline__ int bucket_of_threshold(float t, const BucketScale &q)
+{
+    const float f = __fmaf_rn(t, q.scale, q.offset);
     if (!(f >= 0.0f)) return -1;                // below the table, or NaN
-    if (f >= static_cast<float>(kBuckets)) return kBuckets;
+    if (f >= static_cast<float>(q.nb)) return q.nb;
     return __float2int_rz(f);
 }
 
-// Bucket of t = d/s on the fast path: |t| <= 8, so f lies in [0, 512] and one saturating conversion
+// Bucket of t = d/s on the fast path: |t| <= 8, so f lies in [0, nb] and one saturating conversion
 // (negative zero and tiny negatives give 0) is the whole index computation.
-__device__ __forceinline__ uint32_t bucket_of(float t)
+__device__ __forceinline__ uint32_t bucket_of(float t, const BucketScale &q)
 {
-    return static_cast<uint32_t>(__fmaf_rn(t, kBucketScale, kBucketOffset));
+    return static_cast<uint32_t>(__fmaf_rn(t, q.scale, q.offset));
 }
 
 struct Bucket { float thr; int base; };     // the threshold inside the bucket (+inf if none); thresholds in lower buckets
 
-
-// LDS tables of one workgroup: `lut` = codebook replicated per lane (lut[c*64 + lane], conflict-free),
-// `table` = the threshold buckets, `slow` = 1 when the buckets cannot be used (two thresholds in one bucket, a
-// threshold outside [-8, 8), unsorted thresholds).  Contains two workgroup barriers; every thread must call it.
 template <int BITS>
-__device__ __forceinline__ void build_quant_tables(const float *__restrict__ thr, const float *__restrict__ cb,
-                                                   float (&th)[(1 << BITS) - 1], float *lut, Bucket *table, float *s_thr,
-                                                   int *s_slow, int tid, int nthreads)
+__device__ __forceinline__ void load_quant_params(const float *__restrict__ thr, const float *__restrict__ cb,
+                                                  float (&th)[(1 << BITS) - 1], float (&cbv)[1 << BITS])
 {
     constexpr int L = 1 << BITS;
 #pragma unroll
     for (int i = 0; i < L - 1; ++i) th[i] = thr[i];
-    if (tid == 0) *s_slow = 0;
-    if (tid < 64) {
 #pragma unroll
-        for (int c = 0; c < L; ++c) lut[c * 64 + tid] = cb[c];
+    for (int c = 0; c < L; ++c) cbv[c] = cb[c];
+}
+
+// Table construction without barriers, by the `nt` threads numbered t = 0 .. nt-1 (nt a multiple of 64; the calling
+// waves must be complete).  `lut` = codebook replicated per lane (lut[c*64 + lane], conflict-free), `table` = the
+// threshold buckets.  Each participating wave reports through its own slot slow_slots[t / 64] whether the buckets
+// are unusable (two thresholds in one bucket, a threshold outside [-8, 8), unsorted thresholds); the caller
+// synchronizes and ORs the slots.
+template <int BITS>
+__device__ __forceinline__ void build_quant_tables_by(const float (&th)[(1 << BITS) - 1], const float (&cbv)[1 << BITS],
+                                                      const BucketScale &q, float *lut, Bucket *table, int *slow_slots,
+                                                      int t, int nt)
+{
+    constexpr int L = 1 << BITS;
+    if (t < 64) {
+#pragma unroll
+        for (int c = 0; c < L; ++c) lut[c * 64 + t] = cbv[c];
     }
-    if (tid < L - 1) s_thr[tid] = thr[tid];
-    __syncthreads();
-    {
-        int tb[L - 1];
-        bool bad = false;
+    int tb[L - 1];
+    bool bad = false;
+#pragma unroll
+    for (int i = 0; i < L - 1; ++i) {
+        tb[i] = bucket_of_threshold(th[i], q);
+        bad = bad || tb[i] < 0 || tb[i] >= q.nb;
+    }
+#pragma unroll
+    for (int i = 0; i + 1 < L - 1; ++i) bad = bad || !(th[i] <= th[i + 1]);
+    for (int b = t; b <= q.nb; b += nt) {
+        int below = 0, upto = 0;   // thresholds in buckets < b, <= b
+        float inside_thr = __int_as_float(0x7f800000);   // +inf: never exceeded
 #pragma unroll
         for (int i = 0; i < L - 1; ++i) {
-            tb[i] = bucket_of_threshold(th[i]);
-            bad = bad || tb[i] < 0 || tb[i] >= kBuckets;
+            below += (tb[i] < b) ? 1 : 0;
+            upto += (tb[i] <= b) ? 1 : 0;
+            inside_thr = (tb[i] == b) ? th[i] : inside_thr;
         }
-#pragma unroll
-        for (int i = 0; i + 1 < L - 1; ++i) bad = bad || !(th[i] <= th[i + 1]);
-        for (int b = tid; b < kBuckets + 64; b += nthreads) {
-            int below = 0, upto = 0;   // thresholds in buckets < b, <= b
-#pragma unroll
-            for (int i = 0; i < L - 1; ++i) {
-                below += (tb[i] < b) ? 1 : 0;
-                upto += (tb[i] <= b) ? 1 : 0;
-            }
-            const int inside = upto - below;
-            bad = bad || inside > 1;
-            Bucket e;
-            e.base = below;
-            e.thr = (inside == 1) ? s_thr[below] : __int_as_float(0x7f800000);   // +inf: never exceeded
-            table[b] = e;
-        }
-        if (bad) *s_slow = 1;
+        bad = bad || (upto - below) > 1;
+        Bucket e;
+        e.base = below;
+        e.thr = inside_thr;
+        table[b] = e;
     }
-    __syncthreads();
+    const bool any_bad = __any(bad);
+    if ((t & 63) == 0) slow_slots[t >> 6] = any_bad ? 1 : 0;
 }
 
 // One group per lane, first half: xv holds the 64 inputs on entry and the residuals d_j = x_j - mu on exit.
@@ -100,8 +127,9 @@ __device__ __forceinline__ void group_stats64(float (&xv)[64], float eps, float 
 // decision is wave-uniform).
 template <int BITS, bool CODES>
 __device__ __forceinline__ void group_codes64(float (&xv)[64], float mu, float var, float s,
-                                              const float (&th)[(1 << BITS) - 1], const Bucket *table, const float *lut,
-                                              bool table_ok, int lane, float &sum_out, uint32_t (&code)[CODES ? 64 : 1])
+                                              const float (&th)[(1 << BITS) - 1], const BucketScale &bq,
+                                              const Bucket *table, const float *lut, bool table_ok, int lane,
+                                              float &sum_out, uint32_t (&code)[CODES ? 64 : 1])
 {
     constexpr int L = 1 << BITS;
     // Range in which d*y, the residuals and the corrections are exact or harmlessly rounded:
@@ -123,7 +151,7 @@ __device__ __forceinline__ void group_codes64(float (&xv)[64], float mu, float v
             q = __fmaf_rn(e, y, q);
             e = __fmaf_rn(ns, q, d);
             q = __fmaf_rn(e, y, q);        // == RN(d / s)
-            const Bucket bk = table[bucket_of(q)];
+            const Bucket bk = table[bucket_of(q, bq)];
             const uint32_t c = static_cast<uint32_t>(bk.base) + ((q > bk.thr) ? 1u : 0u);
             if constexpr (CODES) code[j] = c;
             const float v = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(lut) + ((c << 8) | lane4));
@@ -148,62 +176,6 @@ __device__ __forceinline__ void group_codes64(float (&xv)[64], float mu, float v
         }
     }
     sum_out = sum_codes;
-}
-
-// Both halves: xv holds the 64 inputs on entry and cb[code_j] on exit.
-template <int BITS, bool CODES>
-__device__ __forceinline__ void quantize_group64(float (&xv)[64], const float (&th)[(1 << BITS) - 1],
-                                                 const Bucket *table, const float *lut, bool table_ok, int lane,
-                                                 float eps, float &mu_out, float &s_out, float &sum_out,
-                                                 uint32_t (&code)[CODES ? 64 : 1])
-{
-    float var;
-    group_stats64(xv, eps, mu_out, var, s_out);
-    group_codes64<BITS, CODES>(xv, mu_out, var, s_out, th, table, lut, table_ok, lane, sum_out, code);
-}
-
-// Table construction without barriers, by the `nt` threads numbered t = 0 .. nt-1 (nt a multiple of 64; other
-// threads pass t < 0 and only load the thresholds).  Each participating wave reports through its own slot
-// slow_slots[t / 64] whether the buckets are unusable; the caller synchronizes and ORs the slots.
-template <int BITS>
-__device__ __forceinline__ void build_quant_tables_by(const float *__restrict__ thr, const float *__restrict__ cb,
-                                                      float (&th)[(1 << BITS) - 1], float *lut, Bucket *table,
-                                                      int *slow_slots, int t, int nt)
-{
-    constexpr int L = 1 << BITS;
-#pragma unroll
-    for (int i = 0; i < L - 1; ++i) th[i] = thr[i];
-    if (t < 0) return;
-    if (t < 64) {
-#pragma unroll
-        for (int c = 0; c < L; ++c) lut[c * 64 + t] = cb[c];
-    }
-    int tb[L - 1];
-    bool bad = false;
-#pragma unroll
-    for (int i = 0; i < L - 1; ++i) {
-        tb[i] = bucket_of_threshold(th[i]);
-        bad = bad || tb[i] < 0 || tb[i] >= kBuckets;
-    }
-#pragma unroll
-    for (int i = 0; i + 1 < L - 1; ++i) bad = bad || !(th[i] <= th[i + 1]);
-    for (int b = t; b < kBuckets + 64; b += nt) {
-        int below = 0, upto = 0;   // thresholds in buckets < b, <= b
-        float inside_thr = __int_as_float(0x7f800000);   // +inf: never exceeded
-#pragma unroll
-        for (int i = 0; i < L - 1; ++i) {
-            below += (tb[i] < b) ? 1 : 0;
-            upto += (tb[i] <= b) ? 1 : 0;
-            inside_thr = (tb[i] == b) ? th[i] : inside_thr;
-        }
-        bad = bad || (upto - below) > 1;
-        Bucket e;
-        e.base = below;
-        e.thr = inside_thr;
-        table[b] = e;
-    }
-    const bool any_bad = __any(bad);
-    if ((t & 63) == 0) slow_slots[t >> 6] = any_bad ? 1 : 0;
 }
 
 }  // namespace arcq

@@ -108,7 +108,7 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     float *a_lut = reinterpret_cast<float *>(partial + kOsWaves * RT * kOsRedPitch);
     float *w_lut = a_lut + L * 64;
     Bucket *table = reinterpret_cast<Bucket *>(w_lut + L * 64);
-    int *slow_slots = reinterpret_cast<int *>(table + kBuckets + 64);
+    int *slow_slots = reinterpret_cast<int *>(table + kMaxBuckets + 64);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -158,9 +158,11 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     const int tile_waves = (groups + 63) / 64;
     const bool has_tile = wave < tile_waves;
     if (has_tile) fetch_x(wave * 64);
-    float th[L - 1];
-    build_quant_tables_by<BITS>(a_thr, a_cb, th, a_lut, table, slow_slots, has_tile ? -1 : tid - tile_waves * 64,
-                                (kOsWaves - tile_waves) * 64);
+    float th[L - 1], cbv[L];
+    load_quant_params<BITS>(a_thr, a_cb, th, cbv);
+    const BucketScale bq = pick_bucket_scale<BITS>(th);
+    if (!has_tile)
+        build_quant_tables_by<BITS>(th, cbv, bq, a_lut, table, slow_slots, tid - tile_waves * 64, (kOsWaves - tile_waves) * 64);
     if (wave == kOsWaves - 1) {
 #pragma unroll
         for (int c = 0; c < L; ++c) w_lut[c * 64 + lane] = w_cb[c];
@@ -181,7 +183,7 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
         const bool valid = f < groups && m0 + row < M;
         float sum_codes;
         uint32_t code[1];
-        group_codes64<BITS, false>(xv, mu, var, s, th, table, a_lut, table_ok, lane, sum_codes, code);
+        group_codes64<BITS, false>(xv, mu, var, s, th, bq, table, a_lut, table_ok, lane, sum_codes, code);
         const float code_mean = sum_codes * 0.015625f;
         u32x4_t out[8];
 #pragma unroll
@@ -313,7 +315,7 @@ static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
     const int xhat_bytes = RT * os_row_pitch(G);
     const int partial_bytes = kOsWaves * RT * kOsRedPitch;
     const int tile_bytes = xhat_bytes;
-    const size_t smem = tile_bytes + partial_bytes + 2 * L * 64 * sizeof(float) + (kBuckets + 64) * sizeof(Bucket) + 64;
+    const size_t smem = tile_bytes + partial_bytes + 2 * L * 64 * sizeof(float) + (kMaxBuckets + 64) * sizeof(Bucket) + 64;
     auto kernel = otf_small_kernel<TIN, BITS, TOUT, RB>;
     static int configured = 0;        // per instantiation: largest dynamic LDS size requested so far
     if (static_cast<int>(smem) > configured) {
