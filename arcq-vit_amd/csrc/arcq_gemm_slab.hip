@@ -64,11 +64,12 @@ __device__ __forceinline__ uint32_t slab_code_at(const uint32_t (&w)[BITS], int 
     return v & ((1u << BITS) - 1u);
 }
 
+// Ordering point between LDS accesses of different lanes of one wave.  LDS operations of a wave execute in issue
+// order, so no wait is needed; this only keeps the compiler from moving code across.  (A release/acquire fence here
+// would also wait for the wave's outstanding global stores and serialize the epilogue on their latency.)
 __device__ __forceinline__ void wave_sync()
 {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 template <int BITS, typename TOUT>
@@ -111,11 +112,6 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
     const int passes = (per_wave + kTI - 1) / kTI;          // same for all four waves: barriers stay uniform
     const int slices = (G + kSliceGroups - 1) / kSliceGroups;
 
-    if (tid < 64) {
-#pragma unroll
-        for (int c = 0; c < L; ++c) lut[c * 64 + lane] = cb[c];
-    }
-    if (tid < kSlabN) s_bias[tid] = (bias && n_base + tid < N) ? bias[n_base + tid] : 0.0f;
 
     // Dequantization roles: a slab slice is 128 rows x 12 half groups (32 codes = 4*BITS bytes each, the 12 of a row
     // contiguous in memory); half group number p = round * 256 + tid, so that consecutive lanes read consecutive
@@ -130,9 +126,11 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
     unsigned char *a_wr = a_tile + ld_row * kAPitch + ld_c * 16;
     const unsigned char *a_rd = a_tile + lr * kAPitch + lh * 64;
 
-    auto dequant_slice = [&](int g0, int ng) {
-        uint32_t codes[kSliceGroups][BITS];
-        float c[kSliceGroups], s[kSliceGroups], m[kSliceGroups];
+    // Codes and metadata of one slice: fetched into registers first (for the first slice at the very top of the
+    // kernel, so that this latency, the codebook's and the first x_hat units' all overlap), converted afterwards.
+    uint32_t codes[kSliceGroups][BITS];
+    float c[kSliceGroups], s[kSliceGroups], m[kSliceGroups];
+    auto fetch_slice = [&](int g0) {
 #pragma unroll
         for (int r = 0; r < kSliceGroups; ++r) {
             const int p = r * 256 + tid;
@@ -145,6 +143,14 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
             s[r] = ws[mi];
             m[r] = wcs[mi];
         }
+    };
+    fetch_slice(0);
+    if (tid < 64) {
+#pragma unroll
+        for (int cc = 0; cc < L; ++cc) lut[cc * 64 + lane] = cb[cc];
+    }
+    if (tid < kSlabN) s_bias[tid] = (bias && n_base + tid < N) ? bias[n_base + tid] : 0.0f;
+    auto dequant_slice = [&](int ng) {
 #pragma unroll
         for (int r = 0; r < kSliceGroups; ++r) {
             const int p = r * 256 + tid;
@@ -259,8 +265,9 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
             const int g0 = sl * kSliceGroups;
             const int ng = min(kSliceGroups, G - g0);
             if (!(slices == 1 && pass > 0)) {
+                if (!(pass == 0 && sl == 0)) fetch_slice(g0);
                 __syncthreads();          // every wave is done reading the previous slice (and the LUT is filled)
-                dequant_slice(g0, ng);
+                dequant_slice(ng);
                 __syncthreads();
             }
 #pragma unroll

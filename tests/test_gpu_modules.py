@@ -311,3 +311,39 @@ def test_fullsize_properties(cuda, oracle, bits):
     # (7) sampled rows against the fp64 oracle with the fp32-accumulation bound
     y64, mag = oracle.linear_f64_c(_np(xh[rows.to(cuda)]), _np(w16), None)
     assert np.all(np.abs(_np(y[rows.to(cuda)]).astype(np.float64) - y64) <= (k + 2) * 2.0 ** -24 * mag)
+
+
+@pytest.mark.parametrize("m,n,k,bits", [(12608, 384, 384, 4), (12608, 1536, 384, 4), (12608, 384, 1536, 4),
+                                        (12608, 1536, 384, 3), (12608, 3072, 768, 4), (12608, 768, 3072, 3),
+                                        (50432, 1024, 1024, 3)])
+def test_fullsize_gemm_shapes(cuda, oracle, m, n, k, bits):
+    """The remaining BASELINE layer shapes (DeiT-S proj/fc1/fc2, DeiT-B fc1/fc2, ViT-L proj at batch 256) through
+    whichever large-M kernel the dispatcher picks: row permutation and M-split leave rows unchanged (tiles do not
+    interact), the result matches a library GEMM on the stage-2 output and, on sampled rows, the fp64 oracle within
+    the fp32-accumulation bound."""
+    cb = synth.quantile_codebook(bits)
+    thr = synth.midpoint_thresholds(cb)
+    x = synth.make_activation(m, k, 81, "gelu" if k > n else "ln").to(cuda)
+    xh = ops.quantize_activation_dequant(x, thr.to(cuda), cb.to(cuda), bits, 64).half()
+    del x
+    w = synth.make_weight(n, k, 82)
+    wcodes, wc, ws, wcs = oracle.quantize_weight_torch(w, thr, cb, 64, 1e-6)
+    pw = A.pack_codes_py(wcodes, bits).to(cuda)
+    cb, wc, ws, wcs = cb.to(cuda), wc.to(cuda), ws.to(cuda), wcs.to(cuda)
+    bias = synth.make_bias(n, 83).to(cuda)
+    y = ops.linear_fused(xh, pw, cb, wc, ws, wcs, bias, bits, 64, out_dtype=torch.float32)
+    perm = torch.randperm(m, device=cuda)
+    yp = ops.linear_fused(xh[perm].contiguous(), pw, cb, wc, ws, wcs, bias, bits, 64, out_dtype=torch.float32)
+    assert torch.equal(yp, y[perm])
+    del yp
+    cut = 5000
+    y_part = ops.linear_fused(xh[:cut].contiguous(), pw, cb, wc, ws, wcs, bias, bits, 64, out_dtype=torch.float32)
+    assert torch.equal(y_part, y[:cut])
+    y16 = ops.linear_fused(xh, pw, cb, wc, ws, wcs, bias, bits, 64, out_dtype=torch.float16)
+    assert torch.equal(y16, y.half())                       # same fp32 value, rounded once
+    w16 = ops.unpack_weight_hip(pw, cb, wc, ws, wcs, bits, 64)
+    rows = torch.randint(0, m, (48,), device=cuda)
+    lib = torch.nn.functional.linear(xh[rows].float(), w16.float(), bias)
+    assert (y[rows] - lib).abs().max() < 1e-3 * lib.abs().max()
+    y64, mag = oracle.linear_f64_c(_np(xh[rows]), _np(w16), _np(bias))
+    assert np.all(np.abs(_np(y[rows]).astype(np.float64) - y64) <= (k + 2) * 2.0 ** -24 * mag)
