@@ -20,6 +20,8 @@
 #include "arcq_common.h"
 #include "arcq_gemm.h"
 
+#include <type_traits>
+
 namespace arcq {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -232,7 +234,8 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
         // unit's; k-step 0 parks the next unit in the LDS tile, k-step 1 fetches the unit after the one in flight.
         // `bf[0]` holds the fragments of (gl, k-step 0) on entry and of (gl + 1, k-step 0) on exit.
         half8_t bf[2][kTJ];
-        auto unit = [&](u32x4_t (&rw)[8], int gl) {
+        auto unit = [&](u32x4_t (&rw)[8], int gl, auto nfc) {
+            constexpr int NFU = decltype(nfc)::value;      // row blocks really multiplied (1 on a wave's last, odd pass)
             const unsigned char *bsrc = slab_lane + gl * 128;
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
@@ -243,7 +246,7 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
                 if (kk == 0) park_unit(rw);
                 if (kk == 1) load_unit(rw);
 #pragma unroll
-                for (int i = 0; i < kTI; ++i) {
+                for (int i = 0; i < NFU; ++i) {
                     half8_t af;
                     __builtin_memcpy(&af, &frag[i][kk], 16);
 #pragma unroll
@@ -252,11 +255,11 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
                     frag[i][kk] = *reinterpret_cast<const u32x4_t *>(a_rd + i * 32 * kAPitch + kk * 16);
                 }
 #pragma unroll
-                for (int q = 0; q < 8; ++q) {
+                for (int q = 0; q < 4 * NFU; ++q) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // 1 MFMA
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 // 1 LDS read
-                    if (kk == 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);    // 1 LDS write
-                    if (kk == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // 1 global load
+                    if (kk == 0) __builtin_amdgcn_sched_group_barrier(0x200, 2 / NFU, 0);    // LDS writes
+                    if (kk == 1) __builtin_amdgcn_sched_group_barrier(0x020, 2 / NFU, 0);    // global loads
                 }
             }
         };
@@ -272,9 +275,18 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
             }
 #pragma unroll
             for (int j = 0; j < kTJ; ++j) bf[0][j] = *reinterpret_cast<const half8_t *>(slab_lane + j * 32 * kPitch);
-            for (int gl = 0; gl < ng; gl += 2) {
-                unit(r1, gl);
-                if (gl + 1 < ng) unit(r0, gl + 1);
+            // A pass with a single row block (the tail of an odd count; later passes are then empty) skips the
+            // second block's MFMAs and fragment reads instead of multiplying a duplicate.
+            if (nf == 1) {
+                for (int gl = 0; gl < ng; gl += 2) {
+                    unit(r1, gl, std::integral_constant<int, 1>{});
+                    if (gl + 1 < ng) unit(r0, gl + 1, std::integral_constant<int, 1>{});
+                }
+            } else {
+                for (int gl = 0; gl < ng; gl += 2) {
+                    unit(r1, gl, std::integral_constant<int, 2>{});
+                    if (gl + 1 < ng) unit(r0, gl + 1, std::integral_constant<int, 2>{});
+                }
             }
             if (ng & 1) {               // odd unit count: restore the alternation for the next slice
 #pragma unroll
