@@ -337,7 +337,7 @@ def main():
         "value": res["images_per_s"], "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": f"{args.model} 48 packed linears (12 blocks x qkv/proj/fc1/fc2), W{args.bits}A{args.bits}, "
+        "config": {"workload": f"{args.model} {res['layers']} packed linears ({res['layers'] // 4} blocks x qkv/proj/fc1/fc2), W{args.bits}A{args.bits}, "
                                f"g=64, batch {args.batch} (M={res['M']}), fp16 in/out, stage 1 + fused unpack+GEMM",
                    "model_shapes": args.model, "bits": args.bits, "batch": args.batch, "group_size": 64},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": dk["tflops"],

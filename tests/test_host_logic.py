@@ -320,3 +320,19 @@ def test_synth():
     assert synth.algorithmic_bytes(197, 1152, 384, 3) == 858716
     assert synth.algorithmic_flops(12608, 1536, 384) == 2 * 12608 * 1536 * 384
     assert [s[1:] for s in synth.block_linear_shapes("deit_small")] == [(384, 1152), (384, 384), (384, 1536), (1536, 384)]
+
+
+def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
+    """arcq_linear_fused_kernel is a pure function of the shape (and of the ARCQ_GEMM_KERNEL override)."""
+    lib = A._lib.load()
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL", raising=False)
+    assert lib.arcq_linear_fused_kernel(197, 1152, 384) == b"gemm_splitk_kernel"
+    assert lib.arcq_linear_fused_kernel(12608, 1152, 384) == b"gemm_stream_kernel"      # wide N, one round of tiles
+    assert lib.arcq_linear_fused_kernel(12608, 384, 1536) == b"gemm_slab_kernel"        # few slabs, many row ranges
+    assert lib.arcq_linear_fused_kernel(12608, 1536, 384) == b"gemm_slab_kernel"        # K in one slab slice
+    assert lib.arcq_linear_fused_kernel(50432, 4096, 1024) == b"gemm_stream_kernel"
+    assert lib.arcq_linear_fused_kernel(5, 5, 0) == b"gemm_fused_kernel"                # K = 0: bias only
+    monkeypatch.setenv("ARCQ_GEMM_KERNEL", "slab")
+    assert lib.arcq_linear_fused_kernel(12608, 1152, 384) == b"gemm_slab_kernel"
+    monkeypatch.setenv("ARCQ_GEMM_KERNEL", "stream")
+    assert lib.arcq_linear_fused_kernel(12608, 384, 384) == b"gemm_stream_kernel"
