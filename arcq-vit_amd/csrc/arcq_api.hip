@@ -36,10 +36,10 @@ ARCQ_API const char *arcq_last_error(void) { return arcq::g_last_error; }
 
 // FQ/arcq_packed_on_the_fly.py:137-161: quantize+reconstruct the activation
 // into an fp16 buffer, then run the fused unpack+GEMM on it.
-ARCQ_API int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const float *a_codebook,
+static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds, const float *a_codebook,
                              const uint8_t *packed_w, const float *w_codebook,
                              const float *w_center, const float *w_scale, const float *w_code_sum,
-                             const float *bias, void *x_hat_ws, void *y, int y_dtype,
+                             const float *bias, void *x_hat_ws, void *w_hat_ws, void *y, int y_dtype,
                              int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
 {
     if (!x_hat_ws) return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf: x_hat_ws must not be NULL");
@@ -66,6 +66,28 @@ ARCQ_API int arcq_linear_otf(const void *x, int x_dtype, const float *a_threshol
     int rc = arcq_act_quant(x, x_dtype, a_thresholds, a_codebook, nullptr, nullptr, nullptr, nullptr, nullptr,
                             x_hat_ws, ARCQ_F16, M, K, bits, group_size, 1.0e-6f, stream);
     if (rc != ARCQ_OK) return rc;
-    return arcq_linear_fused(x_hat_ws, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype,
-                             M, N, K, bits, group_size, stream);
+    return arcq_linear_fused_ws(x_hat_ws, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, w_hat_ws, y, y_dtype,
+                                M, N, K, bits, group_size, stream);
+}
+
+ARCQ_API int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const float *a_codebook,
+                             const uint8_t *packed_w, const float *w_codebook,
+                             const float *w_center, const float *w_scale, const float *w_code_sum,
+                             const float *bias, void *x_hat_ws, void *y, int y_dtype,
+                             int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
+{
+    return linear_otf_impl(x, x_dtype, a_thresholds, a_codebook, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias,
+                           x_hat_ws, nullptr, y, y_dtype, M, N, K, bits, group_size, stream);
+}
+
+// The same layer with a second scratch buffer, for the reconstructed weights ([N,K] fp16; the counterpart of the
+// reference module's _weight_buffer, FQ/arcq_packed_on_the_fly.py:148-158).  NULL behaves like arcq_linear_otf.
+ARCQ_API int arcq_linear_otf_ws(const void *x, int x_dtype, const float *a_thresholds, const float *a_codebook,
+                                const uint8_t *packed_w, const float *w_codebook,
+                                const float *w_center, const float *w_scale, const float *w_code_sum,
+                                const float *bias, void *x_hat_ws, void *w_hat_ws, void *y, int y_dtype,
+                                int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
+{
+    return linear_otf_impl(x, x_dtype, a_thresholds, a_codebook, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias,
+                           x_hat_ws, w_hat_ws, y, y_dtype, M, N, K, bits, group_size, stream);
 }

@@ -22,6 +22,8 @@ void launch_gemm_stream(const GemmArgs &g, hipStream_t stream);
 
 // Large-M weight-stationary kernel (128-column slabs dequantized once per workgroup into LDS); requires K >= 64.
 void launch_gemm_slab(const GemmArgs &g, hipStream_t stream);
+// The same kernel fed from weights reconstructed beforehand into w_hat ([N,K] fp16, 16-byte aligned).
+void launch_gemm_slab_prebuilt(const GemmArgs &g, const void *w_hat, hipStream_t stream);
 
 // Small-M kernel (64 x 64 tiles, K split across the waves of a workgroup); requires K >= 64.
 void launch_gemm_splitk(const GemmArgs &g, hipStream_t stream);

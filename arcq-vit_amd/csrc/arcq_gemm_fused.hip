@@ -219,19 +219,21 @@ static int forced_kernel()
     return 0;
 }
 
-// Picks between the two large-M kernels with a cost model fitted to measured launch durations (microseconds,
-// output write-out excluded since both pay it alike):
+// Cost model of the large-M kernels, fitted to measured launch durations (microseconds, output write-out excluded
+// since all pay it alike):
 //   streaming kernel: waves of 256 workgroup tiles (256 x 256), each 5 + 2.0 per quantization group;
 //   weight-stationary kernel: 5.5 + 0.85 per (64-row x group) unit of a wave + 3.5 per slab slice rebuilt
-//   (4.2 when K spans several slices, which adds two barriers per slice).
+//   (4.2 when K spans several slices, which adds two barriers per slice);
 // The weight-stationary kernel wins when K fits one slice or N is small (few slabs, many row ranges); the
 // streaming kernel wins for wide N and long K.
-static bool prefer_slab(int64_t M, int64_t N, int64_t K)
+struct GemmCosts { double stream, slab; };
+
+static GemmCosts gemm_costs(int64_t M, int64_t N, int64_t K)
 {
-    if (M * K * 2 >= (int64_t(1) << 32)) return false;      // the slab kernel addresses x_hat with 32-bit byte offsets
     const int64_t G = K / 64;
     const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
-    const double stream = static_cast<double>((tiles + 255) / 256) * (5.0 + 2.0 * static_cast<double>(G));
+    GemmCosts c;
+    c.stream = static_cast<double>((tiles + 255) / 256) * (5.0 + 2.0 * static_cast<double>(G));
     const int64_t n_slabs = (N + 127) / 128, blocks = (M + 31) / 32;
     int64_t ranges = 256 / n_slabs;
     if (ranges < 1) ranges = 1;
@@ -241,9 +243,17 @@ static bool prefer_slab(int64_t M, int64_t N, int64_t K)
     const int64_t rounds = (n_slabs * ranges + 255) / 256;
     const int64_t passes = ((per_range + 3) / 4 + 1) / 2;
     const int64_t slices = (G + 5) / 6;
-    const double rebuilds = slices == 1 ? 3.5 : 4.2 * static_cast<double>(passes * slices);
-    const double slab = static_cast<double>(rounds) * (5.5 + rebuilds + 0.85 * static_cast<double>(passes * G));
-    return slab < stream;
+    const double fills = slices == 1 ? 1.0 : static_cast<double>(passes * slices);
+    const double units = 0.85 * static_cast<double>(passes * G);
+    c.slab = static_cast<double>(rounds) * (5.5 + (slices == 1 ? 3.5 : 4.2) * fills + units);
+    if (M * K * 2 >= (int64_t(1) << 32)) c.slab = 1.0e30;      // 32-bit byte offsets into x_hat
+    return c;
+}
+
+static bool prefer_slab(int64_t M, int64_t N, int64_t K)
+{
+    const GemmCosts c = gemm_costs(M, N, K);
+    return c.slab < c.stream;
 }
 
 enum GemmKernel { kTiled = 0, kStream = 1, kSlab = 2, kSplitK = 4 };
@@ -309,4 +319,48 @@ ARCQ_API int arcq_linear_fused(const void *x_hat,
             launch_out<float>(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, m, n, k, bits, st);
     }
     return launch_status("arcq_linear_fused");
+}
+
+// Whether arcq_linear_fused_ws, given a workspace, rebuilds the weights into it and runs the copying slab kernel.
+static bool workspace_pays(int64_t M, int64_t N, int64_t K)
+{
+    if (M < 512 || K < 64 || K % 64 != 0 || M * K * 2 >= (int64_t(1) << 32)) return false;
+    const char *e = getenv("ARCQ_GEMM_KERNEL");
+    if (e) return !strcmp(e, "prebuilt");
+    // Measured: copying beats both fused kernels when few slabs (N <= 1024) meet a K of three or more slab slices,
+    // i.e. when up to 256 / slabs workgroups per slab would each rebuild the same long weight rows (fc2 of DeiT-S:
+    // 36.9 us against 42.2; 50432 x 1024 x 4096: 533 us against 667 and 693).
+    return (N + 127) / 128 <= 8 && (K / 64 + 5) / 6 >= 3;
+}
+
+ARCQ_API const char *arcq_linear_fused_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace)
+{
+    if (have_workspace && N > 0 && workspace_pays(M, N, K)) return "weight_dequant8_kernel+gemm_slab_kernel";
+    return arcq_linear_fused_kernel(M, N, K);
+}
+
+// arcq_linear_fused with a scratch buffer for the reconstructed weights.  When the cost model says that rebuilding
+// the weights once (arcq_weight_dequant into w_hat_ws) and copying slab slices beats both fused kernels, that is
+// what runs; otherwise, or without a workspace, this is arcq_linear_fused.  Results are bit-identical either way.
+ARCQ_API int arcq_linear_fused_ws(const void *x_hat,
+                                  const uint8_t *packed_w, const float *w_codebook,
+                                  const float *w_center, const float *w_scale, const float *w_code_sum,
+                                  const float *bias, void *w_hat_ws, void *y, int y_dtype,
+                                  int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
+{
+    const bool prebuilt = w_hat_ws && group_size == 64 && bits_ok(bits) && N > 0 &&
+        M < (int64_t(1) << 31) - 256 && N < (int64_t(1) << 31) - 256 && K < (int64_t(1) << 31) - 256 &&
+        (y_dtype == ARCQ_F16 || y_dtype == ARCQ_F32) && x_hat && y && packed_w && w_codebook && w_center && w_scale &&
+        w_code_sum && aligned(x_hat, 16) && aligned(y, 16) && aligned(packed_w, 16) && aligned(w_hat_ws, 16) &&
+        workspace_pays(M, N, K);
+    if (!prebuilt)
+        return arcq_linear_fused(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype, M, N, K,
+                                 bits, group_size, stream);
+    const int rc = arcq_weight_dequant(packed_w, w_codebook, w_center, w_scale, w_code_sum, w_hat_ws, ARCQ_F16, N, K, bits,
+                                       group_size, stream);
+    if (rc != ARCQ_OK) return rc;
+    GemmArgs g{x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype == ARCQ_F16,
+               static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), bits};
+    launch_gemm_slab_prebuilt(g, w_hat_ws, static_cast<hipStream_t>(stream));
+    return launch_status("arcq_linear_fused_ws");
 }

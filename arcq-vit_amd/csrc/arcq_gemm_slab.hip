@@ -74,12 +74,17 @@ __device__ __forceinline__ void wave_sync()
     __builtin_amdgcn_wave_barrier();
 }
 
-template <int BITS, typename TOUT>
+// PRE = true: the weights were reconstructed beforehand (arcq_weight_dequant into a caller-provided fp16 [N,K]
+// buffer); the slab slices are then copied, global -> LDS directly, instead of rebuilt, which is what pays when many
+// workgroups would otherwise repeat the rebuild (long K, few columns, many passes).  (Copying the next slice under the
+// running slice's MFMA loop measured 2-4x slower: vector memory operations complete in issue order, so the x_hat
+// loads issued behind a copy wait for it.)
+template <int BITS, typename TOUT, bool PRE>
 __global__ void __launch_bounds__(256)
 gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, const float *__restrict__ cb,
                  const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
                  const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K,
-                 int row_ranges, int blocks_per_range)
+                 int row_ranges, int blocks_per_range, const __half *__restrict__ w_hat)
 {
     constexpr int L = 1 << BITS;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -146,12 +151,27 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
             m[r] = wcs[mi];
         }
     };
-    fetch_slice(0);
-    if (tid < 64) {
+    if constexpr (!PRE) {
+        fetch_slice(0);
+        if (tid < 64) {
 #pragma unroll
-        for (int cc = 0; cc < L; ++cc) lut[cc * 64 + lane] = cb[cc];
+            for (int cc = 0; cc < L; ++cc) lut[cc * 64 + lane] = cb[cc];
+        }
     }
     if (tid < kSlabN) s_bias[tid] = (bias && n_base + tid < N) ? bias[n_base + tid] : 0.0f;
+    // PRE: one direct global -> LDS load per slab row and wave (lanes 0..47 carry the row's 48 16-byte pieces, the
+    // hardware writes lane l's piece at the wave-uniform LDS base + 16 l); the caller waits for vmcnt and the barrier.
+    auto copy_slice = [&](int g0, int ng) {
+        const bool active = lane < 8 * ng;
+        for (int rr = 0; rr < kSlabN / 4; ++rr) {
+            const int row = wave * (kSlabN / 4) + rr;
+            const int n = min(n_base + row, N - 1);
+            if (active)
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void *)(w_hat + static_cast<int64_t>(n) * K + g0 * 64 + lane * 8),
+                    (__attribute__((address_space(3))) void *)(slab + row * kPitch), 16, 0, 0);
+        }
+    };
     auto dequant_slice = [&](int ng) {
 #pragma unroll
         for (int r = 0; r < kSliceGroups; ++r) {
@@ -268,10 +288,17 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
             const int g0 = sl * kSliceGroups;
             const int ng = min(kSliceGroups, G - g0);
             if (!(slices == 1 && pass > 0)) {
-                if (!(pass == 0 && sl == 0)) fetch_slice(g0);
-                __syncthreads();          // every wave is done reading the previous slice (and the LUT is filled)
-                dequant_slice(ng);
-                __syncthreads();
+                if constexpr (PRE) {
+                    __syncthreads();      // every wave is done reading the previous slice
+                    copy_slice(g0, ng);
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __syncthreads();
+                } else {
+                    if (!(pass == 0 && sl == 0)) fetch_slice(g0);
+                    __syncthreads();      // every wave is done reading the previous slice (and the LUT is filled)
+                    dequant_slice(ng);
+                    __syncthreads();
+                }
             }
 #pragma unroll
             for (int j = 0; j < kTJ; ++j) bf[0][j] = *reinterpret_cast<const half8_t *>(slab_lane + j * 32 * kPitch);
@@ -358,12 +385,12 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
     }
 }
 
-template <int BITS, typename TOUT>
-static void launch_slab(const GemmArgs &g, hipStream_t stream)
+template <int BITS, typename TOUT, bool PRE>
+static void launch_slab(const GemmArgs &g, hipStream_t stream, const void *w_hat)
 {
     constexpr int L = 1 << BITS;
     const size_t smem = kSlabBytes + kStageBytes + L * 64 * sizeof(float) + kSlabN * sizeof(float);
-    auto kernel = gemm_slab_kernel<BITS, TOUT>;
+    auto kernel = gemm_slab_kernel<BITS, TOUT, PRE>;
     static bool configured = false;   // per instantiation; the attribute is sticky for the process
     if (!configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -381,20 +408,28 @@ static void launch_slab(const GemmArgs &g, hipStream_t stream)
     const int tiles = n_slabs * ranges;
     hipLaunchKernelGGL(kernel, dim3(8 * ((tiles + 7) / 8)), dim3(256), smem, stream,
                        static_cast<const __half *>(g.x_hat), g.pw, g.cb, g.wc, g.ws, g.wcs, g.bias,
-                       static_cast<TOUT *>(g.y), g.M, g.N, g.K, ranges, blocks_per_range);
+                       static_cast<TOUT *>(g.y), g.M, g.N, g.K, ranges, blocks_per_range,
+                       static_cast<const __half *>(w_hat));
 }
 
 void launch_gemm_slab(const GemmArgs &g, hipStream_t stream)
 {
     if (g.y_f16) {
-        if (g.bits == 4) launch_slab<4, __half>(g, stream);
-        else if (g.bits == 3) launch_slab<3, __half>(g, stream);
-        else launch_slab<2, __half>(g, stream);
+        if (g.bits == 4) launch_slab<4, __half, false>(g, stream, nullptr);
+        else if (g.bits == 3) launch_slab<3, __half, false>(g, stream, nullptr);
+        else launch_slab<2, __half, false>(g, stream, nullptr);
     } else {
-        if (g.bits == 4) launch_slab<4, float>(g, stream);
-        else if (g.bits == 3) launch_slab<3, float>(g, stream);
-        else launch_slab<2, float>(g, stream);
+        if (g.bits == 4) launch_slab<4, float, false>(g, stream, nullptr);
+        else if (g.bits == 3) launch_slab<3, float, false>(g, stream, nullptr);
+        else launch_slab<2, float, false>(g, stream, nullptr);
     }
+}
+
+// Same product with the weights already reconstructed into w_hat ([N,K] fp16).
+void launch_gemm_slab_prebuilt(const GemmArgs &g, const void *w_hat, hipStream_t stream)
+{
+    if (g.y_f16) launch_slab<4, __half, true>(g, stream, w_hat);
+    else launch_slab<4, float, true>(g, stream, w_hat);
 }
 
 }  // namespace arcq

@@ -233,8 +233,11 @@ unpack_weight_triton = unpack_weight_hip
 # ---------------------------------------------------------------------------------------------
 def linear_fused(x_hat: torch.Tensor, packed_w: torch.Tensor, w_codebook: torch.Tensor, w_center: torch.Tensor,
                  w_scale: torch.Tensor, w_code_sum: torch.Tensor, bias: Optional[torch.Tensor], bits: int,
-                 group_size: int, out_dtype: torch.dtype = torch.float16) -> torch.Tensor:
-    """``y = x_hat @ w_hat.T + bias`` with ``w_hat`` rebuilt from packed codes inside the GEMM."""
+                 group_size: int, out_dtype: torch.dtype = torch.float16,
+                 w_hat_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``y = x_hat @ w_hat.T + bias`` with ``w_hat`` rebuilt from packed codes inside the GEMM.  ``w_hat_ws``
+    (fp16, at least N*K elements; the role of the reference module's ``_weight_buffer``) lets shapes that would
+    repeat the reconstruction in many workgroups rebuild the weights once instead; ``y`` is the same either way."""
     _check(x_hat.is_cuda and packed_w.is_cuda, "x_hat and packed_w must be CUDA tensors")
     _check(x_hat.dim() == 2 and x_hat.dtype == torch.float16, "x_hat must be float16 [M, K]")
     _check(packed_w.dtype == torch.uint8 and packed_w.dim() == 2, "packed_w must be uint8 [N, K*bits/8]")
@@ -246,19 +249,26 @@ def linear_fused(x_hat: torch.Tensor, packed_w: torch.Tensor, w_codebook: torch.
     y = torch.empty((m, n), dtype=out_dtype, device=x_hat.device)
     b = None if bias is None or bias.numel() == 0 else _f32c(bias)
     w = [packed_w.contiguous(), _f32c(w_codebook), _f32c(w_center), _f32c(w_scale), _f32c(w_code_sum)]
+    _check_w_ws(w_hat_ws, n, k)
     with torch.cuda.device(x_hat.device):
-        _lib.check(_lib.load().arcq_linear_fused(
-            _ptr(x_hat), *[_ptr(t) for t in w], _ptr(b), _ptr(y), _dtype_code(y, "y"),
+        _lib.check(_lib.load().arcq_linear_fused_ws(
+            _ptr(x_hat), *[_ptr(t) for t in w], _ptr(b), _ptr(w_hat_ws), _ptr(y), _dtype_code(y, "y"),
             m, n, k, bits, int(group_size), _stream()))
     return y
+
+
+def _check_w_ws(w_hat_ws: Optional[torch.Tensor], n: int, k: int) -> None:
+    if w_hat_ws is not None:
+        _check(w_hat_ws.is_cuda and w_hat_ws.dtype == torch.float16 and w_hat_ws.is_contiguous()
+               and w_hat_ws.numel() >= n * k, "w_hat_ws must be a contiguous float16 CUDA buffer of at least N*K elements")
 
 
 def linear_otf(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Tensor, packed_w: torch.Tensor,
                w_codebook: torch.Tensor, w_center: torch.Tensor, w_scale: torch.Tensor, w_code_sum: torch.Tensor,
                bias: Optional[torch.Tensor], bits: int, group_size: int, out_dtype: torch.dtype = torch.float16,
-               x_hat_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+               x_hat_ws: Optional[torch.Tensor] = None, w_hat_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Whole packed on-the-fly layer on ``x [M, K]`` (fp16 or fp32): stage 1 into ``x_hat_ws`` (fp16
-    ``[M, K]``, allocated if not given), then the fused GEMM."""
+    ``[M, K]``, allocated if not given), then the fused GEMM (``w_hat_ws``: see ``linear_fused``)."""
     _check(x.is_cuda and packed_w.is_cuda, "x and packed_w must be CUDA tensors")
     _check(x.dim() == 2, "x must have shape [M, K]")
     _check_bits(bits)
@@ -275,10 +285,11 @@ def linear_otf(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Te
     b = None if bias is None or bias.numel() == 0 else _f32c(bias)
     a = [_f32c(a_thresholds), _f32c(a_codebook)]
     w = [packed_w.contiguous(), _f32c(w_codebook), _f32c(w_center), _f32c(w_scale), _f32c(w_code_sum)]
+    _check_w_ws(w_hat_ws, n, k)
     with torch.cuda.device(x.device):
-        _lib.check(_lib.load().arcq_linear_otf(
+        _lib.check(_lib.load().arcq_linear_otf_ws(
             _ptr(x), _dtype_code(x, "x"), *[_ptr(t) for t in a], *[_ptr(t) for t in w], _ptr(b), _ptr(x_hat_ws),
-            _ptr(y), _dtype_code(y, "y"), m, n, k, bits, int(group_size), _stream()))
+            _ptr(w_hat_ws), _ptr(y), _dtype_code(y, "y"), m, n, k, bits, int(group_size), _stream()))
     return y
 
 

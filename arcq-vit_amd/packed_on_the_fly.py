@@ -4,10 +4,14 @@ benchmarks), constructor and buffers as FQ/arcq_packed_on_the_fly.py:93-135.
 Reference forward (:137-161): fp16 copy of x -> Triton quantize+reconstruct in place -> Triton
 unpack of the whole weight into an fp16 buffer in HBM -> cuBLAS ``F.linear``.  Here: one HIP
 stage-1 kernel writes x_hat (fp16) into a workspace, and one HIP kernel streams the packed
-codes, rebuilds the weight tile by tile in LDS and feeds fp16 MFMA; the dense weight never
-exists in HBM.  Differences a caller can observe: the input tensor is never overwritten (the
-reference overwrites a contiguous fp16 input), statistics are taken in fp32 even for fp16 input,
-and ``_weight_buffer`` is accepted but unused.
+codes, rebuilds the weight tile by tile in LDS and feeds fp16 MFMA; by default the dense weight
+never exists in HBM.  ``_weight_buffer`` (the flat fp16 scratch the reference's benchmark shares
+between all layers, scripts/benchmark_arcq_on_the_fly.py:182-191, read at :148-158) is honoured as
+an optional workspace: when it is set and the shape is one where rebuilding the weight once beats
+rebuilding it per row tile, the library reconstructs the weight into it and the GEMM copies from
+there; the result is bit-identical either way.  Differences a caller can observe: the input
+tensor is never overwritten (the reference overwrites a contiguous fp16 input) and statistics are
+taken in fp32 even for fp16 input.
 """
 from __future__ import annotations
 
@@ -103,9 +107,15 @@ class ARCQPackedLinearOnTheFly(nn.Module):
         x2 = x2.contiguous()
         ws = _workspace(x2.device, x2.numel())
         bias = self.bias_tensor if self.bias_tensor.numel() > 0 else None
+        w_ws = getattr(self, "_weight_buffer", None)
+        if w_ws is not None and (not w_ws.is_cuda or w_ws.dtype != torch.float16 or not w_ws.is_contiguous()
+                                 or w_ws.numel() < self.out_features * self.in_features):
+            raise ValueError("_weight_buffer must be a contiguous float16 CUDA tensor of at least "
+                             "out_features * in_features elements")
         y = ops.linear_otf(x2, self.activation_thresholds, self.activation_codebook, self.packed_weight_codes,
                            self.weight_codebook, self.weight_center, self.weight_scale, self.weight_code_sum,
-                           bias, self.bits, self.group_size, out_dtype=self.out_dtype, x_hat_ws=ws)
+                           bias, self.bits, self.group_size, out_dtype=self.out_dtype, x_hat_ws=ws,
+                           w_hat_ws=w_ws)
         return y.reshape(*original_shape[:-1], self.out_features)
 
     def estimated_persistent_mb(self) -> float:

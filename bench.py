@@ -31,7 +31,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch of each fused-GEMM kernel at the default workload (average over the layer shapes it serves),
 # from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a plain 256 MiB
 # copy (factors 2.00 and 1.00).  Summary: profiles/deit_small_w4a4_bs64_packed_linears.md.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): {"gemm_slab_kernel": 45.2e6, "gemm_stream_kernel": 42.8e6}}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): {"gemm_slab_kernel": 38.6e6, "gemm_stream_kernel": 42.8e6,
+                                                         "weight_dequant8_kernel+gemm_slab_kernel": 66.3e6}}
 
 
 def parse_args():
@@ -78,18 +79,23 @@ class Layer:
             setattr(c, name, getattr(self, name).clone())
         return c
 
+    # Argument lists of arcq_linear_otf_ws / arcq_linear_fused_ws.  W_WS is one fp16 scratch buffer for the
+    # reconstructed weights, shared by all layers (they run back to back on one stream).
+    W_WS = None
+
     def otf_args(self, x, ws, y, stream):
         from arcq_vit_amd._lib import ARCQ_F16
         m = x.shape[0]
         return (x.data_ptr(), ARCQ_F16, self.thr.data_ptr(), self.cb.data_ptr(), self.packed.data_ptr(),
                 self.cb.data_ptr(), self.center.data_ptr(), self.scale.data_ptr(), self.code_sum.data_ptr(),
-                self.bias.data_ptr(), ws.data_ptr(), y.data_ptr(), ARCQ_F16, m, self.n, self.k, self.bits, 64, stream)
+                self.bias.data_ptr(), ws.data_ptr(), Layer.W_WS.data_ptr(), y.data_ptr(), ARCQ_F16, m, self.n, self.k,
+                self.bits, 64, stream)
 
     def gemm_args(self, ws, y, m, stream):
         from arcq_vit_amd._lib import ARCQ_F16
         return (ws.data_ptr(), self.packed.data_ptr(), self.cb.data_ptr(), self.center.data_ptr(),
-                self.scale.data_ptr(), self.code_sum.data_ptr(), self.bias.data_ptr(), y.data_ptr(), ARCQ_F16,
-                m, self.n, self.k, self.bits, 64, stream)
+                self.scale.data_ptr(), self.code_sum.data_ptr(), self.bias.data_ptr(), Layer.W_WS.data_ptr(),
+                y.data_ptr(), ARCQ_F16, m, self.n, self.k, self.bits, 64, stream)
 
     def act_args(self, x, ws, stream):
         from arcq_vit_amd._lib import ARCQ_F16
@@ -115,6 +121,9 @@ def build_workload(model, bits, batch, dev):
     nmax = max(l.n for l in layers)
     ws = torch.empty(m * kmax, dtype=torch.float16, device=dev)
     y = torch.empty(m * nmax, dtype=torch.float16, device=dev)
+    need = max(l.n * l.k for l in layers)
+    if Layer.W_WS is None or Layer.W_WS.numel() < need:
+        Layer.W_WS = torch.empty(need, dtype=torch.float16, device=dev)
     return m, layers, inputs, ws, y
 
 
@@ -151,7 +160,7 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
 
     def step_full():
         for a in otf:
-            rc = lib.arcq_linear_otf(*a)
+            rc = lib.arcq_linear_otf_ws(*a)
             if rc:
                 _lib.check(rc)
 
@@ -163,7 +172,7 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
 
     def step_gemm():
         for a in gemms:
-            rc = lib.arcq_linear_fused(*a)
+            rc = lib.arcq_linear_fused_ws(*a)
             if rc:
                 _lib.check(rc)
 
@@ -178,11 +187,11 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
                 for l in (layers if subset is None else subset):
                     x = inputs[short(l)]
                     if kind == "full":
-                        rc = lib.arcq_linear_otf(*l.otf_args(x, ws, y, sp))
+                        rc = lib.arcq_linear_otf_ws(*l.otf_args(x, ws, y, sp))
                     elif kind == "act":
                         rc = lib.arcq_act_quant(*l.act_args(x, ws, sp))
                     else:
-                        rc = lib.arcq_linear_fused(*l.gemm_args(ws, y, m, sp))
+                        rc = lib.arcq_linear_fused_ws(*l.gemm_args(ws, y, m, sp))
                     if rc:
                         _lib.check(rc)
             return g.replay
@@ -199,7 +208,7 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
     per_kernel = {}
     by_kernel = {}
     for l in layers:
-        by_kernel.setdefault(lib.arcq_linear_fused_kernel(m, l.n, l.k).decode(), []).append(l)
+        by_kernel.setdefault(lib.arcq_linear_fused_ws_kernel(m, l.n, l.k, 1).decode(), []).append(l)
     for name, sub in by_kernel.items():
         if use_graph:
             fn = capture("gemm", sub)
@@ -208,7 +217,7 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
 
             def fn(sub_args=sub_args):
                 for a in sub_args:
-                    lib.arcq_linear_fused(*a)
+                    lib.arcq_linear_fused_ws(*a)
         t = time_loop(fn, steps, warmup)
         kf = sum(synth.algorithmic_flops(m, l.n, l.k) for l in sub)
         kb = sum(synth.algorithmic_bytes(m, l.n, l.k, bits) for l in sub)
@@ -253,13 +262,13 @@ def cold_cache_bs1(model, bits, steps, warmup, dev, footprint_bytes=512 << 20):
         ls = layers if c == 0 else [l.clone_weights() for l in layers]
         xs = {k: v.clone() for k, v in inputs.items()}
         for l in ls:                                   # warm the code path once outside capture
-            lib.arcq_linear_otf(*l.otf_args(xs[l.name.rsplit(".", 1)[-1]], ws, y, torch.cuda.current_stream().cuda_stream))
+            lib.arcq_linear_otf_ws(*l.otf_args(xs[l.name.rsplit(".", 1)[-1]], ws, y, torch.cuda.current_stream().cuda_stream))
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             sp = torch.cuda.current_stream().cuda_stream
             for l in ls:
-                rc = lib.arcq_linear_otf(*l.otf_args(xs[l.name.rsplit(".", 1)[-1]], ws, y, sp))
+                rc = lib.arcq_linear_otf_ws(*l.otf_args(xs[l.name.rsplit(".", 1)[-1]], ws, y, sp))
                 if rc:
                     _lib.check(rc)
         graphs.append((g, ls, xs))

@@ -130,6 +130,28 @@ int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const
                     const float *bias, void *x_hat_ws, void *y, int y_dtype,
                     int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
 
+/* The two entry points above with one more caller-owned scratch buffer, w_hat_ws: fp16 [N,K], 16-byte aligned, the
+ * counterpart of the reference module's optional _weight_buffer (FQ/arcq_packed_on_the_fly.py:148-158, the `out=` of
+ * unpack_weight_triton).  For shapes where many workgroups would each repeat the weight reconstruction (long K with few
+ * output columns, large models) the weights are rebuilt once into w_hat_ws (arcq_weight_dequant) and the GEMM copies
+ * them; for all other shapes, or with w_hat_ws == NULL, these behave exactly like arcq_linear_fused / arcq_linear_otf.
+ * y is bit-identical in every case; the contents of w_hat_ws after the call are unspecified. */
+int arcq_linear_fused_ws(const void *x_hat,
+                         const uint8_t *packed_w, const float *w_codebook,
+                         const float *w_center, const float *w_scale, const float *w_code_sum,
+                         const float *bias, void *w_hat_ws, void *y, int y_dtype,
+                         int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
+int arcq_linear_otf_ws(const void *x, int x_dtype, const float *a_thresholds, const float *a_codebook,
+                       const uint8_t *packed_w, const float *w_codebook,
+                       const float *w_center, const float *w_scale, const float *w_code_sum,
+                       const float *bias, void *x_hat_ws, void *w_hat_ws, void *y, int y_dtype,
+                       int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
+
+/* As arcq_linear_fused_kernel, for arcq_linear_fused_ws: "weight_dequant8_kernel+gemm_slab_kernel" when a call with
+ * these sizes and a workspace (have_workspace != 0) rebuilds the weights first, else arcq_linear_fused_kernel's
+ * answer.  A profiling aid with no counterpart in the reference. */
+const char *arcq_linear_fused_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace);
+
 /* ---- index-space linears (no reconstruction, product-table gather) ---------
  * Replace arcq_linear_forward_cuda (EXT/arcq_linear_kernel.cu:206-278; fp64
  * accumulation, kernel :22-78) and arcq_linear_forward_u8_cuda (:280-353; fp32,

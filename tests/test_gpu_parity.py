@@ -291,6 +291,73 @@ def test_fused_gemm_kernel_variants(cuda, oracle, monkeypatch, bits, out_dtype, 
     assert torch.equal(auto, outs["slab"])
 
 
+@pytest.mark.parametrize("bits,out_dtype", [(4, torch.float16), (3, torch.float32), (2, torch.float16)])
+@pytest.mark.parametrize("m,n,k", [(1500, 384, 1536),     # four slab slices: the shape class the workspace is chosen for
+                                   (1000, 200, 448),      # ragged N, a full slice plus a one-group slice
+                                   (700, 130, 64),        # one group, last slab two columns wide
+                                   (515, 520, 1216),      # 19 groups, ragged M and N
+                                   (197, 384, 1536)])     # below 512 rows: the workspace is never used
+def test_fused_gemm_weight_workspace(cuda, oracle, monkeypatch, bits, out_dtype, m, n, k):
+    """arcq_linear_fused_ws: with a weight workspace the result is bit-identical to the one without, both when the
+    library chooses (no override) and when the copy-from-workspace kernel is pinned; a pinned run leaves the
+    reconstructed fp16 weight in the workspace, bit-equal to the oracle's; a run that does not take the workspace
+    leaves it untouched."""
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 37)
+    _, thr = _cb(bits)
+    x = synth.make_activation(m, k, 37, "gelu" if k > n else "ln")
+    a = torch.from_numpy(oracle.act_quant_c(x.numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)).to(cuda)
+    bias = synth.make_bias(n, 37).to(cuda)
+    w = [t.to(cuda) for t in (packed, cb, center, scale, code_sum)]
+    run = lambda ws: ops.linear_fused(a, *w, bias, bits, 64, out_dtype=out_dtype, w_hat_ws=ws)
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL", raising=False)
+    plain = run(None)
+    ws = torch.full((n * k + 8,), -3.0, dtype=torch.float16, device=cuda)   # longer than needed: the tail stays
+    assert torch.equal(run(ws), plain)
+    ws.fill_(-3.0)
+    monkeypatch.setenv("ARCQ_GEMM_KERNEL", "prebuilt")
+    assert torch.equal(run(ws), plain)
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL")
+    got = _np(ws)
+    assert np.all(got[n * k:] == np.float16(-3.0))
+    if m >= 512:
+        want = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, bits, 64, fma=True).astype(np.float16)
+        assert np.array_equal(got[:n * k].view(np.uint16), want.reshape(-1).view(np.uint16))
+    else:
+        assert np.all(got == np.float16(-3.0))
+    monkeypatch.setenv("ARCQ_GEMM_KERNEL", "stream")                       # another pinned kernel ignores the workspace
+    ws.fill_(-3.0)
+    assert torch.equal(run(ws), run(None))
+    assert bool((ws == -3.0).all())
+
+
+def test_layer_otf_weight_workspace(cuda, oracle, monkeypatch):
+    """arcq_linear_otf_ws with both workspaces == without the weight workspace, on the shape the library picks the
+    workspace for (fc2 of DeiT-S at 8 images) and through the module's ``_weight_buffer`` attribute."""
+    from arcq_vit_amd.packed_on_the_fly import ARCQPackedLinearOnTheFly
+    m, n, k, bits = 1576, 384, 1536, 4
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL", raising=False)
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 41)
+    _, thr = _cb(bits)
+    bias = synth.make_bias(n, 41)
+    x = synth.make_activation(m, k, 41, "gelu").to(torch.float16).to(cuda)
+    d = lambda t: t.to(cuda)
+    args = (d(thr), d(cb), d(packed), d(cb), d(center), d(scale), d(code_sum), d(bias), bits, 64)
+    plain = ops.linear_otf(x, *args, out_dtype=torch.float16)
+    xw = torch.empty((m, k), dtype=torch.float16, device=cuda)
+    ww = torch.zeros(n * k, dtype=torch.float16, device=cuda)
+    assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float16, x_hat_ws=xw, w_hat_ws=ww), plain)
+    assert bool((ww != 0).any())                    # the library took the workspace for this shape
+    layer = ARCQPackedLinearOnTheFly(k, n, True, d(packed), d(cb), d(center), d(scale), d(code_sum), d(cb), d(thr),
+                                     bits, 64, d(bias))
+    y0 = layer(x)
+    layer._weight_buffer = torch.zeros(n * k + 64, dtype=torch.float16, device=cuda)
+    assert torch.equal(layer(x), y0) and torch.equal(y0, plain)
+    assert bool((layer._weight_buffer != 0).any())
+    layer._weight_buffer = torch.zeros(16, dtype=torch.float16, device=cuda)
+    with pytest.raises(ValueError):
+        layer(x)
+
+
 @pytest.mark.parametrize("bits,out_dtype", [(4, torch.float16), (3, torch.float32), (2, torch.float32)])
 @pytest.mark.parametrize("m,n,k", [(197, 1152, 384), (197, 384, 1536), (1, 70, 64), (65, 130, 1088), (300, 64, 4096)])
 def test_fused_gemm_small_m_kernels(cuda, oracle, monkeypatch, bits, out_dtype, m, n, k):

@@ -336,3 +336,16 @@ def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
     assert lib.arcq_linear_fused_kernel(12608, 1152, 384) == b"gemm_slab_kernel"
     monkeypatch.setenv("ARCQ_GEMM_KERNEL", "stream")
     assert lib.arcq_linear_fused_kernel(12608, 384, 384) == b"gemm_stream_kernel"
+    # With a weight workspace: long K and few slabs rebuild the weights once, everything else is unchanged.
+    both = b"weight_dequant8_kernel+gemm_slab_kernel"
+    assert lib.arcq_linear_fused_ws_kernel(12608, 384, 1536, 1) == b"gemm_stream_kernel"   # a pinned kernel wins
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL")
+    assert lib.arcq_linear_fused_ws_kernel(12608, 384, 1536, 1) == both
+    assert lib.arcq_linear_fused_ws_kernel(12608, 384, 1536, 0) == b"gemm_slab_kernel"
+    assert lib.arcq_linear_fused_ws_kernel(12608, 1536, 384, 1) == b"gemm_slab_kernel"     # K in one slice
+    assert lib.arcq_linear_fused_ws_kernel(50432, 4096, 1024, 1) == b"gemm_stream_kernel"  # 32 slabs
+    assert lib.arcq_linear_fused_ws_kernel(50432, 1024, 4096, 1) == both
+    assert lib.arcq_linear_fused_ws_kernel(197, 384, 1536, 1) == b"gemm_splitk_kernel"     # below 512 rows
+    monkeypatch.setenv("ARCQ_GEMM_KERNEL", "prebuilt")
+    assert lib.arcq_linear_fused_ws_kernel(12608, 1152, 384, 1) == both
+    assert lib.arcq_linear_fused_ws_kernel(12608, 1152, 384, 0) == b"gemm_stream_kernel"
