@@ -37,11 +37,14 @@ _SIGNATURES = {
                              _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
     "arcq_linear_otf_ws": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                            _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
+    "arcq_act_quant_blocked": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32, _c_ptr],
+    "arcq_linear_fused_blocked": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                                  _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
     "arcq_linear_forward_packed": [_c_ptr] * 11 + [_c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_ptr],
     "arcq_linear_forward_u8": [_c_ptr] * 11 + [_c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
 }
 EXPORTED_SYMBOLS = ("arcq_version", "arcq_last_error", "arcq_linear_fused_kernel",
-                    "arcq_linear_fused_ws_kernel") + tuple(_SIGNATURES)
+                    "arcq_linear_fused_ws_kernel", "arcq_linear_otf_ws_kernel") + tuple(_SIGNATURES)
 
 _lib = None
 _lock = threading.Lock()
@@ -71,6 +74,8 @@ def load() -> ctypes.CDLL:
             lib.arcq_linear_fused_kernel.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64]
             lib.arcq_linear_fused_ws_kernel.restype = ctypes.c_char_p
             lib.arcq_linear_fused_ws_kernel.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
+            lib.arcq_linear_otf_ws_kernel.restype = ctypes.c_char_p
+            lib.arcq_linear_otf_ws_kernel.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
             for name, argtypes in _SIGNATURES.items():
                 fn = getattr(lib, name)
                 fn.restype = _c_int

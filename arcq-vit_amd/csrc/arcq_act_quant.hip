@@ -88,6 +88,62 @@ __device__ __forceinline__ void store_tile(TOUT *__restrict__ out, int64_t elem0
     }
 }
 
+// Block-layout tiles.  When x_hat is wanted in the 32-row block layout the eight-wave GEMM reads (16-byte pieces
+// ordered [row / 32][k / 8][row % 32]) a tile is 32 rows x 2 groups instead of 64 consecutive groups: lane l owns
+// (row l % 32, group 2 * pair + l / 32), so that every piece column of the tile leaves as one contiguous 512-byte run.
+// (Scattering a 64-consecutive-groups tile into that layout as 16-byte stores measured 1.7x slower for the whole
+// kernel.)  A row's two groups are 128 contiguous values in the input, so the loads stay coalesced.  With an odd
+// group count the last pair has one group and lanes 32..63 idle.
+template <typename TIN> struct BlockTile {
+    static constexpr int pieces = 128 / Tile<TIN>::vec;     // 16-byte pieces per row of the tile (16 fp16 / 32 fp32)
+    static constexpr int rows_per_instr = 64 / pieces;      // 4 / 2
+    static constexpr int iters = 32 / rows_per_instr;       // 8 / 16 == the row-major tile's count
+};
+
+template <typename TIN>
+__device__ __forceinline__ void fetch_tile_blocked(const TIN *__restrict__ x, bool tile_valid, int64_t row0, int pair,
+                                                   int groups_per_row, TileRegs<TIN> &r, int lane)
+{
+    using B = BlockTile<TIN>;
+    const int pc = lane % B::pieces;
+    const bool ok = tile_valid && (2 * pair + pc / (B::pieces / 2) < groups_per_row);
+    const TIN *p = x + (row0 + lane / B::pieces) * (static_cast<int64_t>(groups_per_row) * 64) + pair * 128 + pc * Tile<TIN>::vec;
+#pragma unroll
+    for (int i = 0; i < B::iters; ++i)
+        r.raw[i] = ok ? *reinterpret_cast<const uint4 *>(p + static_cast<int64_t>(i * B::rows_per_instr) * groups_per_row * 64)
+                      : make_uint4(0, 0, 0, 0);
+}
+
+template <typename TIN>
+__device__ __forceinline__ void commit_tile_blocked(const TileRegs<TIN> &r, uint32_t *__restrict__ tile, int lane)
+{
+    using B = BlockTile<TIN>;
+    const int pc = lane % B::pieces;
+    const int gsel = pc / (B::pieces / 2);
+    uint32_t *dst0 = tile + (gsel * 32 + lane / B::pieces) * Tile<TIN>::stride + (pc % (B::pieces / 2)) * 4;
+#pragma unroll
+    for (int i = 0; i < B::iters; ++i) {
+        uint32_t *dst = dst0 + i * B::rows_per_instr * Tile<TIN>::stride;
+        dst[0] = r.raw[i].x; dst[1] = r.raw[i].y; dst[2] = r.raw[i].z; dst[3] = r.raw[i].w;
+    }
+}
+
+// fp16 x_hat of a block tile: instruction j writes piece columns 2j and 2j + 1 of the tile (lanes 0..31 / 32..63),
+// each 32 rows x 16 bytes = 512 contiguous bytes of the block layout.
+__device__ __forceinline__ void store_tile_blocked(__half *__restrict__ out, int64_t row_block, int pair,
+                                                   int groups_per_row, const uint32_t *__restrict__ tile, int lane)
+{
+    const int row = lane & 31;
+    __half *base = out + row_block * (static_cast<int64_t>(groups_per_row) * (64 * 32)) + row * 8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int kp = j * 2 + (lane >> 5);                 // piece column inside the tile: group kp / 8, piece kp % 8
+        if (2 * pair + kp / 8 >= groups_per_row) continue;
+        const uint32_t *src = tile + ((kp / 8) * 32 + row) * Tile<__half>::stride + (kp % 8) * 4;
+        *reinterpret_cast<uint4 *>(base + static_cast<int64_t>(pair * 16 + kp) * (32 * 8)) = make_uint4(src[0], src[1], src[2], src[3]);
+    }
+}
+
 // The lane's own group (row `lane` of the tile) as 64 floats.
 template <typename TIN>
 __device__ __forceinline__ void read_row(const uint32_t *__restrict__ row, float (&v)[64])
@@ -152,12 +208,15 @@ __device__ __forceinline__ void pack64(const uint32_t (&c)[64], uint32_t (&w)[2 
 }
 
 // CODES = false drops everything only the code outputs need (the on-the-fly layer asks for x_hat alone).
-template <typename TIN, typename TOUT, int BITS, bool CODES>
+// BLOCKED (fp16 x_hat only, no other outputs): block tiles and the 32-row block layout for x_hat; `total_groups`
+// then counts tiles' worth of work as row_blocks * pairs tiles, given by `groups_per_row` and `row_blocks`.
+template <typename TIN, typename TOUT, int BITS, bool CODES, bool BLOCKED = false>
 __global__ void __launch_bounds__(64 * kWaves)
 act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, const float *__restrict__ cb,
                      uint8_t *__restrict__ packed, uint8_t *__restrict__ codes_u8,
                      float *__restrict__ center, float *__restrict__ scale, float *__restrict__ code_sum,
-                     TOUT *__restrict__ x_hat, int64_t total_groups, float eps)
+                     TOUT *__restrict__ x_hat, int64_t total_groups, float eps,
+                     int groups_per_row, int row_blocks)
 {
     constexpr int L = 1 << BITS;
     constexpr int kStride = (Tile<TIN>::stride > Tile<TOUT>::stride) ? Tile<TIN>::stride : Tile<TOUT>::stride;
@@ -171,13 +230,20 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
     const int wave = tid >> 6;
 
     // The first tile of this wave is requested before anything else: its latency overlaps the setup below.
-    const int64_t ntiles = (total_groups + kTileGroups - 1) / kTileGroups;
+    const int pairs = BLOCKED ? (groups_per_row + 1) / 2 : 1;
+    const int64_t ntiles = BLOCKED ? static_cast<int64_t>(row_blocks) * pairs : (total_groups + kTileGroups - 1) / kTileGroups;
     const int64_t elem_end = total_groups * 64;
     TileRegs<TIN> regs;
-    {
-        const int64_t first = static_cast<int64_t>(blockIdx.x) * kWaves + wave;
-        fetch_tile<TIN>(x, first * kTileGroups * 64, elem_end, regs, lane);      // zero-fills past the end
-    }
+    auto fetch = [&](int64_t tile_id) {          // zero-fills past the end
+        if constexpr (BLOCKED) {
+            const int64_t rb = tile_id / pairs;
+            fetch_tile_blocked<TIN>(x, tile_id < ntiles, rb * 32, static_cast<int>(tile_id - rb * pairs), groups_per_row,
+                                    regs, lane);
+        } else {
+            fetch_tile<TIN>(x, tile_id * kTileGroups * 64, elem_end, regs, lane);
+        }
+    };
+    fetch(static_cast<int64_t>(blockIdx.x) * kWaves + wave);
 
     // Thresholds and codebook are requested now and first used after the first tile's statistics: the lookup
     // tables are built once per workgroup, between the two halves of the first tile, so that their load latency
@@ -195,8 +261,9 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
          tile0 += static_cast<int64_t>(gridDim.x) * kWaves) {
         const int64_t group0 = (tile0 + wave) * kTileGroups;
         const int64_t elem0 = group0 * 64;
-        if (tile0 != static_cast<int64_t>(blockIdx.x) * kWaves) fetch_tile<TIN>(x, elem0, elem_end, regs, lane);
-        commit_tile<TIN>(regs, tile, lane);
+        if (tile0 != static_cast<int64_t>(blockIdx.x) * kWaves) fetch(tile0 + wave);
+        if constexpr (BLOCKED) commit_tile_blocked<TIN>(regs, tile, lane);
+        else commit_tile<TIN>(regs, tile, lane);
         __syncthreads();
 
         float xv[64];
@@ -217,7 +284,7 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
         group_codes64<BITS, CODES>(xv, mu, var, s, th, bq, table, lut, table_ok, lane, sum_codes, code);
 
         const int64_t g = group0 + lane;
-        if (g < total_groups) {
+        if (!BLOCKED && g < total_groups) {
             if (center) center[g] = mu;
             if (scale) scale[g] = s;
             if (code_sum) code_sum[g] = sum_codes;
@@ -261,7 +328,14 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
             // rewritten now, possibly with a different stride.
             write_row<TOUT>(tile + lane * Tile<TOUT>::stride, xv);
             __syncthreads();
-            store_tile<TOUT>(x_hat, elem0, elem_end, tile, lane);
+            if constexpr (BLOCKED) {
+                const int64_t tile_id = tile0 + wave;
+                const int64_t rb = tile_id / pairs;
+                if (tile_id < ntiles)
+                    store_tile_blocked(x_hat, rb, static_cast<int>(tile_id - rb * pairs), groups_per_row, tile, lane);
+            } else {
+                store_tile<TOUT>(x_hat, elem0, elem_end, tile, lane);
+            }
         }
         __syncthreads();   // the tile is reloaded in the next iteration
     }
@@ -352,7 +426,7 @@ static int launch(const void *x, const float *thr, const float *cb, uint8_t *pac
         const bool codes = packed || codes_u8;
 #define ARCQ_LAUNCH_G64(B, C)                                                                                     \
     hipLaunchKernelGGL((act_quant_g64_kernel<TIN, TOUT, B, C>), dim3(blocks), dim3(64 * kWaves), 0, stream, xin, \
-                       thr, cb, packed, codes_u8, center, scale, code_sum, xo, total_groups, eps)
+                       thr, cb, packed, codes_u8, center, scale, code_sum, xo, total_groups, eps, 0, 0)
         if (bits == 4) { if (codes) ARCQ_LAUNCH_G64(4, true); else ARCQ_LAUNCH_G64(4, false); }
         else if (bits == 3) { if (codes) ARCQ_LAUNCH_G64(3, true); else ARCQ_LAUNCH_G64(3, false); }
         else { if (codes) ARCQ_LAUNCH_G64(2, true); else ARCQ_LAUNCH_G64(2, false); }
@@ -368,9 +442,50 @@ static int launch(const void *x, const float *thr, const float *cb, uint8_t *pac
     return launch_status("arcq_act_quant");
 }
 
+template <typename TIN>
+static int launch_blocked(const void *x, const float *thr, const float *cb, void *x_hat, int64_t rows, int64_t cols,
+                          int bits, float eps, hipStream_t stream)
+{
+    const int groups_per_row = static_cast<int>(cols / 64);
+    const int row_blocks = static_cast<int>(rows / 32);
+    const int64_t ntiles = static_cast<int64_t>(row_blocks) * ((groups_per_row + 1) / 2);
+    const int64_t want = (ntiles + kWaves - 1) / kWaves;
+    const unsigned blocks = static_cast<unsigned>(want < 4096 ? want : 4096);
+#define ARCQ_LAUNCH_BLOCKED(B)                                                                                       \
+    hipLaunchKernelGGL((act_quant_g64_kernel<TIN, __half, B, false, true>), dim3(blocks), dim3(64 * kWaves), 0, stream, \
+                       static_cast<const TIN *>(x), thr, cb, nullptr, nullptr, nullptr, nullptr, nullptr,            \
+                       static_cast<__half *>(x_hat), rows * groups_per_row, eps, groups_per_row, row_blocks)
+    if (bits == 4) ARCQ_LAUNCH_BLOCKED(4);
+    else if (bits == 3) ARCQ_LAUNCH_BLOCKED(3);
+    else ARCQ_LAUNCH_BLOCKED(2);
+#undef ARCQ_LAUNCH_BLOCKED
+    return launch_status("arcq_act_quant_blocked");
+}
+
 }  // namespace arcq
 
 using namespace arcq;
+
+ARCQ_API int arcq_act_quant_blocked(const void *x, int x_dtype, const float *thresholds, const float *codebook,
+                                    void *x_hat_blocked, int64_t rows, int64_t cols, int bits, float eps, void *stream)
+{
+    if (!bits_ok(bits)) return fail(ARCQ_ERR_BITS, "arcq_act_quant_blocked: bits must be 2, 3, or 4");
+    if (rows < 0 || cols < 0) return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked: bad sizes");
+    if (cols % 64 != 0) return fail(ARCQ_ERR_GROUP, "arcq_act_quant_blocked: in_features must be divisible by 64");
+    if (rows % 32 != 0) return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked: rows must be a multiple of 32");
+    if (x_dtype != ARCQ_F32 && x_dtype != ARCQ_F16)
+        return fail(ARCQ_ERR_DTYPE, "arcq_act_quant_blocked: x must be float32 or float16");
+    if (rows * cols == 0) return ARCQ_OK;
+    if (!x || !thresholds || !codebook || !x_hat_blocked)
+        return fail(ARCQ_ERR_NULL, "arcq_act_quant_blocked: x, thresholds, codebook and x_hat_blocked must not be NULL");
+    if (x_hat_blocked == x) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_act_quant_blocked: x_hat_blocked must not alias x");
+    if (rows * cols * 2 >= (int64_t(1) << 32)) return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked: tensor too large");
+    if (!aligned(x, 16) || !aligned(x_hat_blocked, 16))
+        return fail(ARCQ_ERR_ALIGN, "arcq_act_quant_blocked: x and x_hat_blocked must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (x_dtype == ARCQ_F32) return launch_blocked<float>(x, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, st);
+    return launch_blocked<__half>(x, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, st);
+}
 
 ARCQ_API int arcq_act_quant(const void *x, int x_dtype, const float *thresholds, const float *codebook,
                             uint8_t *packed, uint8_t *codes_u8, float *center, float *scale, float *code_sum,

@@ -39,7 +39,7 @@ ARCQ_API const char *arcq_last_error(void) { return arcq::g_last_error; }
 static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds, const float *a_codebook,
                              const uint8_t *packed_w, const float *w_codebook,
                              const float *w_center, const float *w_scale, const float *w_code_sum,
-                             const float *bias, void *x_hat_ws, void *w_hat_ws, void *y, int y_dtype,
+                             const float *bias, void *x_hat_ws, void *w_hat_ws, bool scratch_only, void *y, int y_dtype,
                              int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
 {
     if (!x_hat_ws) return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf: x_hat_ws must not be NULL");
@@ -63,6 +63,14 @@ static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds
             return arcq::launch_status("arcq_linear_otf");
         }
     }
+    // Scratch-only workspaces and whole 32-row blocks: x_hat in the block layout, eight-wave weight-stationary GEMM
+    // (bit-identical results; invalid arguments fall through to the entry points below, which report them).
+    if (scratch_only && group_size == 64 && arcq::bits_ok(bits) && arcq::otf_blocked_pays(M, N, K) && x != x_hat_ws) {
+        const int rc = arcq_act_quant_blocked(x, x_dtype, a_thresholds, a_codebook, x_hat_ws, M, K, bits, 1.0e-6f, stream);
+        if (rc != ARCQ_OK) return rc;
+        return arcq_linear_fused_blocked(x_hat_ws, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, w_hat_ws, y,
+                                         y_dtype, M, N, K, bits, group_size, stream);
+    }
     int rc = arcq_act_quant(x, x_dtype, a_thresholds, a_codebook, nullptr, nullptr, nullptr, nullptr, nullptr,
                             x_hat_ws, ARCQ_F16, M, K, bits, group_size, 1.0e-6f, stream);
     if (rc != ARCQ_OK) return rc;
@@ -77,7 +85,7 @@ ARCQ_API int arcq_linear_otf(const void *x, int x_dtype, const float *a_threshol
                              int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
 {
     return linear_otf_impl(x, x_dtype, a_thresholds, a_codebook, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias,
-                           x_hat_ws, nullptr, y, y_dtype, M, N, K, bits, group_size, stream);
+                           x_hat_ws, nullptr, false, y, y_dtype, M, N, K, bits, group_size, stream);
 }
 
 // The same layer with a second scratch buffer, for the reconstructed weights ([N,K] fp16; the counterpart of the
@@ -89,5 +97,5 @@ ARCQ_API int arcq_linear_otf_ws(const void *x, int x_dtype, const float *a_thres
                                 int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
 {
     return linear_otf_impl(x, x_dtype, a_thresholds, a_codebook, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias,
-                           x_hat_ws, w_hat_ws, y, y_dtype, M, N, K, bits, group_size, stream);
+                           x_hat_ws, w_hat_ws, true, y, y_dtype, M, N, K, bits, group_size, stream);
 }

@@ -333,10 +333,78 @@ static bool workspace_pays(int64_t M, int64_t N, int64_t K)
     return (N + 127) / 128 <= 8 && (K / 64 + 5) / 6 >= 3;
 }
 
+// The same question for the eight-wave kernel, which has less to gain from each rebuild it skips: measured, copying
+// wins from two slab slices on while the slabs are few (DeiT-B proj 36.0 us against 37.9, fc2 107 against 130;
+// ViT-L proj 144 against 169, fc2 491 against 616) and loses or ties everywhere else.  "prebuilt" forces the copy.
+static bool workspace_pays_blocked(int64_t N, int64_t K)
+{
+    if (K < 64 || K % 64 != 0) return false;
+    const char *e = getenv("ARCQ_GEMM_KERNEL");
+    if (e && !strcmp(e, "prebuilt")) return true;
+    return (N + 127) / 128 <= 8 && (K / 64 + 5) / 6 >= 2;
+}
+
 ARCQ_API const char *arcq_linear_fused_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace)
 {
     if (have_workspace && N > 0 && workspace_pays(M, N, K)) return "weight_dequant8_kernel+gemm_slab_kernel";
     return arcq_linear_fused_kernel(M, N, K);
+}
+
+// Shapes for which arcq_linear_otf_ws quantizes into the 32-row block layout and multiplies with the eight-wave
+// weight-stationary kernel: whole 32-row blocks from 512 rows on.  Measured against the row-major kernels on the
+// twelve DeiT-S / DeiT-B / ViT-L layer shapes it is the fastest on ten and within 3 % (DeiT-B proj, ViT-L fc1) on
+// two.  ARCQ_GEMM_KERNEL pins a row-major kernel, or this one with "slab8" / "prebuilt".
+bool arcq::otf_blocked_pays(int64_t M, int64_t N, int64_t K)
+{
+    if (M < 512 || M % 32 != 0 || N <= 0 || K < 64 || K % 64 != 0 || M * K * 2 >= (int64_t(1) << 32)) return false;
+    if (M >= (int64_t(1) << 31) - 256 || N >= (int64_t(1) << 31) - 256) return false;
+    const char *e = getenv("ARCQ_GEMM_KERNEL");
+    if (e) return !strcmp(e, "slab8") || !strcmp(e, "prebuilt");
+    return true;
+}
+
+ARCQ_API const char *arcq_linear_otf_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace)
+{
+    if (otf_blocked_pays(M, N, K))
+        return (have_workspace && workspace_pays_blocked(N, K)) ? "weight_dequant8_kernel+gemm_slab8_kernel"
+                                                                   : "gemm_slab8_kernel";
+    return arcq_linear_fused_ws_kernel(M, N, K, have_workspace);
+}
+
+// The fused GEMM on x_hat in the 32-row block layout (what arcq_act_quant_blocked writes): always the eight-wave
+// weight-stationary kernel; with a weight workspace, and a shape where that pays, on weights reconstructed once.
+ARCQ_API int arcq_linear_fused_blocked(const void *x_hat_blocked,
+                                       const uint8_t *packed_w, const float *w_codebook,
+                                       const float *w_center, const float *w_scale, const float *w_code_sum,
+                                       const float *bias, void *w_hat_ws, void *y, int y_dtype,
+                                       int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
+{
+    if (!bits_ok(bits)) return fail(ARCQ_ERR_BITS, "arcq_linear_fused_blocked: bits must be 2, 3, or 4");
+    if (group_size != 64) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_fused_blocked: group_size must be 64 (got %d)", group_size);
+    if (M < 0 || N < 0 || K < 0) return fail(ARCQ_ERR_SHAPE, "arcq_linear_fused_blocked: negative size");
+    if (K % 64 != 0) return fail(ARCQ_ERR_GROUP, "arcq_linear_fused_blocked: in_features must be divisible by group_size");
+    if (M % 32 != 0) return fail(ARCQ_ERR_SHAPE, "arcq_linear_fused_blocked: rows must be a multiple of 32");
+    if (y_dtype != ARCQ_F16 && y_dtype != ARCQ_F32)
+        return fail(ARCQ_ERR_DTYPE, "arcq_linear_fused_blocked: y must be float16 or float32");
+    if (M == 0 || N == 0) return ARCQ_OK;
+    if (K == 0) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_fused_blocked: in_features must not be 0");
+    if (!y || !x_hat_blocked || !packed_w || !w_codebook || !w_center || !w_scale || !w_code_sum)
+        return fail(ARCQ_ERR_NULL, "arcq_linear_fused_blocked: NULL tensor pointer");
+    if (M >= (int64_t(1) << 31) - 256 || N >= (int64_t(1) << 31) - 256 || M * K * 2 >= (int64_t(1) << 32))
+        return fail(ARCQ_ERR_SHAPE, "arcq_linear_fused_blocked: M, N or K too large");
+    if (!aligned(x_hat_blocked, 16) || !aligned(y, 16) || !aligned(packed_w, 16) || !aligned(w_hat_ws, 16))
+        return fail(ARCQ_ERR_ALIGN, "arcq_linear_fused_blocked: x_hat_blocked, y, packed_w and w_hat_ws must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool prebuilt = w_hat_ws && workspace_pays_blocked(N, K);
+    if (prebuilt) {
+        const int rc = arcq_weight_dequant(packed_w, w_codebook, w_center, w_scale, w_code_sum, w_hat_ws, ARCQ_F16, N, K,
+                                           bits, group_size, stream);
+        if (rc != ARCQ_OK) return rc;
+    }
+    GemmArgs g{x_hat_blocked, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype == ARCQ_F16,
+               static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), bits};
+    launch_gemm_slab8(g, prebuilt ? w_hat_ws : nullptr, st);
+    return launch_status("arcq_linear_fused_blocked");
 }
 
 // arcq_linear_fused with a scratch buffer for the reconstructed weights.  When the cost model says that rebuilding

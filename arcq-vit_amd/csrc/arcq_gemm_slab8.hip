@@ -1,0 +1,393 @@
+// Stages 2+3 fused, weight-stationary kernel for x_hat in the 32-row block layout:
+//   y[M,N] = x_hat[M,K] * w_hat[N,K]^T + bias,   x_hat stored as 16-byte pieces [M/32][K/8][32 rows][8 values].
+//
+// In that layout the MFMA fragment of a 32-row block and k-step (lane = row, 8 consecutive k) is one fully coalesced
+// 16-byte load per lane (512 contiguous bytes per half wave), so x_hat goes from L2 straight into the operand
+// registers: no LDS tile, no LDS writes, no wave-level synchronization.  That frees enough registers and LDS
+// bandwidth for EIGHT waves per workgroup (two per SIMD), each multiplying one 32-row block at a time with the
+// resident 128-column slab; the second wave of a SIMD keeps the matrix pipe busy while the first waits on L2.
+// (With x_hat row-major a fragment load touches 32 rows per instruction, which costs the texture path more than the
+// MFMAs it feeds; staging through LDS instead saturates LDS bandwidth at two waves per SIMD.)
+//
+// Slab handling (a slice of up to 6 groups rebuilt from the packed codes once per workgroup, or copied from weights
+// reconstructed beforehand), k order inside a group (lane half h covers k = 32h + 8*step ... + 7 in k-step `step`)
+// and operand roles (w_hat is the MFMA "A" operand; accumulator element v of lane l is
+// y[m = l%32][n = 32j + 8*(v/4) + 4*(l/32) + v%4]) are those of the four-wave kernel; both accumulate in the same
+// k order, so their results are bit-identical.
+#include "arcq_common.h"
+#include "arcq_gemm.h"
+
+#include <type_traits>
+
+namespace arcq {
+namespace {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 512;
+constexpr int kWaves = kThreads / 64;
+constexpr int kSlabN = 128;                 // columns per slab
+constexpr int kSliceGroups = 6;             // groups per K slice
+constexpr int kPitch = kSliceGroups * 128 + 16;   // bytes per slab row: 384 halves + 16 B pad (conflict-free 16-B reads)
+constexpr int kSlabBytes = kSlabN * kPitch;       // 100352
+constexpr int kTJ = kSlabN / 32;            // 4 column blocks
+constexpr int kStageRow = 144;              // bytes per staged output row: 128 + 16 pad
+constexpr int kStageTile = 32 * kStageRow;  // 4608 B per wave
+constexpr int kStageBytes = kWaves * kStageTile;
+constexpr int kHalves = 2 * kSliceGroups;   // half groups (32 codes) per slab row and slice
+constexpr int kRounds = kSlabN * kHalves / kThreads;       // half groups per thread and slice
+static_assert(kSlabN * kHalves % kThreads == 0, "slice work must divide evenly");
+
+template <int BITS>
+__device__ __forceinline__ void load_codes(const uint8_t *__restrict__ p, uint32_t (&w)[BITS])
+{
+    if constexpr (BITS == 4) {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(p);
+        w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
+    } else if constexpr (BITS == 2) {
+        const u32x2_t v = *reinterpret_cast<const u32x2_t *>(p);
+        w[0] = v[0]; w[1] = v[1];
+    } else {
+        const uint32_t *q = reinterpret_cast<const uint32_t *>(p);
+        w[0] = q[0]; w[1] = q[1]; w[2] = q[2];
+    }
+}
+
+template <int BITS>
+__device__ __forceinline__ uint32_t code_at(const uint32_t (&w)[BITS], int q)
+{
+    const int bit = q * BITS;
+    const int d = bit >> 5, sh = bit & 31;
+    uint32_t v = w[d] >> sh;
+    if (sh + BITS > 32) v |= w[d + 1] << (32 - sh);
+    return v & ((1u << BITS) - 1u);
+}
+
+// PRE = true: the weights were reconstructed beforehand into a fp16 [N,K] buffer; slab slices are copied,
+// global -> LDS directly, instead of rebuilt.
+template <int BITS, typename TOUT, bool PRE>
+__global__ void __launch_bounds__(kThreads)
+gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw, const float *__restrict__ cb,
+                  const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
+                  const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K,
+                  int row_ranges, int blocks_per_range, const __half *__restrict__ w_hat)
+{
+    constexpr int L = 1 << BITS;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    unsigned char *slab = smem;
+    float *lut = reinterpret_cast<float *>(smem + kSlabBytes + kStageBytes);      // [L][64]
+    float *s_bias = lut + L * 64;                                                   // [128]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int lr = lane & 31;
+    const int lh = lane >> 5;
+    const int G = K / 64;
+    const int64_t pcols = static_cast<int64_t>(K) * BITS / 8;
+
+    // Tile = (row range, slab), slab fastest; each XCD (workgroups are dealt to the 8 XCDs round-robin) takes a
+    // contiguous run of tiles so that the slabs sharing a row range read x_hat through one L2.
+    const int n_slabs = (N + kSlabN - 1) / kSlabN;
+    const int tiles = n_slabs * row_ranges;
+    const int per_xcd = (tiles + 7) / 8;
+    const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (tile >= tiles) return;
+    const int n_base = (tile % n_slabs) * kSlabN;
+    const int total_blocks = M / 32;
+    const int blk0 = (tile / n_slabs) * blocks_per_range;
+    const int blk1 = min(total_blocks, blk0 + blocks_per_range);
+    // Row blocks of this wave: a contiguous eighth of the workgroup's range, one block per pass.
+    const int passes = (blk1 - blk0 + kWaves - 1) / kWaves;      // same for all waves: barriers stay uniform
+    const int wblk0 = min(blk1, blk0 + wave * passes);
+    const int wblk1 = min(blk1, wblk0 + passes);
+    const int slices = (G + kSliceGroups - 1) / kSliceGroups;
+
+    const unsigned char *slab_lane = slab + lr * kPitch + lh * 64;
+    unsigned char *stage = smem + kSlabBytes + wave * kStageTile;
+
+    // Codes and metadata of one slice: fetched into registers first (for the first slice at the very top of the
+    // kernel, so that this latency, the codebook's and the first x_hat units' all overlap), converted afterwards.
+    // Half group number p = round * 512 + tid: consecutive lanes read consecutive pieces of a weight row.
+    uint32_t codes[kRounds][BITS];
+    float c[kRounds], s[kRounds], m[kRounds];
+    auto fetch_slice = [&](int g0) {
+#pragma unroll
+        for (int r = 0; r < kRounds; ++r) {
+            const int p = r * kThreads + tid;
+            const int row = p / kHalves, q = p % kHalves;
+            const int n = min(n_base + row, N - 1);
+            const int g = min(g0 + (q >> 1), G - 1);
+            load_codes<BITS>(pw + static_cast<int64_t>(n) * pcols + g * (8 * BITS) + (q & 1) * (4 * BITS), codes[r]);
+            const int64_t mi = static_cast<int64_t>(n) * G + g;
+            c[r] = wc[mi];
+            s[r] = ws[mi];
+            m[r] = wcs[mi];
+        }
+    };
+    if constexpr (!PRE) {
+        fetch_slice(0);
+        if (tid < 64) {
+#pragma unroll
+            for (int cc = 0; cc < L; ++cc) lut[cc * 64 + lane] = cb[cc];
+        }
+    }
+    if (tid < kSlabN) s_bias[tid] = (bias && n_base + tid < N) ? bias[n_base + tid] : 0.0f;
+    // PRE: one direct global -> LDS load per slab row (lanes 0..47 carry the row's 48 16-byte pieces, the hardware
+    // writes lane l's piece at the wave-uniform LDS base + 16 l); the caller waits for vmcnt and the barrier.
+    auto copy_slice = [&](int g0, int ng) {
+        const bool active = lane < 8 * ng;
+        for (int rr = 0; rr < kSlabN / kWaves; ++rr) {
+            const int row = wave * (kSlabN / kWaves) + rr;
+            const int n = min(n_base + row, N - 1);
+            if (active)
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void *)(w_hat + static_cast<int64_t>(n) * K + g0 * 64 + lane * 8),
+                    (__attribute__((address_space(3))) void *)(slab + row * kPitch), 16, 0, 0);
+        }
+    };
+    auto dequant_slice = [&](int ng) {
+#pragma unroll
+        for (int r = 0; r < kRounds; ++r) {
+            const int p = r * kThreads + tid;
+            const int row = p / kHalves, q = p % kHalves;
+            if ((q >> 1) < ng) {
+                // All 32 table lookups of this half group are issued before the first is used.
+                const float mg = m[r] * 0.015625f;          // S/64, exact
+                float v[32];
+#pragma unroll
+                for (int e = 0; e < 32; ++e) {
+                    const uint32_t code = code_at<BITS>(codes[r], e);
+                    v[e] = *reinterpret_cast<const float *>(
+                        reinterpret_cast<const char *>(lut) + ((code << 8) | (static_cast<uint32_t>(lane) << 2)));
+                }
+                unsigned char *dst = slab + row * kPitch + q * 64;
+#pragma unroll
+                for (int q8 = 0; q8 < 4; ++q8) {
+                    half8_t hv;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        hv[e] = static_cast<_Float16>(fma_f32(v[q8 * 8 + e] - mg, s[r], c[r]));
+                    *reinterpret_cast<half8_t *>(dst + q8 * 16) = hv;
+                }
+            }
+        }
+    };
+
+    // x_hat load cursor: the next unit (pass, group) to fetch; it runs two units ahead of the MFMA loop.  A unit is
+    // one group of the wave's current 32-row block: four fragments (k-steps) of 16 bytes per lane, 512 contiguous
+    // bytes per half wave and k-step.  Past the wave's last block the cursor keeps re-reading a valid block.
+    int ld_pass = 0, ld_g = 0;
+    const char *ld_base;
+    const int lane_off = lh * 2048 + lr * 16;
+    auto set_base = [&](int pass) {
+        const int blk = min(wblk0 + pass, total_blocks - 1);
+        ld_base = reinterpret_cast<const char *>(xb) + static_cast<int64_t>(blk) * K * 64 + lane_off;
+    };
+    auto load_unit = [&](u32x4_t (&r)[4]) {
+        const char *p = ld_base + ld_g * 4096;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) r[kk] = *reinterpret_cast<const u32x4_t *>(p + kk * 512);
+        if (++ld_g == G) {
+            ld_g = 0;
+            if (ld_pass + 1 < passes) set_base(++ld_pass);
+        }
+    };
+
+    u32x4_t r0[4], r1[4], r2[4];       // ring: the unit being multiplied, the next one, the one after
+    set_base(0);
+    load_unit(r0);
+    load_unit(r1);
+
+    for (int pass = 0; pass < passes; ++pass) {
+        const int pblk = wblk0 + pass;
+        const bool live = pblk < wblk1;          // a wave past its last block only keeps the barriers company
+        float16_t acc[kTJ];
+#pragma unroll
+        for (int j = 0; j < kTJ; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][v] = 0.0f;
+
+        // One unit = one group = four k-steps of 4 MFMAs.  Every k-step also issues the LDS reads of the next
+        // k-step's w_hat fragments; k-step 1 fetches the unit two ahead into the ring slot the previous unit used.
+        // `bf[0]` holds the fragments of (gl, k-step 0) on entry and of (gl + 1, k-step 0) on exit.
+        half8_t bf[2][kTJ];
+        auto unit = [&](const u32x4_t (&cur_set)[4], u32x4_t (&load_set)[4], int gl) {
+            const unsigned char *bsrc = slab_lane + gl * 128;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const int cur = kk & 1, nxt = cur ^ 1;
+#pragma unroll
+                for (int j = 0; j < kTJ; ++j)       // kk == 3 reads the next group (past the slice on its last unit: unused)
+                    bf[nxt][j] = *reinterpret_cast<const half8_t *>(bsrc + j * 32 * kPitch + (kk + 1) * 16 + (kk == 3 ? 64 : 0));
+                if (kk == 1) load_unit(load_set);
+                half8_t af;
+                __builtin_memcpy(&af, &cur_set[kk], 16);
+#pragma unroll
+                for (int j = 0; j < kTJ; ++j)
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af, acc[j], 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < kTJ; ++q) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // 1 MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 // 1 LDS read
+                    if (kk == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // 1 global load
+                }
+            }
+        };
+
+        for (int sl = 0; sl < slices; ++sl) {
+            const int g0 = sl * kSliceGroups;
+            const int ng = min(kSliceGroups, G - g0);
+            if (!(slices == 1 && pass > 0)) {
+                if constexpr (PRE) {
+                    __syncthreads();      // every wave is done reading the previous slice
+                    copy_slice(g0, ng);
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __syncthreads();
+                } else {
+                    if (!(pass == 0 && sl == 0)) fetch_slice(g0);
+                    __syncthreads();      // every wave is done reading the previous slice (and the LUT is filled)
+                    dequant_slice(ng);
+                    __syncthreads();
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < kTJ; ++j) bf[0][j] = *reinterpret_cast<const half8_t *>(slab_lane + j * 32 * kPitch);
+            // The ring is walked with fixed register names, three units at a time; every slice but the last has
+            // six units, and a last slice that is not a multiple of three rotates the ring back into place.
+            for (int gl = 0; gl < ng; gl += 3) {
+                unit(r0, r2, gl);
+                if (gl + 1 < ng) unit(r1, r0, gl + 1);
+                if (gl + 2 < ng) unit(r2, r1, gl + 2);
+            }
+            const int rot = ng % 3;
+            if (rot == 1) {             // r0 consumed (r2 refilled): next unit is in r1, the one after in r2
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const u32x4_t a0 = r1[t], a1 = r2[t];
+                    r0[t] = a0;
+                    r1[t] = a1;
+                }
+            } else if (rot == 2) {      // r0, r1 consumed (r2, r0 refilled): next unit is in r2, the one after in r0
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const u32x4_t a0 = r2[t], a1 = r0[t];
+                    r0[t] = a0;
+                    r1[t] = a1;
+                }
+            }
+        }
+
+        // ---- epilogue of this pass: the 32 x 128 block leaves in chunks of 128 bytes per row through the wave's
+        // private staging tile (LDS operations of one wave execute in order: no wait is needed between them) ----
+        constexpr int kChunkCols = 128 / static_cast<int>(sizeof(TOUT));     // 64 (fp16) / 32 (fp32)
+        constexpr int kChunks = kSlabN / kChunkCols;
+        constexpr int kBlocksPerChunk = kChunkCols / 32;
+        constexpr int kVec = 16 / static_cast<int>(sizeof(TOUT));
+        if (live) {
+#pragma unroll
+            for (int ch = 0; ch < kChunks; ++ch) {
+#pragma unroll
+                for (int jj = 0; jj < kBlocksPerChunk; ++jj) {
+                    const int j = ch * kBlocksPerChunk + jj;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int cl = jj * 32 + 8 * q + 4 * lh;            // column inside the chunk
+                        const float4 bv = *reinterpret_cast<const float4 *>(s_bias + j * 32 + 8 * q + 4 * lh);
+                        const float o0 = acc[j][4 * q] + bv.x, o1 = acc[j][4 * q + 1] + bv.y;
+                        const float o2 = acc[j][4 * q + 2] + bv.z, o3 = acc[j][4 * q + 3] + bv.w;
+                        unsigned char *dst = stage + lr * kStageRow + cl * static_cast<int>(sizeof(TOUT));
+                        if constexpr (sizeof(TOUT) == 2) {
+                            const __half2 lo = __floats2half2_rn(o0, o1), hi = __floats2half2_rn(o2, o3);
+                            u32x2_t pk;
+                            pk[0] = *reinterpret_cast<const uint32_t *>(&lo);
+                            pk[1] = *reinterpret_cast<const uint32_t *>(&hi);
+                            *reinterpret_cast<u32x2_t *>(dst) = pk;
+                        } else {
+                            u32x4_t pk;
+                            pk[0] = __float_as_uint(o0); pk[1] = __float_as_uint(o1);
+                            pk[2] = __float_as_uint(o2); pk[3] = __float_as_uint(o3);
+                            *reinterpret_cast<u32x4_t *>(dst) = pk;
+                        }
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();
+                const int col0 = n_base + ch * kChunkCols;
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    const int r = it * 8 + (lane >> 3);
+                    const int cseg = lane & 7;
+                    const int row = pblk * 32 + r;
+                    const int col = col0 + cseg * kVec;
+                    if (col < N) {
+                        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(stage + r * kStageRow + cseg * 16);
+                        TOUT *dst = y + static_cast<int64_t>(row) * N + col;
+                        if ((N % kVec) == 0 && col + kVec <= N) {
+                            *reinterpret_cast<u32x4_t *>(dst) = v;
+                        } else {
+                            const TOUT *e = reinterpret_cast<const TOUT *>(&v);
+#pragma unroll
+                            for (int k = 0; k < kVec; ++k)
+                                if (col + k < N) dst[k] = e[k];
+                        }
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+    }
+}
+
+template <int BITS, typename TOUT, bool PRE>
+void launch_slab8(const GemmArgs &g, hipStream_t stream, const void *w_hat)
+{
+    constexpr int L = 1 << BITS;
+    const size_t smem = kSlabBytes + kStageBytes + L * 64 * sizeof(float) + kSlabN * sizeof(float);
+    auto kernel = gemm_slab8_kernel<BITS, TOUT, PRE>;
+    static bool configured = false;   // per instantiation; the attribute is sticky for the process
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  static_cast<int>(smem));
+        configured = true;
+    }
+    // One workgroup per CU where possible: split the 32-row blocks into as many ranges as CUs/slabs allow.
+    const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
+    const int total_blocks = g.M / 32;
+    int ranges = 256 / n_slabs;
+    if (ranges < 1) ranges = 1;
+    if (ranges > total_blocks) ranges = total_blocks;
+    const int blocks_per_range = (total_blocks + ranges - 1) / ranges;
+    ranges = (total_blocks + blocks_per_range - 1) / blocks_per_range;
+    const int tiles = n_slabs * ranges;
+    hipLaunchKernelGGL(kernel, dim3(8 * ((tiles + 7) / 8)), dim3(kThreads), smem, stream,
+                       static_cast<const __half *>(g.x_hat), g.pw, g.cb, g.wc, g.ws, g.wcs, g.bias,
+                       static_cast<TOUT *>(g.y), g.M, g.N, g.K, ranges, blocks_per_range,
+                       static_cast<const __half *>(w_hat));
+}
+
+}  // namespace
+
+// g.x_hat is in the 32-row block layout; g.M must be a positive multiple of 32 and g.K of 64.  w_hat != nullptr:
+// weights already reconstructed ([N,K] fp16), slab slices are copied from there.
+void launch_gemm_slab8(const GemmArgs &g, const void *w_hat, hipStream_t stream)
+{
+    if (w_hat) {
+        if (g.y_f16) launch_slab8<4, __half, true>(g, stream, w_hat);
+        else launch_slab8<4, float, true>(g, stream, w_hat);
+        return;
+    }
+    if (g.y_f16) {
+        if (g.bits == 4) launch_slab8<4, __half, false>(g, stream, nullptr);
+        else if (g.bits == 3) launch_slab8<3, __half, false>(g, stream, nullptr);
+        else launch_slab8<2, __half, false>(g, stream, nullptr);
+    } else {
+        if (g.bits == 4) launch_slab8<4, float, false>(g, stream, nullptr);
+        else if (g.bits == 3) launch_slab8<3, float, false>(g, stream, nullptr);
+        else launch_slab8<2, float, false>(g, stream, nullptr);
+    }
+}
+
+}  // namespace arcq

@@ -266,9 +266,14 @@ def _check_w_ws(w_hat_ws: Optional[torch.Tensor], n: int, k: int) -> None:
 def linear_otf(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Tensor, packed_w: torch.Tensor,
                w_codebook: torch.Tensor, w_center: torch.Tensor, w_scale: torch.Tensor, w_code_sum: torch.Tensor,
                bias: Optional[torch.Tensor], bits: int, group_size: int, out_dtype: torch.dtype = torch.float16,
-               x_hat_ws: Optional[torch.Tensor] = None, w_hat_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+               x_hat_ws: Optional[torch.Tensor] = None, w_hat_ws: Optional[torch.Tensor] = None,
+               scratch: bool = False) -> torch.Tensor:
     """Whole packed on-the-fly layer on ``x [M, K]`` (fp16 or fp32): stage 1 into ``x_hat_ws`` (fp16
-    ``[M, K]``, allocated if not given), then the fused GEMM (``w_hat_ws``: see ``linear_fused``)."""
+    ``[M, K]``, allocated if not given), then the fused GEMM (``w_hat_ws``: see ``linear_fused``).
+
+    With ``scratch=True`` or a ``w_hat_ws`` both workspaces are scratch only: ``y`` is the same bit for bit, but
+    ``x_hat_ws`` may afterwards hold ``x_hat`` in the library's 32-row block layout instead of row-major (the
+    faster path for whole 32-row blocks).  Otherwise ``x_hat_ws`` holds ``x_hat`` row-major after the call."""
     _check(x.is_cuda and packed_w.is_cuda, "x and packed_w must be CUDA tensors")
     _check(x.dim() == 2, "x must have shape [M, K]")
     _check_bits(bits)
@@ -287,9 +292,57 @@ def linear_otf(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Te
     w = [packed_w.contiguous(), _f32c(w_codebook), _f32c(w_center), _f32c(w_scale), _f32c(w_code_sum)]
     _check_w_ws(w_hat_ws, n, k)
     with torch.cuda.device(x.device):
-        _lib.check(_lib.load().arcq_linear_otf_ws(
-            _ptr(x), _dtype_code(x, "x"), *[_ptr(t) for t in a], *[_ptr(t) for t in w], _ptr(b), _ptr(x_hat_ws),
-            _ptr(w_hat_ws), _ptr(y), _dtype_code(y, "y"), m, n, k, bits, int(group_size), _stream()))
+        if scratch or w_hat_ws is not None:
+            _lib.check(_lib.load().arcq_linear_otf_ws(
+                _ptr(x), _dtype_code(x, "x"), *[_ptr(t) for t in a], *[_ptr(t) for t in w], _ptr(b), _ptr(x_hat_ws),
+                _ptr(w_hat_ws), _ptr(y), _dtype_code(y, "y"), m, n, k, bits, int(group_size), _stream()))
+        else:
+            _lib.check(_lib.load().arcq_linear_otf(
+                _ptr(x), _dtype_code(x, "x"), *[_ptr(t) for t in a], *[_ptr(t) for t in w], _ptr(b), _ptr(x_hat_ws),
+                _ptr(y), _dtype_code(y, "y"), m, n, k, bits, int(group_size), _stream()))
+    return y
+
+
+def quantize_activation_blocked(x: torch.Tensor, thresholds: torch.Tensor, codebook: torch.Tensor, bits: int,
+                                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Stage 1 (group size 64) with ``x_hat`` written as fp16 in the 32-row block layout
+    ``[M/32, K/8, 32, 8]`` that ``linear_fused_blocked`` reads; same values as ``dequant_activation_hip``."""
+    _check(x.is_cuda and x.dim() == 2, "x must be a CUDA tensor [M, K]")
+    _check_bits(bits)
+    x = x.contiguous()
+    m, k = x.shape
+    _check(m % 32 == 0 and k % 64 == 0, "the block layout needs M divisible by 32 and K by 64")
+    if out is None:
+        out = torch.empty((m // 32, k // 8, 32, 8), dtype=torch.float16, device=x.device)
+    else:
+        _check(out.is_cuda and out.dtype == torch.float16 and out.is_contiguous() and out.numel() >= m * k,
+               "out must be a contiguous float16 CUDA buffer of at least M*K elements")
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().arcq_act_quant_blocked(
+            _ptr(x), _dtype_code(x, "x"), _ptr(_f32c(thresholds)), _ptr(_f32c(codebook)), _ptr(out), m, k, bits, 1.0e-6,
+            _stream()))
+    return out
+
+
+def linear_fused_blocked(x_hat_blocked: torch.Tensor, m: int, k: int, packed_w: torch.Tensor, w_codebook: torch.Tensor,
+                         w_center: torch.Tensor, w_scale: torch.Tensor, w_code_sum: torch.Tensor,
+                         bias: Optional[torch.Tensor], bits: int, out_dtype: torch.dtype = torch.float16,
+                         w_hat_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``linear_fused`` on ``x_hat`` ``[m, k]`` held in the 32-row block layout (``quantize_activation_blocked``)."""
+    _check(x_hat_blocked.is_cuda and x_hat_blocked.dtype == torch.float16 and x_hat_blocked.is_contiguous()
+           and x_hat_blocked.numel() >= m * k, "x_hat_blocked must be a contiguous float16 CUDA buffer of M*K elements")
+    _check(packed_w.is_cuda and packed_w.dtype == torch.uint8 and packed_w.dim() == 2, "packed_w must be uint8 [N, K*bits/8]")
+    _check_bits(bits)
+    n = packed_w.shape[0]
+    _check(packed_w.shape[1] == (k * bits + 7) // 8, "packed_w row length does not match K*bits/8")
+    y = torch.empty((m, n), dtype=out_dtype, device=x_hat_blocked.device)
+    b = None if bias is None or bias.numel() == 0 else _f32c(bias)
+    w = [packed_w.contiguous(), _f32c(w_codebook), _f32c(w_center), _f32c(w_scale), _f32c(w_code_sum)]
+    _check_w_ws(w_hat_ws, n, k)
+    with torch.cuda.device(x_hat_blocked.device):
+        _lib.check(_lib.load().arcq_linear_fused_blocked(
+            _ptr(x_hat_blocked), *[_ptr(t) for t in w], _ptr(b), _ptr(w_hat_ws), _ptr(y), _dtype_code(y, "y"),
+            m, n, k, bits, 64, _stream()))
     return y
 
 

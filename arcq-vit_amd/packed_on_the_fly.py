@@ -115,7 +115,7 @@ class ARCQPackedLinearOnTheFly(nn.Module):
         y = ops.linear_otf(x2, self.activation_thresholds, self.activation_codebook, self.packed_weight_codes,
                            self.weight_codebook, self.weight_center, self.weight_scale, self.weight_code_sum,
                            bias, self.bits, self.group_size, out_dtype=self.out_dtype, x_hat_ws=ws,
-                           w_hat_ws=w_ws)
+                           w_hat_ws=w_ws, scratch=True)
         return y.reshape(*original_shape[:-1], self.out_features)
 
     def estimated_persistent_mb(self) -> float:

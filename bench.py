@@ -97,6 +97,24 @@ class Layer:
                 self.scale.data_ptr(), self.code_sum.data_ptr(), self.bias.data_ptr(), Layer.W_WS.data_ptr(),
                 y.data_ptr(), ARCQ_F16, m, self.n, self.k, self.bits, 64, stream)
 
+    # The two halves of arcq_linear_otf_ws on their own: for shapes it runs in the 32-row block layout the halves are
+    # arcq_act_quant_blocked / arcq_linear_fused_blocked, else arcq_act_quant / arcq_linear_fused_ws.
+    def blocked(self, lib, m):
+        return b"slab8" in lib.arcq_linear_otf_ws_kernel(m, self.n, self.k, 1)
+
+    def call_act(self, lib, x, ws, stream):
+        from arcq_vit_amd._lib import ARCQ_F16
+        if self.blocked(lib, x.shape[0]):
+            return lib.arcq_act_quant_blocked(x.data_ptr(), ARCQ_F16, self.thr.data_ptr(), self.cb.data_ptr(),
+                                              ws.data_ptr(), x.shape[0], self.k, self.bits, 1.0e-6, stream)
+        return lib.arcq_act_quant(*self.act_args(x, ws, stream))
+
+    def call_gemm(self, lib, ws, y, m, stream):
+        if self.blocked(lib, m):
+            a = self.gemm_args(ws, y, m, stream)
+            return lib.arcq_linear_fused_blocked(*a)
+        return lib.arcq_linear_fused_ws(*self.gemm_args(ws, y, m, stream))
+
     def act_args(self, x, ws, stream):
         from arcq_vit_amd._lib import ARCQ_F16
         m = x.shape[0]
@@ -155,8 +173,6 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
         return l.name.rsplit(".", 1)[-1]
 
     otf = [l.otf_args(inputs[short(l)], ws, y, stream) for l in layers]
-    acts = [l.act_args(inputs[short(l)], ws, stream) for l in layers]
-    gemms = [l.gemm_args(ws, y, m, stream) for l in layers]
 
     def step_full():
         for a in otf:
@@ -165,14 +181,14 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
                 _lib.check(rc)
 
     def step_act():
-        for a in acts:
-            rc = lib.arcq_act_quant(*a)
+        for l in layers:
+            rc = l.call_act(lib, inputs[short(l)], ws, stream)
             if rc:
                 _lib.check(rc)
 
     def step_gemm():
-        for a in gemms:
-            rc = lib.arcq_linear_fused_ws(*a)
+        for l in layers:
+            rc = l.call_gemm(lib, ws, y, m, stream)
             if rc:
                 _lib.check(rc)
 
@@ -189,9 +205,9 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
                     if kind == "full":
                         rc = lib.arcq_linear_otf_ws(*l.otf_args(x, ws, y, sp))
                     elif kind == "act":
-                        rc = lib.arcq_act_quant(*l.act_args(x, ws, sp))
+                        rc = l.call_act(lib, x, ws, sp)
                     else:
-                        rc = lib.arcq_linear_fused_ws(*l.gemm_args(ws, y, m, sp))
+                        rc = l.call_gemm(lib, ws, y, m, sp)
                     if rc:
                         _lib.check(rc)
             return g.replay
@@ -208,16 +224,14 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
     per_kernel = {}
     by_kernel = {}
     for l in layers:
-        by_kernel.setdefault(lib.arcq_linear_fused_ws_kernel(m, l.n, l.k, 1).decode(), []).append(l)
+        by_kernel.setdefault(lib.arcq_linear_otf_ws_kernel(m, l.n, l.k, 1).decode(), []).append(l)
     for name, sub in by_kernel.items():
         if use_graph:
             fn = capture("gemm", sub)
         else:
-            sub_args = [l.gemm_args(ws, y, m, stream) for l in sub]
-
-            def fn(sub_args=sub_args):
-                for a in sub_args:
-                    lib.arcq_linear_fused_ws(*a)
+            def fn(sub=sub):
+                for l in sub:
+                    l.call_gemm(lib, ws, y, m, stream)
         t = time_loop(fn, steps, warmup)
         kf = sum(synth.algorithmic_flops(m, l.n, l.k) for l in sub)
         kb = sum(synth.algorithmic_bytes(m, l.n, l.k, bits) for l in sub)

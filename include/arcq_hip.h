@@ -135,7 +135,9 @@ int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const
  * unpack_weight_triton).  For shapes where many workgroups would each repeat the weight reconstruction (long K with few
  * output columns, large models) the weights are rebuilt once into w_hat_ws (arcq_weight_dequant) and the GEMM copies
  * them; for all other shapes, or with w_hat_ws == NULL, these behave exactly like arcq_linear_fused / arcq_linear_otf.
- * y is bit-identical in every case; the contents of w_hat_ws after the call are unspecified. */
+ * y is bit-identical in every case; the contents of w_hat_ws after the call are unspecified.  arcq_linear_otf_ws treats
+ * x_hat_ws as scratch too (unspecified contents afterwards: it may hold x_hat in the block layout described below);
+ * call arcq_linear_otf to get x_hat row-major in x_hat_ws. */
 int arcq_linear_fused_ws(const void *x_hat,
                          const uint8_t *packed_w, const float *w_codebook,
                          const float *w_center, const float *w_scale, const float *w_code_sum,
@@ -151,6 +153,27 @@ int arcq_linear_otf_ws(const void *x, int x_dtype, const float *a_thresholds, co
  * these sizes and a workspace (have_workspace != 0) rebuilds the weights first, else arcq_linear_fused_kernel's
  * answer.  A profiling aid with no counterpart in the reference. */
 const char *arcq_linear_fused_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace);
+
+/* ---- 32-row block layout for x_hat ------------------------------------------
+ * No counterpart in the reference (its x_hat goes to cuBLAS row-major, FQ/arcq_packed_on_the_fly.py:141-160): these
+ * are the two halves arcq_linear_otf_ws is made of when its workspaces are scratch only, exposed so that each can be
+ * called, timed and tested on its own.  The layout stores 16-byte pieces of 8 values as
+ *     x_hat_blocked[((row / 32) * (K / 8) + k / 8) * 32 + row % 32][k % 8]        (rows a multiple of 32, K of 64),
+ * which makes an MFMA operand fragment (32 rows x 8 values) one contiguous 512-byte run.  Values are the ones
+ * arcq_act_quant writes row-major, bit for bit; arcq_linear_fused_blocked's result equals arcq_linear_fused's on the
+ * row-major tensor, bit for bit.  group_size is 64; M * K must stay below 2^31. */
+int arcq_act_quant_blocked(const void *x, int x_dtype, const float *thresholds, const float *codebook,
+                           void *x_hat_blocked, int64_t rows, int64_t cols, int bits, float eps, void *stream);
+int arcq_linear_fused_blocked(const void *x_hat_blocked,
+                              const uint8_t *packed_w, const float *w_codebook,
+                              const float *w_center, const float *w_scale, const float *w_code_sum,
+                              const float *bias, void *w_hat_ws, void *y, int y_dtype,
+                              int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
+
+/* Kernels arcq_linear_otf_ws runs after stage 1 for these sizes: "gemm_slab8_kernel" or
+ * "weight_dequant8_kernel+gemm_slab8_kernel" when it takes the block layout, else arcq_linear_fused_ws_kernel's
+ * answer.  A profiling aid with no counterpart in the reference. */
+const char *arcq_linear_otf_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace);
 
 /* ---- index-space linears (no reconstruction, product-table gather) ---------
  * Replace arcq_linear_forward_cuda (EXT/arcq_linear_kernel.cu:206-278; fp64

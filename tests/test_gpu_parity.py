@@ -358,6 +358,100 @@ def test_layer_otf_weight_workspace(cuda, oracle, monkeypatch):
         layer(x)
 
 
+def _to_blocked(t):
+    """Row-major [M, K] -> the 32-row block layout [M/32, K/8, 32, 8]."""
+    m, k = t.shape
+    return t.reshape(m // 32, 32, k // 8, 8).permute(0, 2, 1, 3).contiguous()
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("m,k,in_dtype", [(64, 384, torch.float16), (96, 448, torch.float32),    # 7 groups: a half-empty tile
+                                          (32, 64, torch.float16),                               # one group per row
+                                          (1024, 1536, torch.float16), (160, 832, torch.float32)])
+def test_stage1_block_layout(cuda, oracle, bits, m, k, in_dtype):
+    """arcq_act_quant_blocked writes the values of the row-major stage 1 (and of the oracle), bit for bit, at
+    [row / 32][k / 8][row % 32][k % 8]."""
+    cb, thr = _cb(bits)
+    x = synth.make_activation(m, k, 43, "gelu").to(in_dtype)
+    want = oracle.act_quant_c(x.float().numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)
+    got = ops.quantize_activation_blocked(x.to(cuda), thr.to(cuda), cb.to(cuda), bits)
+    assert tuple(got.shape) == (m // 32, k // 8, 32, 8) and got.dtype == torch.float16
+    assert np.array_equal(_np(got).view(np.uint16), _np(_to_blocked(torch.from_numpy(want))).view(np.uint16))
+    if in_dtype == torch.float16:
+        assert torch.equal(_to_blocked(ops.dequant_activation_hip(x.to(cuda), thr.to(cuda), cb.to(cuda), 64)), got)
+    # a larger out buffer is only written where the layout says
+    buf = torch.full((m * k + 64,), -3.0, dtype=torch.float16, device=cuda)
+    ops.quantize_activation_blocked(x.to(cuda), thr.to(cuda), cb.to(cuda), bits, out=buf)
+    assert torch.equal(buf[:m * k].view(m // 32, k // 8, 32, 8), got) and bool((buf[m * k:] == -3.0).all())
+
+
+@pytest.mark.parametrize("bits,out_dtype", [(4, torch.float16), (3, torch.float32), (2, torch.float16)])
+@pytest.mark.parametrize("m,n,k", [(1504, 384, 1536),     # four slab slices; 47 blocks over 8 waves
+                                   (1024, 200, 448),      # ragged N, a full slice plus a one-group slice (ring rotation by 1)
+                                   (704, 130, 64),        # one group, last slab two columns wide
+                                   (512, 520, 832),       # 13 groups (ring rotation by 1), ragged N
+                                   (544, 256, 512),       # 8 groups: last slice of two (ring rotation by 2)
+                                   (2112, 1152, 384),     # K in one slice, several passes per wave
+                                   (32, 128, 128)])       # a single row block: seven waves idle
+def test_fused_gemm_block_layout(cuda, oracle, monkeypatch, bits, out_dtype, m, n, k):
+    """arcq_linear_fused_blocked on x_hat in the block layout == arcq_linear_fused on the same x_hat row-major: within
+    the fp64 bound, bit-identical to the four-wave weight-stationary kernel (same k order), with and without a weight
+    workspace and a bias."""
+    monkeypatch.setenv("ARCQ_GEMM_KERNEL", "slab")
+    ref, _ = _check_fused(cuda, oracle, m, n, k, bits, seed=47, out_dtype=out_dtype)
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL")
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 47)
+    _, thr = _cb(bits)
+    x = synth.make_activation(m, k, 47, "gelu" if k > n else "ln")
+    a = torch.from_numpy(oracle.act_quant_c(x.numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16))
+    xb = _to_blocked(a).to(cuda)
+    bias = synth.make_bias(n, 47).to(cuda)
+    w = [t.to(cuda) for t in (packed, cb, center, scale, code_sum)]
+    y = ops.linear_fused_blocked(xb, m, k, *w, bias, bits, out_dtype=out_dtype)
+    assert y.dtype == out_dtype and tuple(y.shape) == (m, n)
+    if m >= 512:
+        assert torch.equal(y, ref)
+    else:       # below 512 rows the row-major entry point takes the split-K kernel: another summation order
+        assert torch.allclose(y.float(), ref.float(), rtol=2e-3, atol=2e-3)
+    ws = torch.full((n * k + 8,), -3.0, dtype=torch.float16, device=cuda)
+    monkeypatch.setenv("ARCQ_GEMM_KERNEL", "prebuilt")
+    assert torch.equal(ops.linear_fused_blocked(xb, m, k, *w, bias, bits, out_dtype=out_dtype, w_hat_ws=ws), y)
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL")
+    want_w = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, bits, 64, fma=True).astype(np.float16)
+    assert np.array_equal(_np(ws)[:n * k].view(np.uint16), want_w.reshape(-1).view(np.uint16))
+    assert bool((ws[n * k:] == -3.0).all())
+    assert torch.equal(ops.linear_fused_blocked(xb, m, k, *w, bias, bits, out_dtype=out_dtype, w_hat_ws=ws), y)   # library's choice
+    nb = ops.linear_fused_blocked(xb, m, k, *w, None, bits, out_dtype=torch.float32)
+    yb = ops.linear_fused_blocked(xb, m, k, *w, bias, bits, out_dtype=torch.float32)
+    assert torch.equal(nb + bias, yb)            # the bias is one fp32 addition before the output rounding
+
+
+@pytest.mark.parametrize("m", [1504, 1576])     # whole 32-row blocks (block layout inside) / not (row-major inside)
+def test_layer_otf_scratch_workspaces(cuda, oracle, monkeypatch, m):
+    """arcq_linear_otf_ws (scratch-only workspaces) == arcq_linear_otf bit for bit, whichever layout it uses inside."""
+    n, k, bits = 384, 1536, 4
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL", raising=False)
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 53)
+    _, thr = _cb(bits)
+    bias = synth.make_bias(n, 53)
+    x = synth.make_activation(m, k, 53, "gelu").to(torch.float16).to(cuda)
+    d = lambda t: t.to(cuda)
+    args = (d(thr), d(cb), d(packed), d(cb), d(center), d(scale), d(code_sum), d(bias), bits, 64)
+    xw = torch.empty((m, k), dtype=torch.float16, device=cuda)
+    plain = ops.linear_otf(x, *args, out_dtype=torch.float16, x_hat_ws=xw)
+    want_xhat = oracle.act_quant_c(x.float().cpu().numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)
+    assert np.array_equal(_np(xw).view(np.uint16), want_xhat.view(np.uint16))       # row-major without `scratch`
+    xs = torch.empty((m, k), dtype=torch.float16, device=cuda)
+    assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float16, x_hat_ws=xs, scratch=True), plain)
+    if m % 32 == 0:
+        assert torch.equal(xs.view(m // 32, k // 8, 32, 8), _to_blocked(xw))
+    ww = torch.zeros(n * k, dtype=torch.float16, device=cuda)
+    assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float16, x_hat_ws=xs, w_hat_ws=ww), plain)
+    assert bool((ww != 0).any())
+    y32 = ops.linear_otf(x.float(), *args, out_dtype=torch.float32, scratch=True)   # fp32 in, fp32 out
+    assert torch.allclose(y32, plain.float(), rtol=2e-3, atol=2e-3)
+
+
 @pytest.mark.parametrize("bits,out_dtype", [(4, torch.float16), (3, torch.float32), (2, torch.float32)])
 @pytest.mark.parametrize("m,n,k", [(197, 1152, 384), (197, 384, 1536), (1, 70, 64), (65, 130, 1088), (300, 64, 4096)])
 def test_fused_gemm_small_m_kernels(cuda, oracle, monkeypatch, bits, out_dtype, m, n, k):
