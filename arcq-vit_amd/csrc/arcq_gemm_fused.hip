@@ -333,15 +333,17 @@ static bool workspace_pays(int64_t M, int64_t N, int64_t K)
     return (N + 127) / 128 <= 8 && (K / 64 + 5) / 6 >= 3;
 }
 
-// The same question for the eight-wave kernel, which has less to gain from each rebuild it skips: measured, copying
-// wins from two slab slices on while the slabs are few (DeiT-B proj 36.0 us against 37.9, fc2 107 against 130;
-// ViT-L proj 144 against 169, fc2 491 against 616) and loses or ties everywhere else.  "prebuilt" forces the copy.
+// The same question for the eight-wave kernel.  Measured: copying wins whenever K spans three or more slab slices
+// (DeiT-S fc2 31.1 us against 33.9, DeiT-B fc2 87.5 against 108, ViT-L proj 136 against 160, fc1 450 against 468,
+// fc2 461 against 588), with two slices only while the slabs are few (DeiT-B proj 31.4 against 33.0, but qkv 76.6
+// against 72.1), and never when the slab stays resident (one slice).  "prebuilt" forces the copy.
 static bool workspace_pays_blocked(int64_t N, int64_t K)
 {
     if (K < 64 || K % 64 != 0) return false;
     const char *e = getenv("ARCQ_GEMM_KERNEL");
     if (e && !strcmp(e, "prebuilt")) return true;
-    return (N + 127) / 128 <= 8 && (K / 64 + 5) / 6 >= 2;
+    const int64_t slabs = (N + 127) / 128, slices = (K / 64 + 5) / 6;
+    return slices >= 3 || (slices == 2 && slabs <= 8);
 }
 
 ARCQ_API const char *arcq_linear_fused_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace)

@@ -100,10 +100,9 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     const int total_blocks = M / 32;
     const int blk0 = (tile / n_slabs) * blocks_per_range;
     const int blk1 = min(total_blocks, blk0 + blocks_per_range);
-    // Row blocks of this wave: a contiguous eighth of the workgroup's range, one block per pass.
+    // Row blocks of this wave: blk0 + wave, + 8, + 16, ... (one per pass).  Dealing them round-robin instead of in
+    // contiguous runs keeps the four SIMDs (waves w and w + 4 share one) within one block of each other.
     const int passes = (blk1 - blk0 + kWaves - 1) / kWaves;      // same for all waves: barriers stay uniform
-    const int wblk0 = min(blk1, blk0 + wave * passes);
-    const int wblk1 = min(blk1, wblk0 + passes);
     const int slices = (G + kSliceGroups - 1) / kSliceGroups;
 
     const unsigned char *slab_lane = slab + lr * kPitch + lh * 64;
@@ -184,7 +183,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     const char *ld_base;
     const int lane_off = lh * 2048 + lr * 16;
     auto set_base = [&](int pass) {
-        const int blk = min(wblk0 + pass, total_blocks - 1);
+        const int blk = min(blk0 + pass * kWaves + wave, total_blocks - 1);
         ld_base = reinterpret_cast<const char *>(xb) + static_cast<int64_t>(blk) * K * 64 + lane_off;
     };
     auto load_unit = [&](u32x4_t (&r)[4]) {
@@ -203,8 +202,8 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     load_unit(r1);
 
     for (int pass = 0; pass < passes; ++pass) {
-        const int pblk = wblk0 + pass;
-        const bool live = pblk < wblk1;          // a wave past its last block only keeps the barriers company
+        const int pblk = blk0 + pass * kWaves + wave;
+        const bool live = pblk < blk1;           // a wave past its last block only keeps the barriers company
         float16_t acc[kTJ];
 #pragma unroll
         for (int j = 0; j < kTJ; ++j)
@@ -254,6 +253,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
                     __syncthreads();
                 }
             }
+            if (!live) continue;        // (once past its last block a wave stays past it: the ring no longer matters)
 #pragma unroll
             for (int j = 0; j < kTJ; ++j) bf[0][j] = *reinterpret_cast<const half8_t *>(slab_lane + j * 32 * kPitch);
             // The ring is walked with fixed register names, three units at a time; every slice but the last has

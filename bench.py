@@ -31,8 +31,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch of each fused-GEMM kernel at the default workload (average over the layer shapes it serves),
 # from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a plain 256 MiB
 # copy (factors 2.00 and 1.00).  Summary: profiles/deit_small_w4a4_bs64_packed_linears.md.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): {"gemm_slab_kernel": 38.6e6, "gemm_stream_kernel": 42.8e6,
-                                                         "weight_dequant8_kernel+gemm_slab_kernel": 66.3e6}}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): {"gemm_slab8_kernel": 39.8e6,
+                                                         "weight_dequant8_kernel+gemm_slab8_kernel": 63.2e6}}
 
 
 def parse_args():

@@ -356,7 +356,8 @@ def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 1) == both8
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 0) == b"gemm_slab8_kernel"
     assert lib.arcq_linear_otf_ws_kernel(12608, 768, 768, 1) == both8                      # two slices, six slabs
-    assert lib.arcq_linear_otf_ws_kernel(50432, 4096, 1024, 1) == b"gemm_slab8_kernel"     # 32 slabs: no copy
+    assert lib.arcq_linear_otf_ws_kernel(50432, 4096, 1024, 1) == both8                    # three slices
+    assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 1) == b"gemm_slab8_kernel"      # two slices, 18 slabs
     assert lib.arcq_linear_otf_ws_kernel(1576, 384, 1536, 1) == both                       # 1576 % 32 != 0: row-major
     assert lib.arcq_linear_otf_ws_kernel(197, 1152, 384, 1) == b"gemm_splitk_kernel"
     monkeypatch.setenv("ARCQ_GEMM_KERNEL", "stream")
