@@ -33,6 +33,8 @@
 //    the kernel falls back to the compare chain.
 // The arithmetic itself lives in arcq_act_quant_core.h (shared with the fused small-M layer kernel).
 #include "arcq_act_quant_core.h"
+#include "arcq_gemm.h"
+#include "arcq_weight_dequant_core.h"
 
 namespace arcq {
 
@@ -208,15 +210,26 @@ __device__ __forceinline__ void pack64(const uint32_t (&c)[64], uint32_t (&w)[2 
 }
 
 // CODES = false drops everything only the code outputs need (the on-the-fly layer asks for x_hat alone).
-// BLOCKED (fp16 x_hat only, no other outputs): block tiles and the 32-row block layout for x_hat; `total_groups`
-// then counts tiles' worth of work as row_blocks * pairs tiles, given by `groups_per_row` and `row_blocks`.
+// Weight reconstruction carried along by a block-layout stage-1 launch: the first `blocks` workgroups of the grid
+// rebuild out[N,K] (fp16) from packed codes instead of quantizing activations.  Both are inputs of the same GEMM and
+// independent of each other, so one launch does for two.  blocks == 0: nothing to carry.
+struct WeightJob {
+    const uint8_t *packed;
+    const float *cb, *center, *scale, *code_sum;
+    __half *out;
+    int64_t N, K;
+    unsigned blocks;
+};
+
+// BLOCKED (fp16 x_hat only, no other outputs): block tiles and the 32-row block layout for x_hat; the work is
+// row_blocks * ceil(groups_per_row / 2) tiles, and `wj` may add weight-reconstruction workgroups in front.
 template <typename TIN, typename TOUT, int BITS, bool CODES, bool BLOCKED = false>
 __global__ void __launch_bounds__(64 * kWaves)
 act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, const float *__restrict__ cb,
                      uint8_t *__restrict__ packed, uint8_t *__restrict__ codes_u8,
                      float *__restrict__ center, float *__restrict__ scale, float *__restrict__ code_sum,
                      TOUT *__restrict__ x_hat, int64_t total_groups, float eps,
-                     int groups_per_row, int row_blocks)
+                     int groups_per_row, int row_blocks, WeightJob wj)
 {
     constexpr int L = 1 << BITS;
     constexpr int kStride = (Tile<TIN>::stride > Tile<TOUT>::stride) ? Tile<TIN>::stride : Tile<TOUT>::stride;
@@ -228,6 +241,18 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+
+    unsigned first_block = 0, act_blocks = gridDim.x;
+    if constexpr (BLOCKED) {
+        if (blockIdx.x < wj.blocks) {          // workgroup-uniform: this workgroup rebuilds weights and is done
+            weight_dequant8_block<__half, BITS>(blockIdx.x, lut, wj.packed, wj.cb, wj.center, wj.scale, wj.code_sum,
+                                                wj.out, wj.N, wj.K, 64);
+            return;
+        }
+        first_block = wj.blocks;
+        act_blocks = gridDim.x - wj.blocks;
+    }
+    const int64_t wg = blockIdx.x - first_block;       // workgroup number among the activation workgroups
 
     // The first tile of this wave is requested before anything else: its latency overlaps the setup below.
     const int pairs = BLOCKED ? (groups_per_row + 1) / 2 : 1;
@@ -243,7 +268,7 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
             fetch_tile<TIN>(x, tile_id * kTileGroups * 64, elem_end, regs, lane);
         }
     };
-    fetch(static_cast<int64_t>(blockIdx.x) * kWaves + wave);
+    fetch(wg * kWaves + wave);
 
     // Thresholds and codebook are requested now and first used after the first tile's statistics: the lookup
     // tables are built once per workgroup, between the two halves of the first tile, so that their load latency
@@ -257,11 +282,10 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
     uint32_t *tile = tiles[wave];
 
     // All four waves run the same number of iterations so that the barriers below are uniform.
-    for (int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kWaves; tile0 < ntiles;
-         tile0 += static_cast<int64_t>(gridDim.x) * kWaves) {
+    for (int64_t tile0 = wg * kWaves; tile0 < ntiles; tile0 += static_cast<int64_t>(act_blocks) * kWaves) {
         const int64_t group0 = (tile0 + wave) * kTileGroups;
         const int64_t elem0 = group0 * 64;
-        if (tile0 != static_cast<int64_t>(blockIdx.x) * kWaves) fetch(tile0 + wave);
+        if (tile0 != wg * kWaves) fetch(tile0 + wave);
         if constexpr (BLOCKED) commit_tile_blocked<TIN>(regs, tile, lane);
         else commit_tile<TIN>(regs, tile, lane);
         __syncthreads();
@@ -426,7 +450,7 @@ static int launch(const void *x, const float *thr, const float *cb, uint8_t *pac
         const bool codes = packed || codes_u8;
 #define ARCQ_LAUNCH_G64(B, C)                                                                                     \
     hipLaunchKernelGGL((act_quant_g64_kernel<TIN, TOUT, B, C>), dim3(blocks), dim3(64 * kWaves), 0, stream, xin, \
-                       thr, cb, packed, codes_u8, center, scale, code_sum, xo, total_groups, eps, 0, 0)
+                       thr, cb, packed, codes_u8, center, scale, code_sum, xo, total_groups, eps, 0, 0, WeightJob{})
         if (bits == 4) { if (codes) ARCQ_LAUNCH_G64(4, true); else ARCQ_LAUNCH_G64(4, false); }
         else if (bits == 3) { if (codes) ARCQ_LAUNCH_G64(3, true); else ARCQ_LAUNCH_G64(3, false); }
         else { if (codes) ARCQ_LAUNCH_G64(2, true); else ARCQ_LAUNCH_G64(2, false); }
@@ -444,17 +468,17 @@ static int launch(const void *x, const float *thr, const float *cb, uint8_t *pac
 
 template <typename TIN>
 static int launch_blocked(const void *x, const float *thr, const float *cb, void *x_hat, int64_t rows, int64_t cols,
-                          int bits, float eps, hipStream_t stream)
+                          int bits, float eps, hipStream_t stream, const WeightJob &wj)
 {
     const int groups_per_row = static_cast<int>(cols / 64);
     const int row_blocks = static_cast<int>(rows / 32);
     const int64_t ntiles = static_cast<int64_t>(row_blocks) * ((groups_per_row + 1) / 2);
     const int64_t want = (ntiles + kWaves - 1) / kWaves;
-    const unsigned blocks = static_cast<unsigned>(want < 4096 ? want : 4096);
+    const unsigned blocks = static_cast<unsigned>(want < 4096 ? want : 4096) + wj.blocks;
 #define ARCQ_LAUNCH_BLOCKED(B)                                                                                       \
     hipLaunchKernelGGL((act_quant_g64_kernel<TIN, __half, B, false, true>), dim3(blocks), dim3(64 * kWaves), 0, stream, \
                        static_cast<const TIN *>(x), thr, cb, nullptr, nullptr, nullptr, nullptr, nullptr,            \
-                       static_cast<__half *>(x_hat), rows * groups_per_row, eps, groups_per_row, row_blocks)
+                       static_cast<__half *>(x_hat), rows * groups_per_row, eps, groups_per_row, row_blocks, wj)
     if (bits == 4) ARCQ_LAUNCH_BLOCKED(4);
     else if (bits == 3) ARCQ_LAUNCH_BLOCKED(3);
     else ARCQ_LAUNCH_BLOCKED(2);
@@ -466,8 +490,9 @@ static int launch_blocked(const void *x, const float *thr, const float *cb, void
 
 using namespace arcq;
 
-ARCQ_API int arcq_act_quant_blocked(const void *x, int x_dtype, const float *thresholds, const float *codebook,
-                                    void *x_hat_blocked, int64_t rows, int64_t cols, int bits, float eps, void *stream)
+static int act_quant_blocked_checked(const void *x, int x_dtype, const float *thresholds, const float *codebook,
+                                     void *x_hat_blocked, int64_t rows, int64_t cols, int bits, float eps, void *stream,
+                                     const WeightJob &wj)
 {
     if (!bits_ok(bits)) return fail(ARCQ_ERR_BITS, "arcq_act_quant_blocked: bits must be 2, 3, or 4");
     if (rows < 0 || cols < 0) return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked: bad sizes");
@@ -475,7 +500,7 @@ ARCQ_API int arcq_act_quant_blocked(const void *x, int x_dtype, const float *thr
     if (rows % 32 != 0) return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked: rows must be a multiple of 32");
     if (x_dtype != ARCQ_F32 && x_dtype != ARCQ_F16)
         return fail(ARCQ_ERR_DTYPE, "arcq_act_quant_blocked: x must be float32 or float16");
-    if (rows * cols == 0) return ARCQ_OK;
+    if (rows * cols == 0 && wj.blocks == 0) return ARCQ_OK;
     if (!x || !thresholds || !codebook || !x_hat_blocked)
         return fail(ARCQ_ERR_NULL, "arcq_act_quant_blocked: x, thresholds, codebook and x_hat_blocked must not be NULL");
     if (x_hat_blocked == x) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_act_quant_blocked: x_hat_blocked must not alias x");
@@ -483,8 +508,32 @@ ARCQ_API int arcq_act_quant_blocked(const void *x, int x_dtype, const float *thr
     if (!aligned(x, 16) || !aligned(x_hat_blocked, 16))
         return fail(ARCQ_ERR_ALIGN, "arcq_act_quant_blocked: x and x_hat_blocked must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (x_dtype == ARCQ_F32) return launch_blocked<float>(x, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, st);
-    return launch_blocked<__half>(x, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, st);
+    if (x_dtype == ARCQ_F32)
+        return launch_blocked<float>(x, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, st, wj);
+    return launch_blocked<__half>(x, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, st, wj);
+}
+
+ARCQ_API int arcq_act_quant_blocked(const void *x, int x_dtype, const float *thresholds, const float *codebook,
+                                    void *x_hat_blocked, int64_t rows, int64_t cols, int bits, float eps, void *stream)
+{
+    return act_quant_blocked_checked(x, x_dtype, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, stream,
+                                     WeightJob{});
+}
+
+// Stage 1 into the block layout and, in the same launch, w_hat[N, cols] (fp16, group size 64) from the layer's packed
+// weights: the two inputs of the copying GEMM variant.
+int arcq::act_quant_blocked_with_weights(const void *x, int x_dtype, const float *thresholds, const float *codebook,
+                                         void *x_hat_blocked, int64_t rows, int64_t cols, int bits, float eps,
+                                         const uint8_t *packed_w, const float *w_codebook, const float *w_center,
+                                         const float *w_scale, const float *w_code_sum, void *w_hat, int64_t N,
+                                         void *stream)
+{
+    if (rows <= 0 || cols <= 0 || N <= 0 || !packed_w || !w_codebook || !w_center || !w_scale || !w_code_sum || !w_hat ||
+        !aligned(w_hat, 16) || !aligned(packed_w, 4) || N * (cols / 8) >= (int64_t(1) << 38))
+        return fail(ARCQ_ERR_NULL, "arcq_linear_otf_ws: bad weight tensors");
+    WeightJob wj{packed_w, w_codebook, w_center, w_scale, w_code_sum, static_cast<__half *>(w_hat), N, cols,
+                 static_cast<unsigned>((N * (cols / 8) + 255) / 256)};
+    return act_quant_blocked_checked(x, x_dtype, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, stream, wj);
 }
 
 ARCQ_API int arcq_act_quant(const void *x, int x_dtype, const float *thresholds, const float *codebook,

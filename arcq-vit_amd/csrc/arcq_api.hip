@@ -66,10 +66,16 @@ static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds
     // Scratch-only workspaces and whole 32-row blocks: x_hat in the block layout, eight-wave weight-stationary GEMM
     // (bit-identical results; invalid arguments fall through to the entry points below, which report them).
     if (scratch_only && group_size == 64 && arcq::bits_ok(bits) && arcq::otf_blocked_pays(M, N, K) && x != x_hat_ws) {
-        const int rc = arcq_act_quant_blocked(x, x_dtype, a_thresholds, a_codebook, x_hat_ws, M, K, bits, 1.0e-6f, stream);
+        // With a weight workspace that pays, its reconstruction rides along in the stage-1 launch.
+        const bool carry = w_hat_ws && arcq::blocked_uses_workspace(N, K) && packed_w && w_codebook && w_center &&
+                           w_scale && w_code_sum && arcq::aligned(w_hat_ws, 16) && arcq::aligned(packed_w, 16);
+        const int rc = carry ? arcq::act_quant_blocked_with_weights(x, x_dtype, a_thresholds, a_codebook, x_hat_ws, M, K, bits,
+                                                                    1.0e-6f, packed_w, w_codebook, w_center, w_scale,
+                                                                    w_code_sum, w_hat_ws, N, stream)
+                             : arcq_act_quant_blocked(x, x_dtype, a_thresholds, a_codebook, x_hat_ws, M, K, bits, 1.0e-6f, stream);
         if (rc != ARCQ_OK) return rc;
-        return arcq_linear_fused_blocked(x_hat_ws, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, w_hat_ws, y,
-                                         y_dtype, M, N, K, bits, group_size, stream);
+        return arcq::linear_fused_blocked(x_hat_ws, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, w_hat_ws, carry,
+                                          y, y_dtype, M, N, K, bits, group_size, stream);
     }
     int rc = arcq_act_quant(x, x_dtype, a_thresholds, a_codebook, nullptr, nullptr, nullptr, nullptr, nullptr,
                             x_hat_ws, ARCQ_F16, M, K, bits, group_size, 1.0e-6f, stream);

@@ -30,6 +30,19 @@ void launch_gemm_slab8(const GemmArgs &g, const void *w_hat, hipStream_t stream)
 // Whether the whole-layer entry point with scratch-only workspaces runs stage 1 into the block layout and the
 // eight-wave kernel for this shape.
 bool otf_blocked_pays(int64_t M, int64_t N, int64_t K);
+// Whether the eight-wave kernel, given a weight workspace, copies weights reconstructed beforehand for this shape.
+bool blocked_uses_workspace(int64_t N, int64_t K);
+// arcq_linear_fused_blocked with the state of the workspace made explicit: w_hat_ready means w_hat_ws already holds
+// the reconstructed weights (and is to be used); otherwise they are rebuilt first where that pays.
+int linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_w, const float *w_codebook,
+                         const float *w_center, const float *w_scale, const float *w_code_sum, const float *bias,
+                         void *w_hat_ws, bool w_hat_ready, void *y, int y_dtype, int64_t M, int64_t N, int64_t K, int bits,
+                         int group_size, void *stream);
+// Stage 1 into the block layout and, in the same launch, w_hat[N, cols] (fp16) from the packed weights.
+int act_quant_blocked_with_weights(const void *x, int x_dtype, const float *thresholds, const float *codebook,
+                                   void *x_hat_blocked, int64_t rows, int64_t cols, int bits, float eps,
+                                   const uint8_t *packed_w, const float *w_codebook, const float *w_center,
+                                   const float *w_scale, const float *w_code_sum, void *w_hat, int64_t N, void *stream);
 
 // Small-M kernel (64 x 64 tiles, K split across the waves of a workgroup); requires K >= 64.
 void launch_gemm_splitk(const GemmArgs &g, hipStream_t stream);

@@ -375,11 +375,22 @@ ARCQ_API const char *arcq_linear_otf_ws_kernel(int64_t M, int64_t N, int64_t K, 
 
 // The fused GEMM on x_hat in the 32-row block layout (what arcq_act_quant_blocked writes): always the eight-wave
 // weight-stationary kernel; with a weight workspace, and a shape where that pays, on weights reconstructed once.
+bool arcq::blocked_uses_workspace(int64_t N, int64_t K) { return workspace_pays_blocked(N, K); }
+
 ARCQ_API int arcq_linear_fused_blocked(const void *x_hat_blocked,
                                        const uint8_t *packed_w, const float *w_codebook,
                                        const float *w_center, const float *w_scale, const float *w_code_sum,
                                        const float *bias, void *w_hat_ws, void *y, int y_dtype,
                                        int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
+{
+    return linear_fused_blocked(x_hat_blocked, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, w_hat_ws, false,
+                                y, y_dtype, M, N, K, bits, group_size, stream);
+}
+
+int arcq::linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_w, const float *w_codebook,
+                               const float *w_center, const float *w_scale, const float *w_code_sum, const float *bias,
+                               void *w_hat_ws, bool w_hat_ready, void *y, int y_dtype, int64_t M, int64_t N, int64_t K,
+                               int bits, int group_size, void *stream)
 {
     if (!bits_ok(bits)) return fail(ARCQ_ERR_BITS, "arcq_linear_fused_blocked: bits must be 2, 3, or 4");
     if (group_size != 64) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_fused_blocked: group_size must be 64 (got %d)", group_size);
@@ -397,8 +408,8 @@ ARCQ_API int arcq_linear_fused_blocked(const void *x_hat_blocked,
     if (!aligned(x_hat_blocked, 16) || !aligned(y, 16) || !aligned(packed_w, 16) || !aligned(w_hat_ws, 16))
         return fail(ARCQ_ERR_ALIGN, "arcq_linear_fused_blocked: x_hat_blocked, y, packed_w and w_hat_ws must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const bool prebuilt = w_hat_ws && workspace_pays_blocked(N, K);
-    if (prebuilt) {
+    const bool prebuilt = w_hat_ws && (w_hat_ready || workspace_pays_blocked(N, K));
+    if (prebuilt && !w_hat_ready) {
         const int rc = arcq_weight_dequant(packed_w, w_codebook, w_center, w_scale, w_code_sum, w_hat_ws, ARCQ_F16, N, K,
                                            bits, group_size, stream);
         if (rc != ARCQ_OK) return rc;

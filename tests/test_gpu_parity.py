@@ -447,9 +447,30 @@ def test_layer_otf_scratch_workspaces(cuda, oracle, monkeypatch, m):
         assert torch.equal(xs.view(m // 32, k // 8, 32, 8), _to_blocked(xw))
     ww = torch.zeros(n * k, dtype=torch.float16, device=cuda)
     assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float16, x_hat_ws=xs, w_hat_ws=ww), plain)
-    assert bool((ww != 0).any())
+    want_w = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, bits, 64, fma=True).astype(np.float16)
+    assert np.array_equal(_np(ww).view(np.uint16), want_w.reshape(-1).view(np.uint16))   # rebuilt in the stage-1 launch
     y32 = ops.linear_otf(x.float(), *args, out_dtype=torch.float32, scratch=True)   # fp32 in, fp32 out
     assert torch.allclose(y32, plain.float(), rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize("bits,in_dtype", [(3, torch.float32), (2, torch.float16)])
+def test_layer_otf_weights_rebuilt_in_stage1_launch(cuda, oracle, monkeypatch, bits, in_dtype):
+    """Whole layer in the block layout with a weight workspace (ragged N, seven groups, fp32 / fp16 input): the weights
+    rebuilt alongside stage 1 equal the oracle's and y equals the path without workspaces, bit for bit."""
+    m, n, k = 512, 200, 448
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL", raising=False)
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 59)
+    _, thr = _cb(bits)
+    bias = synth.make_bias(n, 59)
+    x = synth.make_activation(m, k, 59, "ln").to(in_dtype).to(cuda)
+    d = lambda t: t.to(cuda)
+    args = (d(thr), d(cb), d(packed), d(cb), d(center), d(scale), d(code_sum), d(bias), bits, 64)
+    plain = ops.linear_otf(x, *args, out_dtype=torch.float32)
+    ww = torch.full((n * k + 8,), -3.0, dtype=torch.float16, device=cuda)
+    assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float32, w_hat_ws=ww), plain)
+    want_w = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, bits, 64, fma=True).astype(np.float16)
+    assert np.array_equal(_np(ww)[:n * k].view(np.uint16), want_w.reshape(-1).view(np.uint16))
+    assert bool((ww[n * k:] == -3.0).all())
 
 
 @pytest.mark.parametrize("bits,out_dtype", [(4, torch.float16), (3, torch.float32), (2, torch.float32)])
