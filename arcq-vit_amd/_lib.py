@@ -38,7 +38,9 @@ _SIGNATURES = {
     "arcq_linear_otf_ws": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                            _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
     "arcq_act_quant_blocked": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32, _c_ptr],
-    "arcq_linear_fused_blocked": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
+    "arcq_act_quant_blocked_with_weights": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32,
+                                            _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr],
+    "arcq_linear_fused_blocked": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int,
                                   _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
     "arcq_linear_forward_packed": [_c_ptr] * 11 + [_c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_ptr],
     "arcq_linear_forward_u8": [_c_ptr] * 11 + [_c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],

@@ -522,15 +522,21 @@ ARCQ_API int arcq_act_quant_blocked(const void *x, int x_dtype, const float *thr
 
 // Stage 1 into the block layout and, in the same launch, w_hat[N, cols] (fp16, group size 64) from the layer's packed
 // weights: the two inputs of the copying GEMM variant.
-int arcq::act_quant_blocked_with_weights(const void *x, int x_dtype, const float *thresholds, const float *codebook,
-                                         void *x_hat_blocked, int64_t rows, int64_t cols, int bits, float eps,
-                                         const uint8_t *packed_w, const float *w_codebook, const float *w_center,
-                                         const float *w_scale, const float *w_code_sum, void *w_hat, int64_t N,
-                                         void *stream)
+ARCQ_API int arcq_act_quant_blocked_with_weights(const void *x, int x_dtype, const float *thresholds,
+                                                 const float *codebook, void *x_hat_blocked, int64_t rows, int64_t cols,
+                                                 int bits, float eps, const uint8_t *packed_w, const float *w_codebook,
+                                                 const float *w_center, const float *w_scale, const float *w_code_sum,
+                                                 void *w_hat, int64_t N, void *stream)
 {
-    if (rows <= 0 || cols <= 0 || N <= 0 || !packed_w || !w_codebook || !w_center || !w_scale || !w_code_sum || !w_hat ||
-        !aligned(w_hat, 16) || !aligned(packed_w, 4) || N * (cols / 8) >= (int64_t(1) << 38))
-        return fail(ARCQ_ERR_NULL, "arcq_linear_otf_ws: bad weight tensors");
+    if (N < 0) return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked_with_weights: bad sizes");
+    if (N == 0 || cols <= 0 || cols % 64 != 0)      // no weights to rebuild (or sizes the plain entry point reports)
+        return arcq_act_quant_blocked(x, x_dtype, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, stream);
+    if (!packed_w || !w_codebook || !w_center || !w_scale || !w_code_sum || !w_hat)
+        return fail(ARCQ_ERR_NULL, "arcq_act_quant_blocked_with_weights: NULL weight tensor pointer");
+    if (!aligned(w_hat, 16) || !aligned(packed_w, 4))
+        return fail(ARCQ_ERR_ALIGN, "arcq_act_quant_blocked_with_weights: w_hat must be 16-byte, packed_w 4-byte aligned");
+    if (N * (cols / 8) >= (int64_t(1) << 38))
+        return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked_with_weights: weight tensor too large");
     WeightJob wj{packed_w, w_codebook, w_center, w_scale, w_code_sum, static_cast<__half *>(w_hat), N, cols,
                  static_cast<unsigned>((N * (cols / 8) + 255) / 256)};
     return act_quant_blocked_checked(x, x_dtype, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, stream, wj);

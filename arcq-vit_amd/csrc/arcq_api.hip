@@ -69,7 +69,7 @@ static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds
         // With a weight workspace that pays, its reconstruction rides along in the stage-1 launch.
         const bool carry = w_hat_ws && arcq::blocked_uses_workspace(N, K) && packed_w && w_codebook && w_center &&
                            w_scale && w_code_sum && arcq::aligned(w_hat_ws, 16) && arcq::aligned(packed_w, 16);
-        const int rc = carry ? arcq::act_quant_blocked_with_weights(x, x_dtype, a_thresholds, a_codebook, x_hat_ws, M, K, bits,
+        const int rc = carry ? arcq_act_quant_blocked_with_weights(x, x_dtype, a_thresholds, a_codebook, x_hat_ws, M, K, bits,
                                                                     1.0e-6f, packed_w, w_codebook, w_center, w_scale,
                                                                     w_code_sum, w_hat_ws, N, stream)
                              : arcq_act_quant_blocked(x, x_dtype, a_thresholds, a_codebook, x_hat_ws, M, K, bits, 1.0e-6f, stream);

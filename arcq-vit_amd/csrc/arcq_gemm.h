@@ -38,11 +38,7 @@ int linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_w, con
                          const float *w_center, const float *w_scale, const float *w_code_sum, const float *bias,
                          void *w_hat_ws, bool w_hat_ready, void *y, int y_dtype, int64_t M, int64_t N, int64_t K, int bits,
                          int group_size, void *stream);
-// Stage 1 into the block layout and, in the same launch, w_hat[N, cols] (fp16) from the packed weights.
-int act_quant_blocked_with_weights(const void *x, int x_dtype, const float *thresholds, const float *codebook,
-                                   void *x_hat_blocked, int64_t rows, int64_t cols, int bits, float eps,
-                                   const uint8_t *packed_w, const float *w_codebook, const float *w_center,
-                                   const float *w_scale, const float *w_code_sum, void *w_hat, int64_t N, void *stream);
+
 
 // Small-M kernel (64 x 64 tiles, K split across the waves of a workgroup); requires K >= 64.
 void launch_gemm_splitk(const GemmArgs &g, hipStream_t stream);

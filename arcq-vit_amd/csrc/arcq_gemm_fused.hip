@@ -368,23 +368,35 @@ bool arcq::otf_blocked_pays(int64_t M, int64_t N, int64_t K)
 ARCQ_API const char *arcq_linear_otf_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace)
 {
     if (otf_blocked_pays(M, N, K))
-        return (have_workspace && workspace_pays_blocked(N, K)) ? "weight_dequant8_kernel+gemm_slab8_kernel"
-                                                                   : "gemm_slab8_kernel";
+        return (have_workspace && blocked_uses_workspace(N, K)) ? "gemm_slab8_kernel<copy>" : "gemm_slab8_kernel";
     return arcq_linear_fused_ws_kernel(M, N, K, have_workspace);
 }
 
 // The fused GEMM on x_hat in the 32-row block layout (what arcq_act_quant_blocked writes): always the eight-wave
 // weight-stationary kernel; with a weight workspace, and a shape where that pays, on weights reconstructed once.
-bool arcq::blocked_uses_workspace(int64_t N, int64_t K) { return workspace_pays_blocked(N, K); }
+// In the whole-layer entry point the reconstruction costs no launch of its own (it rides in the stage-1 launch), and
+// copying is then never slower than rebuilding inside the GEMM: for shapes whose K spans several slab slices it is
+// the large win measured above, for the others what the GEMM gains (a 1 us copy instead of a 3.6 us rebuild) the
+// stage-1 launch pays (whole steps of DeiT-S / DeiT-B / ViT-L: 0.5 % / 0.3 % / 0.0 % faster than copying by the
+// stand-alone rule).  "slab8" pins the in-kernel rebuild, "prebuilt" the copy.
+bool arcq::blocked_uses_workspace(int64_t N, int64_t K)
+{
+    if (N <= 0 || K < 64 || K % 64 != 0) return false;
+    const char *e = getenv("ARCQ_GEMM_KERNEL");
+    if (e) return !strcmp(e, "prebuilt");
+    return true;
+}
 
 ARCQ_API int arcq_linear_fused_blocked(const void *x_hat_blocked,
                                        const uint8_t *packed_w, const float *w_codebook,
                                        const float *w_center, const float *w_scale, const float *w_code_sum,
-                                       const float *bias, void *w_hat_ws, void *y, int y_dtype,
+                                       const float *bias, void *w_hat_ws, int w_hat_ready, void *y, int y_dtype,
                                        int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
 {
-    return linear_fused_blocked(x_hat_blocked, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, w_hat_ws, false,
-                                y, y_dtype, M, N, K, bits, group_size, stream);
+    if (w_hat_ready && !w_hat_ws)
+        return fail(ARCQ_ERR_NULL, "arcq_linear_fused_blocked: w_hat_ready needs w_hat_ws");
+    return linear_fused_blocked(x_hat_blocked, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, w_hat_ws,
+                                w_hat_ready != 0, y, y_dtype, M, N, K, bits, group_size, stream);
 }
 
 int arcq::linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_w, const float *w_codebook,

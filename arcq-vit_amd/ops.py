@@ -304,9 +304,13 @@ def linear_otf(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Te
 
 
 def quantize_activation_blocked(x: torch.Tensor, thresholds: torch.Tensor, codebook: torch.Tensor, bits: int,
-                                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                                out: Optional[torch.Tensor] = None, weights=None,
+                                w_hat: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Stage 1 (group size 64) with ``x_hat`` written as fp16 in the 32-row block layout
-    ``[M/32, K/8, 32, 8]`` that ``linear_fused_blocked`` reads; same values as ``dequant_activation_hip``."""
+    ``[M/32, K/8, 32, 8]`` that ``linear_fused_blocked`` reads; same values as ``dequant_activation_hip``.
+
+    ``weights=(packed_w, w_codebook, w_center, w_scale, w_code_sum)`` with ``w_hat`` (fp16, N*K elements): the same
+    launch also reconstructs the layer's weights into ``w_hat`` (what ``unpack_weight_hip`` would write)."""
     _check(x.is_cuda and x.dim() == 2, "x must be a CUDA tensor [M, K]")
     _check_bits(bits)
     x = x.contiguous()
@@ -317,18 +321,31 @@ def quantize_activation_blocked(x: torch.Tensor, thresholds: torch.Tensor, codeb
     else:
         _check(out.is_cuda and out.dtype == torch.float16 and out.is_contiguous() and out.numel() >= m * k,
                "out must be a contiguous float16 CUDA buffer of at least M*K elements")
+    thr, cbk = _f32c(thresholds), _f32c(codebook)
     with torch.cuda.device(x.device):
-        _lib.check(_lib.load().arcq_act_quant_blocked(
-            _ptr(x), _dtype_code(x, "x"), _ptr(_f32c(thresholds)), _ptr(_f32c(codebook)), _ptr(out), m, k, bits, 1.0e-6,
-            _stream()))
+        if weights is None:
+            _lib.check(_lib.load().arcq_act_quant_blocked(
+                _ptr(x), _dtype_code(x, "x"), _ptr(thr), _ptr(cbk), _ptr(out), m, k, bits, 1.0e-6, _stream()))
+        else:
+            packed_w = weights[0].contiguous()
+            n = packed_w.shape[0]
+            _check(packed_w.is_cuda and packed_w.dtype == torch.uint8 and packed_w.dim() == 2
+                   and packed_w.shape[1] == (k * bits + 7) // 8, "packed_w must be uint8 [N, K*bits/8]")
+            _check(w_hat is not None, "weights need a w_hat buffer")
+            _check_w_ws(w_hat, n, k)
+            meta = [_f32c(t) for t in weights[1:]]
+            _lib.check(_lib.load().arcq_act_quant_blocked_with_weights(
+                _ptr(x), _dtype_code(x, "x"), _ptr(thr), _ptr(cbk), _ptr(out), m, k, bits, 1.0e-6,
+                _ptr(packed_w), *[_ptr(t) for t in meta], _ptr(w_hat), n, _stream()))
     return out
 
 
 def linear_fused_blocked(x_hat_blocked: torch.Tensor, m: int, k: int, packed_w: torch.Tensor, w_codebook: torch.Tensor,
                          w_center: torch.Tensor, w_scale: torch.Tensor, w_code_sum: torch.Tensor,
                          bias: Optional[torch.Tensor], bits: int, out_dtype: torch.dtype = torch.float16,
-                         w_hat_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``linear_fused`` on ``x_hat`` ``[m, k]`` held in the 32-row block layout (``quantize_activation_blocked``)."""
+                         w_hat_ws: Optional[torch.Tensor] = None, w_hat_ready: bool = False) -> torch.Tensor:
+    """``linear_fused`` on ``x_hat`` ``[m, k]`` held in the 32-row block layout (``quantize_activation_blocked``).
+    ``w_hat_ready``: ``w_hat_ws`` already holds the reconstructed fp16 weights and is used as is."""
     _check(x_hat_blocked.is_cuda and x_hat_blocked.dtype == torch.float16 and x_hat_blocked.is_contiguous()
            and x_hat_blocked.numel() >= m * k, "x_hat_blocked must be a contiguous float16 CUDA buffer of M*K elements")
     _check(packed_w.is_cuda and packed_w.dtype == torch.uint8 and packed_w.dim() == 2, "packed_w must be uint8 [N, K*bits/8]")
@@ -341,8 +358,8 @@ def linear_fused_blocked(x_hat_blocked: torch.Tensor, m: int, k: int, packed_w: 
     _check_w_ws(w_hat_ws, n, k)
     with torch.cuda.device(x_hat_blocked.device):
         _lib.check(_lib.load().arcq_linear_fused_blocked(
-            _ptr(x_hat_blocked), *[_ptr(t) for t in w], _ptr(b), _ptr(w_hat_ws), _ptr(y), _dtype_code(y, "y"),
-            m, n, k, bits, 64, _stream()))
+            _ptr(x_hat_blocked), *[_ptr(t) for t in w], _ptr(b), _ptr(w_hat_ws), int(bool(w_hat_ready)), _ptr(y),
+            _dtype_code(y, "y"), m, n, k, bits, 64, _stream()))
     return y
 
 

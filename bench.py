@@ -31,8 +31,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch of each fused-GEMM kernel at the default workload (average over the layer shapes it serves),
 # from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a plain 256 MiB
 # copy (factors 2.00 and 1.00).  Summary: profiles/deit_small_w4a4_bs64_packed_linears.md.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): {"gemm_slab8_kernel": 39.8e6,
-                                                         "weight_dequant8_kernel+gemm_slab8_kernel": 63.2e6}}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): {"gemm_slab8_kernel<copy>": None}}
 
 
 def parse_args():
@@ -97,23 +96,36 @@ class Layer:
                 self.scale.data_ptr(), self.code_sum.data_ptr(), self.bias.data_ptr(), Layer.W_WS.data_ptr(),
                 y.data_ptr(), ARCQ_F16, m, self.n, self.k, self.bits, 64, stream)
 
-    # The two halves of arcq_linear_otf_ws on their own: for shapes it runs in the 32-row block layout the halves are
-    # arcq_act_quant_blocked / arcq_linear_fused_blocked, else arcq_act_quant / arcq_linear_fused_ws.
-    def blocked(self, lib, m):
-        return b"slab8" in lib.arcq_linear_otf_ws_kernel(m, self.n, self.k, 1)
+    # The two halves of arcq_linear_otf_ws on their own.  Block-layout shapes: arcq_act_quant_blocked_with_weights
+    # (stage 1 plus the weight reconstruction carried in the same launch) and arcq_linear_fused_blocked on weights
+    # that are ready; other shapes: arcq_act_quant and arcq_linear_fused_ws.
+    def mode(self, lib, m):
+        name = lib.arcq_linear_otf_ws_kernel(m, self.n, self.k, 1)
+        return "copy" if name == b"gemm_slab8_kernel<copy>" else "blocked" if b"slab8" in name else "rowmajor"
 
     def call_act(self, lib, x, ws, stream):
         from arcq_vit_amd._lib import ARCQ_F16
-        if self.blocked(lib, x.shape[0]):
+        mode = self.mode(lib, x.shape[0])
+        if mode == "copy":
+            return lib.arcq_act_quant_blocked_with_weights(
+                x.data_ptr(), ARCQ_F16, self.thr.data_ptr(), self.cb.data_ptr(), ws.data_ptr(), x.shape[0], self.k,
+                self.bits, 1.0e-6, self.packed.data_ptr(), self.cb.data_ptr(), self.center.data_ptr(),
+                self.scale.data_ptr(), self.code_sum.data_ptr(), Layer.W_WS.data_ptr(), self.n, stream)
+        if mode == "blocked":
             return lib.arcq_act_quant_blocked(x.data_ptr(), ARCQ_F16, self.thr.data_ptr(), self.cb.data_ptr(),
                                               ws.data_ptr(), x.shape[0], self.k, self.bits, 1.0e-6, stream)
         return lib.arcq_act_quant(*self.act_args(x, ws, stream))
 
     def call_gemm(self, lib, ws, y, m, stream):
-        if self.blocked(lib, m):
-            a = self.gemm_args(ws, y, m, stream)
-            return lib.arcq_linear_fused_blocked(*a)
-        return lib.arcq_linear_fused_ws(*self.gemm_args(ws, y, m, stream))
+        from arcq_vit_amd._lib import ARCQ_F16
+        mode = self.mode(lib, m)
+        if mode == "rowmajor":
+            return lib.arcq_linear_fused_ws(*self.gemm_args(ws, y, m, stream))
+        # "copy": W_WS holds some layer's reconstructed weights of at least this size (timing does not depend on which)
+        return lib.arcq_linear_fused_blocked(
+            ws.data_ptr(), self.packed.data_ptr(), self.cb.data_ptr(), self.center.data_ptr(), self.scale.data_ptr(),
+            self.code_sum.data_ptr(), self.bias.data_ptr(), Layer.W_WS.data_ptr() if mode == "copy" else 0,
+            1 if mode == "copy" else 0, y.data_ptr(), ARCQ_F16, m, self.n, self.k, self.bits, 64, stream)
 
     def act_args(self, x, ws, stream):
         from arcq_vit_amd._lib import ARCQ_F16

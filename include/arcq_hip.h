@@ -164,15 +164,25 @@ const char *arcq_linear_fused_ws_kernel(int64_t M, int64_t N, int64_t K, int hav
  * row-major tensor, bit for bit.  group_size is 64; M * K must stay below 2^31. */
 int arcq_act_quant_blocked(const void *x, int x_dtype, const float *thresholds, const float *codebook,
                            void *x_hat_blocked, int64_t rows, int64_t cols, int bits, float eps, void *stream);
+/* The same launch also reconstructs w_hat[N, cols] (fp16, what arcq_weight_dequant writes) from the layer's packed
+ * weights, in extra workgroups: the two inputs of arcq_linear_fused_blocked(..., w_hat_ready = 1) for one launch. */
+int arcq_act_quant_blocked_with_weights(const void *x, int x_dtype, const float *thresholds, const float *codebook,
+                                        void *x_hat_blocked, int64_t rows, int64_t cols, int bits, float eps,
+                                        const uint8_t *packed_w, const float *w_codebook, const float *w_center,
+                                        const float *w_scale, const float *w_code_sum, void *w_hat, int64_t N,
+                                        void *stream);
+/* w_hat_ws: NULL, or a fp16 [N,K] buffer.  w_hat_ready != 0: it already holds the reconstructed weights (from
+ * arcq_weight_dequant, arcq_act_quant_blocked_with_weights or an earlier call with the same weights) and the kernel
+ * copies from it; w_hat_ready == 0: scratch, filled first for the shapes where that pays. */
 int arcq_linear_fused_blocked(const void *x_hat_blocked,
                               const uint8_t *packed_w, const float *w_codebook,
                               const float *w_center, const float *w_scale, const float *w_code_sum,
-                              const float *bias, void *w_hat_ws, void *y, int y_dtype,
+                              const float *bias, void *w_hat_ws, int w_hat_ready, void *y, int y_dtype,
                               int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
 
-/* Kernels arcq_linear_otf_ws runs after stage 1 for these sizes: "gemm_slab8_kernel" or
- * "weight_dequant8_kernel+gemm_slab8_kernel" when it takes the block layout, else arcq_linear_fused_ws_kernel's
- * answer.  A profiling aid with no counterpart in the reference. */
+/* Kernels arcq_linear_otf_ws runs after stage 1 for these sizes: "gemm_slab8_kernel", or "gemm_slab8_kernel<copy>"
+ * (weights rebuilt in the stage-1 launch, copied by the GEMM), when it takes the block layout, else
+ * arcq_linear_fused_ws_kernel's answer.  A profiling aid with no counterpart in the reference. */
 const char *arcq_linear_otf_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace);
 
 /* ---- index-space linears (no reconstruction, product-table gather) ---------

@@ -421,6 +421,14 @@ def test_fused_gemm_block_layout(cuda, oracle, monkeypatch, bits, out_dtype, m, 
     assert np.array_equal(_np(ws)[:n * k].view(np.uint16), want_w.reshape(-1).view(np.uint16))
     assert bool((ws[n * k:] == -3.0).all())
     assert torch.equal(ops.linear_fused_blocked(xb, m, k, *w, bias, bits, out_dtype=out_dtype, w_hat_ws=ws), y)   # library's choice
+    # stage 1 with the weight reconstruction carried in its launch, then the GEMM on weights that are ready
+    ws2 = torch.full((n * k + 8,), -3.0, dtype=torch.float16, device=cuda)
+    xb2 = ops.quantize_activation_blocked(x.to(cuda), thr.to(cuda), cb.to(cuda), bits, weights=w, w_hat=ws2)
+    assert torch.equal(xb2, xb)
+    assert np.array_equal(_np(ws2)[:n * k].view(np.uint16), want_w.reshape(-1).view(np.uint16))
+    assert bool((ws2[n * k:] == -3.0).all())
+    assert torch.equal(ops.linear_fused_blocked(xb2, m, k, *w, bias, bits, out_dtype=out_dtype, w_hat_ws=ws2,
+                                                w_hat_ready=True), y)
     nb = ops.linear_fused_blocked(xb, m, k, *w, None, bits, out_dtype=torch.float32)
     yb = ops.linear_fused_blocked(xb, m, k, *w, bias, bits, out_dtype=torch.float32)
     assert torch.equal(nb + bias, yb)            # the bias is one fp32 addition before the output rounding

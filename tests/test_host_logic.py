@@ -351,13 +351,14 @@ def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
     assert lib.arcq_linear_fused_ws_kernel(12608, 1152, 384, 0) == b"gemm_stream_kernel"
     # The whole-layer entry point with scratch workspaces: whole 32-row blocks from 512 rows on take the block layout.
     monkeypatch.delenv("ARCQ_GEMM_KERNEL")
-    both8 = b"weight_dequant8_kernel+gemm_slab8_kernel"
-    assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 1) == b"gemm_slab8_kernel"
+    both8 = b"gemm_slab8_kernel<copy>"
+    assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 1) == both8                     # the rebuild rides in stage 1
+    assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 0) == b"gemm_slab8_kernel"
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 1) == both8
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 0) == b"gemm_slab8_kernel"
     assert lib.arcq_linear_otf_ws_kernel(12608, 768, 768, 1) == both8                      # two slices, six slabs
     assert lib.arcq_linear_otf_ws_kernel(50432, 4096, 1024, 1) == both8                    # three slices
-    assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 1) == b"gemm_slab8_kernel"      # two slices, 18 slabs
+    assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 1) == both8
     assert lib.arcq_linear_otf_ws_kernel(1576, 384, 1536, 1) == both                       # 1576 % 32 != 0: row-major
     assert lib.arcq_linear_otf_ws_kernel(197, 1152, 384, 1) == b"gemm_splitk_kernel"
     monkeypatch.setenv("ARCQ_GEMM_KERNEL", "stream")
@@ -378,9 +379,14 @@ def test_block_layout_entry_points_validate_before_launching():
     assert lib.arcq_act_quant_blocked(p, F16, p, p, None, 32, 64, 4, 1e-6, None) == -3         # NULL output
     assert lib.arcq_act_quant_blocked(p, F16, p, p, p, 32, 64, 4, 1e-6, None) == -6            # in place is not possible
     assert lib.arcq_act_quant_blocked(p, F16, p, p, p + 64, 0, 64, 4, 1e-6, None) == 0         # empty
-    args = lambda m, n, k, bits=4, gs=64: (p, p, p, p, p, p, None, None, p + 64, F16, m, n, k, bits, gs, None)
+    args = lambda m, n, k, bits=4, gs=64, ready=0: (p, p, p, p, p, p, None, None, ready, p + 64, F16, m, n, k, bits, gs, None)
     assert lib.arcq_linear_fused_blocked(*args(33, 8, 64)) == -4
     assert lib.arcq_linear_fused_blocked(*args(32, 8, 96)) == -2
     assert lib.arcq_linear_fused_blocked(*args(32, 8, 64, gs=32)) == -6
     assert lib.arcq_linear_fused_blocked(*args(32, 8, 64, bits=1)) == -1
     assert lib.arcq_linear_fused_blocked(*args(0, 8, 64)) == 0
+    assert lib.arcq_linear_fused_blocked(*args(32, 8, 64, ready=1)) == -3                      # ready without a buffer
+    wargs = lambda n, w_hat=p + 128: (p, F16, p, p, p + 64, 32, 64, 4, 1e-6, p, p, p, p, p, w_hat, n, None)
+    assert lib.arcq_act_quant_blocked_with_weights(*wargs(8, None)) == -3
+    assert lib.arcq_act_quant_blocked_with_weights(*wargs(8, p + 130)) == -7
+    assert lib.arcq_act_quant_blocked_with_weights(*wargs(-1)) == -4
