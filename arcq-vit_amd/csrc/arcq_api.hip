@@ -47,12 +47,12 @@ static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds
         return arcq::fail(ARCQ_ERR_DTYPE, "arcq_linear_otf: x_hat_ws may alias x only when x is fp16");
     // A few hundred rows: one launch for the whole layer (same results bit for bit).  Taken only when every argument
     // is plainly valid; anything else goes through the two entry points below, which report what is wrong.
-    // ARCQ_OTF_FUSED=0 switches the single-launch path off (tuning aid).
+    // ARCQ_OTF_FUSED=0 switches the single-launch path off, =2 takes it for every shape the kernel can run (tuning aids).
     {
         const char *e = getenv("ARCQ_OTF_FUSED");
         const bool enabled = !(e && e[0] == '0');
         if (enabled && group_size == 64 && arcq::bits_ok(bits) && M > 0 && N > 0 && N < (int64_t(1) << 30) &&
-            arcq::otf_small_supported(M, K) && x && x != x_hat_ws && a_thresholds && a_codebook && packed_w &&
+            arcq::otf_small_supported(M, N, K, e && e[0] == '2') && x && x != x_hat_ws && a_thresholds && a_codebook && packed_w &&
             w_codebook && w_center && w_scale && w_code_sum && y && (x_dtype == ARCQ_F16 || x_dtype == ARCQ_F32) &&
             (y_dtype == ARCQ_F16 || y_dtype == ARCQ_F32) && arcq::aligned(x, 16) && arcq::aligned(x_hat_ws, 16) &&
             arcq::aligned(y, 16) && arcq::aligned(packed_w, 16)) {

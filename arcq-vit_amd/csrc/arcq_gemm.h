@@ -56,7 +56,7 @@ struct OtfSmallArgs {
     int M, N, K, bits;
     float eps;
 };
-bool otf_small_supported(int64_t M, int64_t K);
+bool otf_small_supported(int64_t M, int64_t N, int64_t K, bool any_supported);
 void launch_otf_small(const OtfSmallArgs &a, hipStream_t stream);
 
 }  // namespace arcq

@@ -97,15 +97,18 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
                  const uint8_t *__restrict__ pw, const float *__restrict__ w_cb,
                  const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
                  const float *__restrict__ bias, __half *__restrict__ x_hat_ws, TOUT *__restrict__ y,
-                 int M, int N, int K, float eps, int tile_bytes)
+                 int M, int N, int K, float eps, int tile_bytes, int partial_off)
 {
     constexpr int L = 1 << BITS;
     constexpr int RT = 32 * RB;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    // [x_hat tile] [partial tiles] [activation LUT] [weight LUT] [buckets] [per-wave flags]
+    // [x_hat tile | partial tiles] [activation LUT] [weight LUT] [buckets] [per-wave flags]; the partial tiles of
+    // the reduction follow the x_hat tile (partial_off == tile_bytes) or, when K is too long for both, reuse its space
+    // (partial_off == 0) after a barrier.
     unsigned char *xt = smem;
-    unsigned char *partial = smem + tile_bytes;
-    float *a_lut = reinterpret_cast<float *>(partial + kOsWaves * RT * kOsRedPitch);
+    unsigned char *partial = smem + partial_off;
+    const int front = max(tile_bytes, partial_off + kOsWaves * RT * kOsRedPitch);
+    float *a_lut = reinterpret_cast<float *>(smem + front);
     float *w_lut = a_lut + L * 64;
     Bucket *table = reinterpret_cast<Bucket *>(w_lut + L * 64);
     int *slow_slots = reinterpret_cast<int *>(table + kMaxBuckets + 64);
@@ -153,15 +156,18 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
         const int row = f / G, g = f - row * G;
         os_fetch_group<TIN>(x + static_cast<int64_t>(min(m0 + row, M - 1)) * K + g * 64, f < groups && m0 + row < M, in);
     };
-    // Waves 0 .. tile_waves-1 own one 64-group tile each (32 rows x K <= 512 is at most four tiles); the other
-    // waves build the lookup tables meanwhile.  One barrier joins the two halves.
-    const int tile_waves = (groups + 63) / 64;
-    const bool has_tile = wave < tile_waves;
+    // Wave w owns the 64-group tiles w, w + 8, ... of the row tile.  With fewer than eight tiles (K <= 448 for 32
+    // rows) the waves without one build the lookup tables while the others take their statistics, and one barrier
+    // joins the two halves; otherwise all eight waves build the tables between the two halves of their first tile.
+    const int n_tiles = (groups + 63) / 64;
+    const bool spare_waves = n_tiles < kOsWaves;
+    const int tile_waves = spare_waves ? n_tiles : kOsWaves;
+    const bool has_tile = wave < n_tiles;
     if (has_tile) fetch_x(wave * 64);
     float th[L - 1], cbv[L];
     load_quant_params<BITS>(a_thr, a_cb, th, cbv);
     const BucketScale bq = pick_bucket_scale<BITS>(th);
-    if (!has_tile)
+    if (spare_waves && !has_tile)
         build_quant_tables_by<BITS>(th, cbv, bq, a_lut, table, slow_slots, tid - tile_waves * 64, (kOsWaves - tile_waves) * 64);
     if (wave == kOsWaves - 1) {
 #pragma unroll
@@ -171,14 +177,21 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     float mu = 0.0f, var = 0.0f, s = 0.0f;
     if (has_tile) {
         os_convert_group<TIN>(in, xv);
+        if (wave + kOsWaves < n_tiles) fetch_x((wave + kOsWaves) * 64);      // the next tile's inputs, one round ahead
         group_stats64(xv, eps, mu, var, s);
     }
+    if (!spare_waves) build_quant_tables_by<BITS>(th, cbv, bq, a_lut, table, slow_slots, tid, kOsWaves * 64);
     __syncthreads();
     const bool write_ws = (x_hat_ws != nullptr) && blockIdx.x == 0;
-    if (has_tile) {
-        bool table_ok = true;
-        for (int w = tile_waves; w < kOsWaves; ++w) table_ok = table_ok && (slow_slots[w - tile_waves] == 0);
-        const int f = wave * 64 + lane;
+    bool table_ok = true;
+    for (int w = 0; w < (spare_waves ? kOsWaves - tile_waves : kOsWaves); ++w) table_ok = table_ok && (slow_slots[w] == 0);
+    for (int t = wave; t < n_tiles; t += kOsWaves) {
+        if (t != wave) {                       // later tiles of this wave: their inputs were requested a round ago
+            os_convert_group<TIN>(in, xv);
+            if (t + kOsWaves < n_tiles) fetch_x((t + kOsWaves) * 64);
+            group_stats64(xv, eps, mu, var, s);
+        }
+        const int f = t * 64 + lane;
         const int row = f / G, g = f - row * G;
         const bool valid = f < groups && m0 + row < M;
         float sum_codes;
@@ -255,6 +268,7 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
         }
     }
     // ---- reduction over the waves in a fixed order, bias, output -------------------------------------------
+    if (partial_off < tile_bytes) __syncthreads();      // the partial tiles reuse the x_hat tile: every wave is done reading it
     unsigned char *mine = partial + wave * (RT * kOsRedPitch);
 #pragma unroll
     for (int i = 0; i < RB; ++i)
@@ -315,7 +329,10 @@ static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
     const int xhat_bytes = RT * os_row_pitch(G);
     const int partial_bytes = kOsWaves * RT * kOsRedPitch;
     const int tile_bytes = xhat_bytes;
-    const size_t smem = tile_bytes + partial_bytes + 2 * L * 64 * sizeof(float) + (kMaxBuckets + 64) * sizeof(Bucket) + 64;
+    const size_t tables = 2 * L * 64 * sizeof(float) + (kMaxBuckets + 64) * sizeof(Bucket) + 64;
+    // Both regions side by side while they fit 160 KB of LDS; else the partial tiles reuse the x_hat tile's space.
+    const int partial_off = (tile_bytes + partial_bytes + tables <= 160 * 1024) ? tile_bytes : 0;
+    const size_t smem = (partial_off ? tile_bytes + partial_bytes : (tile_bytes > partial_bytes ? tile_bytes : partial_bytes)) + tables;
     auto kernel = otf_small_kernel<TIN, BITS, TOUT, RB>;
     static int configured = 0;        // per instantiation: largest dynamic LDS size requested so far
     if (static_cast<int>(smem) > configured) {
@@ -326,7 +343,7 @@ static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
     const dim3 grid((a.N + kOsCols - 1) / kOsCols, (a.M + RT - 1) / RT);
     hipLaunchKernelGGL(kernel, grid, dim3(kOsWaves * 64), smem, stream, static_cast<const TIN *>(a.x), a.a_thr, a.a_cb,
                        a.pw, a.w_cb, a.wc, a.ws, a.wcs, a.bias, static_cast<__half *>(a.x_hat_ws),
-                       static_cast<TOUT *>(a.y), a.M, a.N, a.K, a.eps, tile_bytes);
+                       static_cast<TOUT *>(a.y), a.M, a.N, a.K, a.eps, tile_bytes, partial_off);
 }
 
 template <typename TIN, int BITS, typename TOUT>
@@ -343,11 +360,16 @@ static void launch_os_bits(const OtfSmallArgs &a, hipStream_t stream)
     else launch_os_rb<TIN, 2, TOUT>(a, stream);
 }
 
-// One launch pays off while the activation quantizer of a 32-row tile is at most one 64-group tile per SIMD
-// (K <= 512): every column tile repeats that work, and beyond it the repeated work is longer than a second launch.
-bool otf_small_supported(int64_t M, int64_t K)
+// Every column tile repeats the activation quantizer of its 32 rows (K / 64 groups each, one 64-group tile per wave
+// and round).  Measured at 197 rows: one launch wins while that is a single round and the grid fits the chip in one
+// wave of workgroups (K = 384: 10.6 us against 12.6; K = 768, N = 2304: 13.8 against 15.5) and loses beyond (K = 768,
+// N = 3072, 336 workgroups: 23.4 against 17.3; K = 1536, three rounds: 23.7 against 19.7).  `any_supported` is what
+// the kernel can run at all (the x_hat tile of 32 rows must fit LDS): ARCQ_OTF_FUSED=2 asks for that.
+bool otf_small_supported(int64_t M, int64_t N, int64_t K, bool any_supported)
 {
-    return M < 512 && K >= 64 && K % 64 == 0 && K <= 512;
+    if (!(M < 512 && K >= 64 && K % 64 == 0 && K <= 1536)) return false;
+    if (any_supported || K <= 512) return true;
+    return K <= 768 && ((N + kOsCols - 1) / kOsCols) * ((M + 31) / 32) <= 256;
 }
 
 void launch_otf_small(const OtfSmallArgs &a, hipStream_t stream)

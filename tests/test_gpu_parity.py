@@ -525,11 +525,16 @@ def test_layer_otf_matches_stagewise(cuda, oracle, bits):
 
 @pytest.mark.parametrize("bits,x_dtype,out_dtype", [(4, torch.float16, torch.float16), (3, torch.float32, torch.float32),
                                                     (2, torch.float16, torch.float32), (4, torch.float32, torch.float16)])
-@pytest.mark.parametrize("m,n,k", [(197, 1152, 384), (197, 384, 1536), (1, 70, 64), (65, 130, 1088), (500, 64, 2048),
-                                   (33, 200, 2112)])
+@pytest.mark.parametrize("m,n,k", [(197, 1152, 384), (1, 70, 64),
+                                   (197, 768, 768),       # six 64-group tiles per row tile: two waves build the tables
+                                   (100, 96, 1024),       # eight tiles: every wave has one, all build the tables
+                                   (65, 130, 1088),       # nine tiles, and the partial tiles reuse the x_hat tile's LDS
+                                   (197, 384, 1536), (500, 384, 1536),      # twelve tiles: two rounds for four waves
+                                   (500, 64, 2048), (33, 200, 2112)])       # beyond the single launch: two launches
 def test_layer_otf_single_launch(cuda, oracle, monkeypatch, bits, x_dtype, out_dtype, m, n, k):
-    """Below 512 rows arcq_linear_otf runs the whole layer in one launch (when K fits LDS); it must equal the
-    two-launch path bit for bit, in y and in the x_hat workspace, and x_hat must equal the oracle's."""
+    """Below 512 rows arcq_linear_otf can run the whole layer in one launch (ARCQ_OTF_FUSED=2: whenever K fits LDS; =1,
+    the default: where that is faster; =0: never); all three must agree bit for bit, in y and in the x_hat workspace,
+    and x_hat must equal the oracle's."""
     cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 37)
     _, thr = _cb(bits)
     bias = synth.make_bias(n, 37)
@@ -537,13 +542,14 @@ def test_layer_otf_single_launch(cuda, oracle, monkeypatch, bits, x_dtype, out_d
     d = lambda t: t.to(cuda)
     args = (d(x), d(thr), d(cb), d(packed), d(cb), d(center), d(scale), d(code_sum), d(bias), bits, 64)
     outs = []
-    for flag in ("1", "0"):
+    for flag in ("2", "0", "1"):
         monkeypatch.setenv("ARCQ_OTF_FUSED", flag)
         ws = torch.full((m, k), float("nan"), dtype=torch.float16, device=cuda)
         y = ops.linear_otf(*args, out_dtype=out_dtype, x_hat_ws=ws)
         outs.append((y, ws))
-    assert torch.equal(outs[0][0], outs[1][0])
-    assert torch.equal(outs[0][1], outs[1][1])
+    for other in outs[1:]:
+        assert torch.equal(outs[0][0], other[0])
+        assert torch.equal(outs[0][1], other[1])
     want_xhat = oracle.act_quant_c(x.float().numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)
     assert np.array_equal(_np(outs[0][1]).view(np.uint16), want_xhat.view(np.uint16))
     w = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, bits, 64).astype(np.float16)
