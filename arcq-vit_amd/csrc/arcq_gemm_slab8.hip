@@ -4,8 +4,8 @@
 // In that layout the MFMA fragment of a 32-row block and k-step (lane = row, 8 consecutive k) is one fully coalesced
 // 16-byte load per lane (512 contiguous bytes per half wave), so x_hat goes from L2 straight into the operand
 // registers: no LDS tile, no LDS writes, no wave-level synchronization.  That frees enough registers and LDS
-// bandwidth for EIGHT waves per workgroup (two per SIMD), each multiplying one 32-row block at a time with the
-// resident 128-column slab; the second wave of a SIMD keeps the matrix pipe busy while the first waits on L2.
+// bandwidth for EIGHT or TWELVE waves per workgroup (two or three per SIMD), each multiplying one 32-row block at a
+// time with the resident 128-column slab; the other waves of a SIMD keep the matrix pipe busy while one waits on L2.
 // (With x_hat row-major a fragment load touches 32 rows per instruction, which costs the texture path more than the
 // MFMAs it feeds; staging through LDS instead saturates LDS bandwidth at two waves per SIMD.)
 //
@@ -27,8 +27,6 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
-constexpr int kThreads = 512;
-constexpr int kWaves = kThreads / 64;
 constexpr int kSlabN = 128;                 // columns per slab
 constexpr int kSliceGroups = 6;             // groups per K slice
 constexpr int kPitch = kSliceGroups * 128 + 16;   // bytes per slab row: 384 halves + 16 B pad (conflict-free 16-B reads)
@@ -36,10 +34,7 @@ constexpr int kSlabBytes = kSlabN * kPitch;       // 100352
 constexpr int kTJ = kSlabN / 32;            // 4 column blocks
 constexpr int kStageRow = 144;              // bytes per staged output row: 128 + 16 pad
 constexpr int kStageTile = 32 * kStageRow;  // 4608 B per wave
-constexpr int kStageBytes = kWaves * kStageTile;
 constexpr int kHalves = 2 * kSliceGroups;   // half groups (32 codes) per slab row and slice
-constexpr int kRounds = kSlabN * kHalves / kThreads;       // half groups per thread and slice
-static_assert(kSlabN * kHalves % kThreads == 0, "slice work must divide evenly");
 
 template <int BITS>
 __device__ __forceinline__ void load_codes(const uint8_t *__restrict__ p, uint32_t (&w)[BITS])
@@ -68,14 +63,20 @@ __device__ __forceinline__ uint32_t code_at(const uint32_t (&w)[BITS], int q)
 
 // PRE = true: the weights were reconstructed beforehand into a fp16 [N,K] buffer; slab slices are copied,
 // global -> LDS directly, instead of rebuilt.
-template <int BITS, typename TOUT, bool PRE>
-__global__ void __launch_bounds__(kThreads)
+// WAVES = 8 or 12 waves per workgroup (two or three per SIMD).
+template <int BITS, typename TOUT, bool PRE, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
 gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw, const float *__restrict__ cb,
                   const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
                   const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K,
                   int row_ranges, int blocks_per_range, const __half *__restrict__ w_hat)
 {
     constexpr int L = 1 << BITS;
+    constexpr int kWaves = WAVES;
+    constexpr int kThreads = 64 * WAVES;
+    constexpr int kStageBytes = kWaves * kStageTile;
+    constexpr int kRounds = kSlabN * kHalves / kThreads;       // half groups per thread and slice
+    static_assert(kSlabN * kHalves % kThreads == 0, "slice work must divide evenly");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     unsigned char *slab = smem;
     float *lut = reinterpret_cast<float *>(smem + kSlabBytes + kStageBytes);      // [L][64]
@@ -101,7 +102,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     const int blk0 = (tile / n_slabs) * blocks_per_range;
     const int blk1 = min(total_blocks, blk0 + blocks_per_range);
     // Row blocks of this wave: blk0 + wave, + 8, + 16, ... (one per pass).  Dealing them round-robin instead of in
-    // contiguous runs keeps the four SIMDs (waves w and w + 4 share one) within one block of each other.
+    // contiguous runs keeps the four SIMDs (waves w, w + 4, w + 8 share one) within one block of each other.
     const int passes = (blk1 - blk0 + kWaves - 1) / kWaves;      // same for all waves: barriers stay uniform
     const int slices = (G + kSliceGroups - 1) / kSliceGroups;
 
@@ -139,8 +140,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     // writes lane l's piece at the wave-uniform LDS base + 16 l); the caller waits for vmcnt and the barrier.
     auto copy_slice = [&](int g0, int ng) {
         const bool active = lane < 8 * ng;
-        for (int rr = 0; rr < kSlabN / kWaves; ++rr) {
-            const int row = wave * (kSlabN / kWaves) + rr;
+        for (int row = wave; row < kSlabN; row += kWaves) {
             const int n = min(n_base + row, N - 1);
             if (active)
                 __builtin_amdgcn_global_load_lds(
@@ -341,12 +341,12 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     }
 }
 
-template <int BITS, typename TOUT, bool PRE>
-void launch_slab8(const GemmArgs &g, hipStream_t stream, const void *w_hat)
+template <int BITS, typename TOUT, bool PRE, int WAVES>
+void launch_slab8_w(const GemmArgs &g, hipStream_t stream, const void *w_hat)
 {
     constexpr int L = 1 << BITS;
-    const size_t smem = kSlabBytes + kStageBytes + L * 64 * sizeof(float) + kSlabN * sizeof(float);
-    auto kernel = gemm_slab8_kernel<BITS, TOUT, PRE>;
+    const size_t smem = kSlabBytes + WAVES * kStageTile + L * 64 * sizeof(float) + kSlabN * sizeof(float);
+    auto kernel = gemm_slab8_kernel<BITS, TOUT, PRE, WAVES>;
     static bool configured = false;   // per instantiation; the attribute is sticky for the process
     if (!configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -362,10 +362,32 @@ void launch_slab8(const GemmArgs &g, hipStream_t stream, const void *w_hat)
     const int blocks_per_range = (total_blocks + ranges - 1) / ranges;
     ranges = (total_blocks + blocks_per_range - 1) / blocks_per_range;
     const int tiles = n_slabs * ranges;
-    hipLaunchKernelGGL(kernel, dim3(8 * ((tiles + 7) / 8)), dim3(kThreads), smem, stream,
+    hipLaunchKernelGGL(kernel, dim3(8 * ((tiles + 7) / 8)), dim3(64 * WAVES), smem, stream,
                        static_cast<const __half *>(g.x_hat), g.pw, g.cb, g.wc, g.ws, g.wcs, g.bias,
                        static_cast<TOUT *>(g.y), g.M, g.N, g.K, ranges, blocks_per_range,
                        static_cast<const __half *>(w_hat));
+}
+
+// Waves per workgroup.  While one wave of a SIMD writes its block out (2-2.5 us per pass: the stores queue behind
+// everybody else's) only the others multiply, so with two waves per SIMD much of the kernel runs one wave per SIMD,
+// at the L2-stall-bound rate.  A third wave (12 per workgroup: the copying variant fits 168 VGPRs) keeps two
+// multiplying: 5-15 % faster on the DeiT-B / ViT-L shapes (ViT-L fc1 562 -> 506 us, DeiT-B fc2 80.6 -> 68.0), but
+// 5-10 % slower where a workgroup has little work to deal out (all four DeiT-S shapes: at most 19 blocks of at most
+// 24 groups).  The variant that rebuilds weights in the kernel needs too many registers for three.
+template <int BITS, typename TOUT, bool PRE>
+void launch_slab8(const GemmArgs &g, hipStream_t stream, const void *w_hat)
+{
+    if constexpr (PRE) {
+        const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
+        const int total_blocks = g.M / 32;
+        const int ranges = max(1, min(256 / n_slabs, total_blocks));
+        const int64_t units = static_cast<int64_t>((total_blocks + ranges - 1) / ranges) * (g.K / 64);
+        if (units >= 256) {
+            launch_slab8_w<BITS, TOUT, PRE, 12>(g, stream, w_hat);
+            return;
+        }
+    }
+    launch_slab8_w<BITS, TOUT, PRE, 8>(g, stream, w_hat);
 }
 
 }  // namespace

@@ -347,3 +347,10 @@ def test_fullsize_gemm_shapes(cuda, oracle, m, n, k, bits):
     assert (y[rows] - lib).abs().max() < 1e-3 * lib.abs().max()
     y64, mag = oracle.linear_f64_c(_np(xh[rows]), _np(w16), _np(bias))
     assert np.all(np.abs(_np(y[rows]).astype(np.float64) - y64) <= (k + 2) * 2.0 ** -24 * mag)
+    # The same product from x_hat in the 32-row block layout (eight waves per workgroup for the DeiT-S shapes, twelve
+    # for the larger ones when the weights are ready): bit-identical, rebuilding the weights or copying them.
+    del y_part, y16, lib
+    xb = xh.reshape(m // 32, 32, k // 8, 8).permute(0, 2, 1, 3).contiguous()
+    assert torch.equal(ops.linear_fused_blocked(xb, m, k, pw, cb, wc, ws, wcs, bias, bits, out_dtype=torch.float32), y)
+    assert torch.equal(ops.linear_fused_blocked(xb, m, k, pw, cb, wc, ws, wcs, bias, bits, out_dtype=torch.float32,
+                                                w_hat_ws=w16.reshape(-1), w_hat_ready=True), y)
