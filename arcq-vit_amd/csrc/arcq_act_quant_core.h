@@ -178,4 +178,91 @@ __device__ __forceinline__ void group_codes64(float (&xv)[64], float mu, float v
     sum_out = sum_codes;
 }
 
+// ---- two lanes per group -------------------------------------------------------------------------------------
+// For launches too small to fill the chip the length of one lane's instruction chain is what counts.  Lanes 2i and
+// 2i + 1 then share group i: the even lane holds inputs 0..31, the odd lane inputs 32..63.  The per-element work
+// halves; the three group sums keep their serial left-to-right order by running in two phases (the even lane folds
+// its half from 0, hands the partial sum to the odd lane, which folds its half on top; every lane executes both
+// phases and the phase that is not its own is discarded), so every result bit is the one-lane routine's.
+__device__ __forceinline__ float from_even_lane(float v)     // the pair's even lane's value, in both lanes
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xA0, 0xf, 0xf, false));    // quad_perm [0,0,2,2]
+}
+__device__ __forceinline__ float from_odd_lane(float v)      // the pair's odd lane's value, in both lanes
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xF5, 0xf, 0xf, false));    // quad_perm [1,1,3,3]
+}
+
+// Serial sum of the group's 64 values v_0 + v_1 + ... (from 0.0f, left to right), this lane holding its half.
+__device__ __forceinline__ float pair_serial_sum(const float (&v)[32])
+{
+    float a = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) a += v[j];           // even lane: values 0..31
+    float b = from_even_lane(a);
+#pragma unroll
+    for (int j = 0; j < 32; ++j) b += v[j];           // odd lane: ... + values 32..63
+    return from_odd_lane(b);
+}
+
+// xv: this lane's 32 inputs on entry, the residuals d_j = x_j - mu on exit; mu, var, s as group_stats64, in both lanes.
+__device__ __forceinline__ void group_stats32x2(float (&xv)[32], float eps, float &mu_out, float &var_out, float &s_out)
+{
+    const float mu = pair_serial_sum(xv) * 0.015625f;     // exact: /64
+    float sq[32];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+        xv[j] -= mu;
+        sq[j] = xv[j] * xv[j];
+    }
+    const float var = pair_serial_sum(sq);
+    mu_out = mu;
+    var_out = var;
+    s_out = sqrtf(var * 0.015625f + eps);
+}
+
+// xv: residuals on entry, cb[code_j] on exit; sum_out = the serial sum of all 64 cb[code_j], in both lanes.  The
+// whole wave must call it (the fast/slow decision is wave-uniform).
+template <int BITS>
+__device__ __forceinline__ void group_codes32x2(float (&xv)[32], float mu, float var, float s,
+                                                const float (&th)[(1 << BITS) - 1], const BucketScale &bq,
+                                                const Bucket *table, const float *lut, bool table_ok, int lane,
+                                                float &sum_out)
+{
+    constexpr int L = 1 << BITS;
+    const bool lane_fast = (s >= 0x1p-60f) && (s <= 0x1p60f) && !(fabsf(mu) < 0x1p-66f && var > 0.0f);
+    const bool fast = table_ok && __all(lane_fast);
+    if (fast) {
+        const float y = 1.0f / s;
+        const float ns = -s;
+        const uint32_t lane4 = static_cast<uint32_t>(lane) * 4u;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            const float d = xv[j];
+            float q = d * y;
+            float e = __fmaf_rn(ns, q, d);
+            q = __fmaf_rn(e, y, q);
+            e = __fmaf_rn(ns, q, d);
+            q = __fmaf_rn(e, y, q);        // == RN(d / s)
+            const Bucket bk = table[bucket_of(q, bq)];
+            const uint32_t c = static_cast<uint32_t>(bk.base) + ((q > bk.thr) ? 1u : 0u);
+            xv[j] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(lut) + ((c << 8) | lane4));
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            const float t = xv[j] / s;
+            uint32_t c = 0;
+            bool alive = true;
+#pragma unroll
+            for (int i = 0; i < L - 1; ++i) {   // while (c < L-1 && t > thr[c]) ++c
+                alive = alive && (t > th[i]);
+                c += alive ? 1u : 0u;
+            }
+            xv[j] = lut[c * 64 + lane];
+        }
+    }
+    sum_out = pair_serial_sum(xv);
+}
+
 }  // namespace arcq

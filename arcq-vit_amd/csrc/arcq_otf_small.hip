@@ -58,25 +58,25 @@ struct OsWeights {                  // what one wave needs of the weights for on
     float c[2], s[2], m[2];
 };
 
-// The lane's group (64 consecutive inputs): raw 16-byte loads (zeros when `valid` is false), converted later so
-// that the loads can be in flight during the table setup.
-template <typename TIN> struct OsGroupRegs { u32x4_t raw[sizeof(TIN) == 2 ? 8 : 16]; };
+// The lane's E consecutive inputs (a whole group, or half of one when two lanes share a group): raw 16-byte loads
+// (zeros when `valid` is false), converted later so that the loads can be in flight during the table setup.
+template <typename TIN, int E> struct OsGroupRegs { u32x4_t raw[E * sizeof(TIN) / 16]; };
 
-template <typename TIN>
-__device__ __forceinline__ void os_fetch_group(const TIN *__restrict__ src, bool valid, OsGroupRegs<TIN> &r)
+template <typename TIN, int E>
+__device__ __forceinline__ void os_fetch_group(const TIN *__restrict__ src, bool valid, OsGroupRegs<TIN, E> &r)
 {
-    constexpr int n = sizeof(TIN) == 2 ? 8 : 16;
+    constexpr int n = E * sizeof(TIN) / 16;
 #pragma unroll
     for (int i = 0; i < n; ++i)
         r.raw[i] = valid ? reinterpret_cast<const u32x4_t *>(src)[i] : u32x4_t{0u, 0u, 0u, 0u};
 }
 
-template <typename TIN>
-__device__ __forceinline__ void os_convert_group(const OsGroupRegs<TIN> &r, float (&xv)[64])
+template <typename TIN, int E>
+__device__ __forceinline__ void os_convert_group(const OsGroupRegs<TIN, E> &r, float (&xv)[E])
 {
     if constexpr (sizeof(TIN) == 2) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < E / 8; ++i)
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
                 const uint32_t w = r.raw[i][d];
@@ -85,13 +85,14 @@ __device__ __forceinline__ void os_convert_group(const OsGroupRegs<TIN> &r, floa
             }
     } else {
 #pragma unroll
-        for (int i = 0; i < 16; ++i)
+        for (int i = 0; i < E / 4; ++i)
 #pragma unroll
             for (int d = 0; d < 4; ++d) xv[4 * i + d] = __uint_as_float(r.raw[i][d]);
     }
 }
 
-template <typename TIN, int BITS, typename TOUT, int RB>   // RB = 32-row blocks per workgroup tile (1 or 2)
+// RB = 32-row blocks per workgroup tile (1 or 2); LPG = lanes per quantization group in stage 1 (1 or 2).
+template <typename TIN, int BITS, typename TOUT, int RB, int LPG>
 __global__ void __launch_bounds__(kOsWaves * 64)
 otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, const float *__restrict__ a_cb,
                  const uint8_t *__restrict__ pw, const float *__restrict__ w_cb,
@@ -147,23 +148,32 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     if (wave < G) fetch_w(wave, o0);
 
     // ---- stage 1: x_hat of the RT rows into LDS -----------------------------------------------------------
-    // Group f = t0 + lane of the row tile (row f / G, group f % G).  The first round's inputs are requested before
-    // the table setup so that one memory latency hides behind it.
+    // A wave tile is GPT consecutive groups of the row tile (group f = row f / G, group f % G), LPG lanes per group,
+    // each lane holding EL consecutive inputs.  With two lanes per group the per-lane instruction chain, which is
+    // what a launch this small waits for, is half as long (arcq_act_quant_core.h); it is used while the row tile is
+    // at most eight such tiles (K <= 512 for 32 rows), i.e. while it does not add a round.
+    constexpr int EL = 64 / LPG, GPT = 64 / LPG;
     const int groups = RT * G;
-    OsGroupRegs<TIN> in;
+    OsGroupRegs<TIN, EL> in;
     auto fetch_x = [&](int t0) {
-        const int f = t0 + lane;
+        const int f = t0 + lane / LPG;
         const int row = f / G, g = f - row * G;
-        os_fetch_group<TIN>(x + static_cast<int64_t>(min(m0 + row, M - 1)) * K + g * 64, f < groups && m0 + row < M, in);
+        os_fetch_group<TIN, EL>(x + static_cast<int64_t>(min(m0 + row, M - 1)) * K + g * 64 + (lane % LPG) * EL,
+                               f < groups && m0 + row < M, in);
     };
-    // Wave w owns the 64-group tiles w, w + 8, ... of the row tile.  With fewer than eight tiles (K <= 448 for 32
-    // rows) the waves without one build the lookup tables while the others take their statistics, and one barrier
-    // joins the two halves; otherwise all eight waves build the tables between the two halves of their first tile.
-    const int n_tiles = (groups + 63) / 64;
+    float xv[EL];
+    float mu = 0.0f, var = 0.0f, s = 0.0f;
+    auto stats = [&]() {
+        os_convert_group<TIN, EL>(in, xv);
+    };
+    // Wave w owns the tiles w, w + 8, ... of the row tile.  With fewer than eight tiles the waves without one build
+    // the lookup tables while the others take their statistics, and one barrier joins the two halves; otherwise all
+    // eight waves build the tables between the two halves of their first tile.
+    const int n_tiles = (groups + GPT - 1) / GPT;
     const bool spare_waves = n_tiles < kOsWaves;
     const int tile_waves = spare_waves ? n_tiles : kOsWaves;
     const bool has_tile = wave < n_tiles;
-    if (has_tile) fetch_x(wave * 64);
+    if (has_tile) fetch_x(wave * GPT);
     float th[L - 1], cbv[L];
     load_quant_params<BITS>(a_thr, a_cb, th, cbv);
     const BucketScale bq = pick_bucket_scale<BITS>(th);
@@ -173,12 +183,11 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
 #pragma unroll
         for (int c = 0; c < L; ++c) w_lut[c * 64 + lane] = w_cb[c];
     }
-    float xv[64];
-    float mu = 0.0f, var = 0.0f, s = 0.0f;
     if (has_tile) {
-        os_convert_group<TIN>(in, xv);
-        if (wave + kOsWaves < n_tiles) fetch_x((wave + kOsWaves) * 64);      // the next tile's inputs, one round ahead
-        group_stats64(xv, eps, mu, var, s);
+        stats();
+        if (wave + kOsWaves < n_tiles) fetch_x((wave + kOsWaves) * GPT);      // the next tile's inputs, one round ahead
+        if constexpr (LPG == 1) group_stats64(xv, eps, mu, var, s);
+        else group_stats32x2(xv, eps, mu, var, s);
     }
     if (!spare_waves) build_quant_tables_by<BITS>(th, cbv, bq, a_lut, table, slow_slots, tid, kOsWaves * 64);
     __syncthreads();
@@ -187,35 +196,41 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     for (int w = 0; w < (spare_waves ? kOsWaves - tile_waves : kOsWaves); ++w) table_ok = table_ok && (slow_slots[w] == 0);
     for (int t = wave; t < n_tiles; t += kOsWaves) {
         if (t != wave) {                       // later tiles of this wave: their inputs were requested a round ago
-            os_convert_group<TIN>(in, xv);
-            if (t + kOsWaves < n_tiles) fetch_x((t + kOsWaves) * 64);
-            group_stats64(xv, eps, mu, var, s);
+            stats();
+            if (t + kOsWaves < n_tiles) fetch_x((t + kOsWaves) * GPT);
+            if constexpr (LPG == 1) group_stats64(xv, eps, mu, var, s);
+            else group_stats32x2(xv, eps, mu, var, s);
         }
-        const int f = t * 64 + lane;
+        const int f = t * GPT + lane / LPG;
         const int row = f / G, g = f - row * G;
         const bool valid = f < groups && m0 + row < M;
         float sum_codes;
-        uint32_t code[1];
-        group_codes64<BITS, false>(xv, mu, var, s, th, bq, table, a_lut, table_ok, lane, sum_codes, code);
+        if constexpr (LPG == 1) {
+            uint32_t code[1];
+            group_codes64<BITS, false>(xv, mu, var, s, th, bq, table, a_lut, table_ok, lane, sum_codes, code);
+        } else {
+            group_codes32x2<BITS>(xv, mu, var, s, th, bq, table, a_lut, table_ok, lane, sum_codes);
+        }
         const float code_mean = sum_codes * 0.015625f;
-        u32x4_t out[8];
+        u32x4_t out[EL / 8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < EL / 8; ++i)
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
                 const int j = i * 8 + 2 * d;
                 const __half2 h = __floats2half2_rn(fma_f32(s, xv[j] - code_mean, mu), fma_f32(s, xv[j + 1] - code_mean, mu));
                 out[i][d] = *reinterpret_cast<const uint32_t *>(&h);
             }
+        const int part = (lane % LPG) * EL;      // first element of this lane inside its group
         if (f < groups) {
-            unsigned char *dst = xt + row * row_pitch + g * kOsGroupPitch;
+            unsigned char *dst = xt + row * row_pitch + g * kOsGroupPitch + part * 2;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) reinterpret_cast<u32x4_t *>(dst)[i] = out[i];
+            for (int i = 0; i < EL / 8; ++i) reinterpret_cast<u32x4_t *>(dst)[i] = out[i];
         }
         if (write_ws && valid) {
-            u32x4_t *dst = reinterpret_cast<u32x4_t *>(x_hat_ws + static_cast<int64_t>(m0 + row) * K + g * 64);
+            u32x4_t *dst = reinterpret_cast<u32x4_t *>(x_hat_ws + static_cast<int64_t>(m0 + row) * K + g * 64 + part);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) dst[i] = out[i];
+            for (int i = 0; i < EL / 8; ++i) dst[i] = out[i];
         }
     }
     __syncthreads();
@@ -320,7 +335,7 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     }
 }
 
-template <typename TIN, int BITS, typename TOUT, int RB>
+template <typename TIN, int BITS, typename TOUT, int RB, int LPG>
 static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
 {
     constexpr int L = 1 << BITS;
@@ -333,7 +348,7 @@ static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
     // Both regions side by side while they fit 160 KB of LDS; else the partial tiles reuse the x_hat tile's space.
     const int partial_off = (tile_bytes + partial_bytes + tables <= 160 * 1024) ? tile_bytes : 0;
     const size_t smem = (partial_off ? tile_bytes + partial_bytes : (tile_bytes > partial_bytes ? tile_bytes : partial_bytes)) + tables;
-    auto kernel = otf_small_kernel<TIN, BITS, TOUT, RB>;
+    auto kernel = otf_small_kernel<TIN, BITS, TOUT, RB, LPG>;
     static int configured = 0;        // per instantiation: largest dynamic LDS size requested so far
     if (static_cast<int>(smem) > configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -349,7 +364,9 @@ static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
 template <typename TIN, int BITS, typename TOUT>
 static void launch_os_rb(const OtfSmallArgs &a, hipStream_t stream)
 {
-    launch_os<TIN, BITS, TOUT, 1>(a, stream);
+    // Two lanes per group while the 32-row tile is at most eight 32-group tiles: half the chain, no extra round.
+    if (32 * (a.K / 64) <= 8 * 32) launch_os<TIN, BITS, TOUT, 1, 2>(a, stream);
+    else launch_os<TIN, BITS, TOUT, 1, 1>(a, stream);
 }
 
 template <typename TIN, typename TOUT>
