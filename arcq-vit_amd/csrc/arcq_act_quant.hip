@@ -365,6 +365,85 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
     }
 }
 
+// Small launches, x_hat only: two lanes per group, no LDS tile.  When the tensor is too small to fill the chip
+// (a few hundred rows) the launch lasts as long as one lane's instruction chain, so the group is shared by two lanes
+// (arcq_act_quant_core.h: half the per-element work per lane, the serial sums in two linked phases, same bits).  A
+// lane's 32 inputs are contiguous and consecutive lanes hold consecutive halves, so plain 16-byte loads and stores
+// are already coalesced.  Every lane reads all its inputs before it writes, so x_hat may alias x.
+template <typename TIN, typename TOUT, int BITS>
+__global__ void __launch_bounds__(64 * kWaves)
+act_quant_small_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, const float *__restrict__ cb,
+                       TOUT *__restrict__ x_hat, int64_t total_groups, float eps)
+{
+    constexpr int L = 1 << BITS;
+    constexpr int kIn = 32 * sizeof(TIN) / 16, kOut = 32 * sizeof(TOUT) / 16;
+    __shared__ float lut[L * 64];
+    __shared__ Bucket table[kMaxBuckets + 1];
+    __shared__ int slow_slots[kWaves];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int64_t f = (static_cast<int64_t>(blockIdx.x) * kWaves + (tid >> 6)) * 32 + (lane >> 1);   // this lane's group
+    const bool valid = f < total_groups;
+    const int64_t e0 = f * 64 + (lane & 1) * 32;                                                    // its first element
+
+    uint4 raw[kIn];
+#pragma unroll
+    for (int i = 0; i < kIn; ++i)
+        raw[i] = valid ? reinterpret_cast<const uint4 *>(x + e0)[i] : make_uint4(0, 0, 0, 0);
+    float th[L - 1], cbv[L];
+    load_quant_params<BITS>(thr, cb, th, cbv);
+    const BucketScale bq = pick_bucket_scale<BITS>(th);
+
+    float xv[32];
+    if constexpr (sizeof(TIN) == 2) {
+#pragma unroll
+        for (int i = 0; i < kIn; ++i) {
+            const uint32_t w[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                xv[i * 8 + 2 * d] = __half2float(__ushort_as_half(static_cast<unsigned short>(w[d] & 0xffffu)));
+                xv[i * 8 + 2 * d + 1] = __half2float(__ushort_as_half(static_cast<unsigned short>(w[d] >> 16)));
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kIn; ++i) {
+            xv[4 * i] = __uint_as_float(raw[i].x); xv[4 * i + 1] = __uint_as_float(raw[i].y);
+            xv[4 * i + 2] = __uint_as_float(raw[i].z); xv[4 * i + 3] = __uint_as_float(raw[i].w);
+        }
+    }
+    float mu, var, s, sum_codes;
+    group_stats32x2(xv, eps, mu, var, s);
+    build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * kWaves);
+    __syncthreads();
+    bool table_ok = true;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) table_ok = table_ok && (slow_slots[w] == 0);
+    group_codes32x2<BITS>(xv, mu, var, s, th, bq, table, lut, table_ok, lane, sum_codes);
+    const float code_mean = sum_codes * 0.015625f;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) xv[j] = fma_f32(s, xv[j] - code_mean, mu);
+    if (!valid) return;
+    uint4 *dst = reinterpret_cast<uint4 *>(x_hat + e0);
+    if constexpr (sizeof(TOUT) == 2) {
+#pragma unroll
+        for (int i = 0; i < kOut; ++i) {
+            uint32_t w[4];
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const __half2 h = __floats2half2_rn(xv[i * 8 + 2 * d], xv[i * 8 + 2 * d + 1]);
+                w[d] = *reinterpret_cast<const uint32_t *>(&h);
+            }
+            dst[i] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kOut; ++i)
+            dst[i] = make_uint4(__float_as_uint(xv[4 * i]), __float_as_uint(xv[4 * i + 1]), __float_as_uint(xv[4 * i + 2]),
+                                __float_as_uint(xv[4 * i + 3]));
+    }
+}
+
 // Any group size: one thread per group, straight from global memory.  Slow
 // (strided reads) but has no layout assumptions; used when gs != 64 or the
 // pointers are not 16-byte aligned.
@@ -442,7 +521,17 @@ static int launch(const void *x, const float *thr, const float *cb, uint8_t *pac
     const TIN *xin = static_cast<const TIN *>(x);
     TOUT *xo = static_cast<TOUT *>(x_hat);
     const bool fast = gs == 64 && aligned(x, 16) && aligned(x_hat, 16) && aligned(packed, 16) && aligned(codes_u8, 16);
-    if (fast) {
+    // Fewer 64-group tiles than SIMDs and nothing but x_hat wanted: the two-lanes-per-group kernel.
+    if (fast && x_hat && !packed && !codes_u8 && !center && !scale && !code_sum && total_groups <= 1024 * 64) {
+        const unsigned blocks = static_cast<unsigned>((total_groups + 32 * kWaves - 1) / (32 * kWaves));
+#define ARCQ_LAUNCH_SMALL(B) \
+    hipLaunchKernelGGL((act_quant_small_kernel<TIN, TOUT, B>), dim3(blocks), dim3(64 * kWaves), 0, stream, xin, thr, cb, xo, \
+                       total_groups, eps)
+        if (bits == 4) ARCQ_LAUNCH_SMALL(4);
+        else if (bits == 3) ARCQ_LAUNCH_SMALL(3);
+        else ARCQ_LAUNCH_SMALL(2);
+#undef ARCQ_LAUNCH_SMALL
+    } else if (fast) {
         const int64_t ntiles = (total_groups + kTileGroups - 1) / kTileGroups;
         // Up to 3 workgroups fit a CU (LDS); more tiles than that are walked by the grid-stride loop.
         const int64_t want = (ntiles + kWaves - 1) / kWaves;
