@@ -90,62 +90,6 @@ __device__ __forceinline__ void store_tile(TOUT *__restrict__ out, int64_t elem0
     }
 }
 
-// Block-layout tiles.  When x_hat is wanted in the 32-row block layout the eight-wave GEMM reads (16-byte pieces
-// ordered [row / 32][k / 8][row % 32]) a tile is 32 rows x 2 groups instead of 64 consecutive groups: lane l owns
-// (row l % 32, group 2 * pair + l / 32), so that every piece column of the tile leaves as one contiguous 512-byte run.
-// (Scattering a 64-consecutive-groups tile into that layout as 16-byte stores measured 1.7x slower for the whole
-// kernel.)  A row's two groups are 128 contiguous values in the input, so the loads stay coalesced.  With an odd
-// group count the last pair has one group and lanes 32..63 idle.
-template <typename TIN> struct BlockTile {
-    static constexpr int pieces = 128 / Tile<TIN>::vec;     // 16-byte pieces per row of the tile (16 fp16 / 32 fp32)
-    static constexpr int rows_per_instr = 64 / pieces;      // 4 / 2
-    static constexpr int iters = 32 / rows_per_instr;       // 8 / 16 == the row-major tile's count
-};
-
-template <typename TIN>
-__device__ __forceinline__ void fetch_tile_blocked(const TIN *__restrict__ x, bool tile_valid, int64_t row0, int pair,
-                                                   int groups_per_row, TileRegs<TIN> &r, int lane)
-{
-    using B = BlockTile<TIN>;
-    const int pc = lane % B::pieces;
-    const bool ok = tile_valid && (2 * pair + pc / (B::pieces / 2) < groups_per_row);
-    const TIN *p = x + (row0 + lane / B::pieces) * (static_cast<int64_t>(groups_per_row) * 64) + pair * 128 + pc * Tile<TIN>::vec;
-#pragma unroll
-    for (int i = 0; i < B::iters; ++i)
-        r.raw[i] = ok ? *reinterpret_cast<const uint4 *>(p + static_cast<int64_t>(i * B::rows_per_instr) * groups_per_row * 64)
-                      : make_uint4(0, 0, 0, 0);
-}
-
-template <typename TIN>
-__device__ __forceinline__ void commit_tile_blocked(const TileRegs<TIN> &r, uint32_t *__restrict__ tile, int lane)
-{
-    using B = BlockTile<TIN>;
-    const int pc = lane % B::pieces;
-    const int gsel = pc / (B::pieces / 2);
-    uint32_t *dst0 = tile + (gsel * 32 + lane / B::pieces) * Tile<TIN>::stride + (pc % (B::pieces / 2)) * 4;
-#pragma unroll
-    for (int i = 0; i < B::iters; ++i) {
-        uint32_t *dst = dst0 + i * B::rows_per_instr * Tile<TIN>::stride;
-        dst[0] = r.raw[i].x; dst[1] = r.raw[i].y; dst[2] = r.raw[i].z; dst[3] = r.raw[i].w;
-    }
-}
-
-// fp16 x_hat of a block tile: instruction j writes piece columns 2j and 2j + 1 of the tile (lanes 0..31 / 32..63),
-// each 32 rows x 16 bytes = 512 contiguous bytes of the block layout.
-__device__ __forceinline__ void store_tile_blocked(__half *__restrict__ out, int64_t row_block, int pair,
-                                                   int groups_per_row, const uint32_t *__restrict__ tile, int lane)
-{
-    const int row = lane & 31;
-    __half *base = out + row_block * (static_cast<int64_t>(groups_per_row) * (64 * 32)) + row * 8;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int kp = j * 2 + (lane >> 5);                 // piece column inside the tile: group kp / 8, piece kp % 8
-        if (2 * pair + kp / 8 >= groups_per_row) continue;
-        const uint32_t *src = tile + ((kp / 8) * 32 + row) * Tile<__half>::stride + (kp % 8) * 4;
-        *reinterpret_cast<uint4 *>(base + static_cast<int64_t>(pair * 16 + kp) * (32 * 8)) = make_uint4(src[0], src[1], src[2], src[3]);
-    }
-}
-
 // The lane's own group (row `lane` of the tile) as 64 floats.
 template <typename TIN>
 __device__ __forceinline__ void read_row(const uint32_t *__restrict__ row, float (&v)[64])
@@ -221,15 +165,12 @@ struct WeightJob {
     unsigned blocks;
 };
 
-// BLOCKED (fp16 x_hat only, no other outputs): block tiles and the 32-row block layout for x_hat; the work is
-// row_blocks * ceil(groups_per_row / 2) tiles, and `wj` may add weight-reconstruction workgroups in front.
-template <typename TIN, typename TOUT, int BITS, bool CODES, bool BLOCKED = false>
+template <typename TIN, typename TOUT, int BITS, bool CODES>
 __global__ void __launch_bounds__(64 * kWaves)
 act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, const float *__restrict__ cb,
                      uint8_t *__restrict__ packed, uint8_t *__restrict__ codes_u8,
                      float *__restrict__ center, float *__restrict__ scale, float *__restrict__ code_sum,
-                     TOUT *__restrict__ x_hat, int64_t total_groups, float eps,
-                     int groups_per_row, int row_blocks, WeightJob wj)
+                     TOUT *__restrict__ x_hat, int64_t total_groups, float eps)
 {
     constexpr int L = 1 << BITS;
     constexpr int kStride = (Tile<TIN>::stride > Tile<TOUT>::stride) ? Tile<TIN>::stride : Tile<TOUT>::stride;
@@ -242,33 +183,14 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
     const int lane = tid & 63;
     const int wave = tid >> 6;
 
-    unsigned first_block = 0, act_blocks = gridDim.x;
-    if constexpr (BLOCKED) {
-        if (blockIdx.x < wj.blocks) {          // workgroup-uniform: this workgroup rebuilds weights and is done
-            weight_dequant8_block<__half, BITS>(blockIdx.x, lut, wj.packed, wj.cb, wj.center, wj.scale, wj.code_sum,
-                                                wj.out, wj.N, wj.K, 64);
-            return;
-        }
-        first_block = wj.blocks;
-        act_blocks = gridDim.x - wj.blocks;
-    }
-    const int64_t wg = blockIdx.x - first_block;       // workgroup number among the activation workgroups
-
     // The first tile of this wave is requested before anything else: its latency overlaps the setup below.
-    const int pairs = BLOCKED ? (groups_per_row + 1) / 2 : 1;
-    const int64_t ntiles = BLOCKED ? static_cast<int64_t>(row_blocks) * pairs : (total_groups + kTileGroups - 1) / kTileGroups;
+    const int64_t ntiles = (total_groups + kTileGroups - 1) / kTileGroups;
     const int64_t elem_end = total_groups * 64;
     TileRegs<TIN> regs;
-    auto fetch = [&](int64_t tile_id) {          // zero-fills past the end
-        if constexpr (BLOCKED) {
-            const int64_t rb = tile_id / pairs;
-            fetch_tile_blocked<TIN>(x, tile_id < ntiles, rb * 32, static_cast<int>(tile_id - rb * pairs), groups_per_row,
-                                    regs, lane);
-        } else {
-            fetch_tile<TIN>(x, tile_id * kTileGroups * 64, elem_end, regs, lane);
-        }
-    };
-    fetch(wg * kWaves + wave);
+    {
+        const int64_t first = static_cast<int64_t>(blockIdx.x) * kWaves + wave;
+        fetch_tile<TIN>(x, first * kTileGroups * 64, elem_end, regs, lane);      // zero-fills past the end
+    }
 
     // Thresholds and codebook are requested now and first used after the first tile's statistics: the lookup
     // tables are built once per workgroup, between the two halves of the first tile, so that their load latency
@@ -282,12 +204,12 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
     uint32_t *tile = tiles[wave];
 
     // All four waves run the same number of iterations so that the barriers below are uniform.
-    for (int64_t tile0 = wg * kWaves; tile0 < ntiles; tile0 += static_cast<int64_t>(act_blocks) * kWaves) {
+    for (int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kWaves; tile0 < ntiles;
+         tile0 += static_cast<int64_t>(gridDim.x) * kWaves) {
         const int64_t group0 = (tile0 + wave) * kTileGroups;
         const int64_t elem0 = group0 * 64;
-        if (tile0 != wg * kWaves) fetch(tile0 + wave);
-        if constexpr (BLOCKED) commit_tile_blocked<TIN>(regs, tile, lane);
-        else commit_tile<TIN>(regs, tile, lane);
+        if (tile0 != static_cast<int64_t>(blockIdx.x) * kWaves) fetch_tile<TIN>(x, elem0, elem_end, regs, lane);
+        commit_tile<TIN>(regs, tile, lane);
         __syncthreads();
 
         float xv[64];
@@ -308,7 +230,7 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
         group_codes64<BITS, CODES>(xv, mu, var, s, th, bq, table, lut, table_ok, lane, sum_codes, code);
 
         const int64_t g = group0 + lane;
-        if (!BLOCKED && g < total_groups) {
+        if (g < total_groups) {
             if (center) center[g] = mu;
             if (scale) scale[g] = s;
             if (code_sum) code_sum[g] = sum_codes;
@@ -352,14 +274,7 @@ act_quant_g64_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, c
             // rewritten now, possibly with a different stride.
             write_row<TOUT>(tile + lane * Tile<TOUT>::stride, xv);
             __syncthreads();
-            if constexpr (BLOCKED) {
-                const int64_t tile_id = tile0 + wave;
-                const int64_t rb = tile_id / pairs;
-                if (tile_id < ntiles)
-                    store_tile_blocked(x_hat, rb, static_cast<int>(tile_id - rb * pairs), groups_per_row, tile, lane);
-            } else {
-                store_tile<TOUT>(x_hat, elem0, elem_end, tile, lane);
-            }
+            store_tile<TOUT>(x_hat, elem0, elem_end, tile, lane);
         }
         __syncthreads();   // the tile is reloaded in the next iteration
     }
@@ -441,6 +356,125 @@ act_quant_small_kernel(const TIN *__restrict__ x, const float *__restrict__ thr,
         for (int i = 0; i < kOut; ++i)
             dst[i] = make_uint4(__float_as_uint(xv[4 * i]), __float_as_uint(xv[4 * i + 1]), __float_as_uint(xv[4 * i + 2]),
                                 __float_as_uint(xv[4 * i + 3]));
+    }
+}
+
+// Block-layout stage 1 with two lanes per group.  A wave tile is 32 rows x ONE group; lane l owns row l / 2 and the
+// half l % 2 of the group (arcq_act_quant_core.h: two-phase serial sums, same bits as one lane per group).  Halving
+// the tile doubles the number of work items, which is what the K = 384 layers of DeiT-S need: 1 182 whole tiles on
+// 1 024 SIMDs leave 158 SIMDs with two tiles (2 x 1 470 instructions), 2 364 half tiles at most three (3 x 740).
+// Data moves through a wave-private LDS tile (rows of the tile = rows of the tensor, odd dword pitch): coalesced
+// 16-byte loads in, every piece column out as one 512-byte run of the block layout.
+template <typename TIN, int BITS>
+__global__ void __launch_bounds__(64 * kWaves)
+act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, const float *__restrict__ cb,
+                          __half *__restrict__ x_hat, float eps, int groups_per_row, int row_blocks, WeightJob wj)
+{
+    constexpr int L = 1 << BITS;
+    constexpr int kInPitch = Tile<TIN>::stride, kOutPitch = Tile<__half>::stride;     // dwords per tile row
+    constexpr int kPieces = 64 / Tile<TIN>::vec;           // 16-byte pieces per row of the tile (8 fp16 / 16 fp32)
+    constexpr int kRowsPerInstr = 64 / kPieces;            // 8 / 4
+    constexpr int kIters = 32 / kRowsPerInstr;             // 4 / 8
+    __shared__ uint32_t tiles[kWaves][32 * kInPitch];
+    __shared__ float lut[L * 64];
+    __shared__ Bucket table[kMaxBuckets + 1];
+    __shared__ int slow_slots[kWaves];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    if (blockIdx.x < wj.blocks) {          // workgroup-uniform: this workgroup rebuilds weights and is done
+        weight_dequant8_block<__half, BITS>(blockIdx.x, lut, wj.packed, wj.cb, wj.center, wj.scale, wj.code_sum, wj.out,
+                                            wj.N, wj.K, 64);
+        return;
+    }
+    const int64_t wg = blockIdx.x - wj.blocks;
+    const int64_t act_blocks = gridDim.x - wj.blocks;
+    const int64_t ntiles = static_cast<int64_t>(row_blocks) * groups_per_row;
+    const int64_t row_elems = static_cast<int64_t>(groups_per_row) * 64;
+    uint32_t *tile = tiles[wave];
+
+    uint4 raw[kIters];
+    auto fetch = [&](int64_t t) {          // tile t = (row block t / G, group t % G); zero-fills past the end
+        const int64_t rb = t / groups_per_row;
+        const int g = static_cast<int>(t - rb * groups_per_row);
+        const TIN *p = x + (rb * 32 + lane / kPieces) * row_elems + g * 64 + (lane % kPieces) * Tile<TIN>::vec;
+#pragma unroll
+        for (int i = 0; i < kIters; ++i)
+            raw[i] = t < ntiles ? *reinterpret_cast<const uint4 *>(p + i * kRowsPerInstr * row_elems) : make_uint4(0, 0, 0, 0);
+    };
+    fetch(wg * kWaves + wave);
+
+    float th[L - 1], cbv[L];
+    load_quant_params<BITS>(thr, cb, th, cbv);
+    bool table_ok = false, tables_built = false;
+    BucketScale bq;
+    const int row = lane >> 1, half = lane & 1;
+
+    for (int64_t tile0 = wg * kWaves; tile0 < ntiles; tile0 += act_blocks * kWaves) {
+        const int64_t t = tile0 + wave;
+        if (tile0 != wg * kWaves) fetch(t);
+        {
+            uint32_t *dst = tile + (lane / kPieces) * kInPitch + (lane % kPieces) * 4;
+#pragma unroll
+            for (int i = 0; i < kIters; ++i) {
+                uint32_t *d = dst + i * kRowsPerInstr * kInPitch;
+                d[0] = raw[i].x; d[1] = raw[i].y; d[2] = raw[i].z; d[3] = raw[i].w;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();      // the tile is private to the wave and LDS operations execute in order
+        float xv[32];
+        {
+            const uint32_t *src = tile + row * kInPitch + half * (32 * static_cast<int>(sizeof(TIN)) / 4);
+            if constexpr (sizeof(TIN) == 4) {
+#pragma unroll
+                for (int j = 0; j < 32; ++j) xv[j] = __uint_as_float(src[j]);
+            } else {
+#pragma unroll
+                for (int p = 0; p < 16; ++p) {
+                    const uint32_t w = src[p];
+                    xv[2 * p] = __half2float(__ushort_as_half(static_cast<unsigned short>(w & 0xffffu)));
+                    xv[2 * p + 1] = __half2float(__ushort_as_half(static_cast<unsigned short>(w >> 16)));
+                }
+            }
+        }
+        float mu, var, s, sum_codes;
+        group_stats32x2(xv, eps, mu, var, s);
+        if (!tables_built) {                  // once per workgroup, between the two halves of its first tile
+            bq = pick_bucket_scale<BITS>(th);
+            build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * kWaves);
+            __syncthreads();
+            table_ok = true;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) table_ok = table_ok && (slow_slots[w] == 0);
+            tables_built = true;
+        }
+        group_codes32x2<BITS>(xv, mu, var, s, th, bq, table, lut, table_ok, lane, sum_codes);
+        const float code_mean = sum_codes * 0.015625f;
+        {
+            // Every lane has read its inputs (program order within the wave), so rows may be rewritten, with the
+            // output pitch.
+            uint32_t *dst = tile + row * kOutPitch + half * 16;
+#pragma unroll
+            for (int p = 0; p < 16; ++p) {
+                const __half2 h = __floats2half2_rn(fma_f32(s, xv[2 * p] - code_mean, mu), fma_f32(s, xv[2 * p + 1] - code_mean, mu));
+                dst[p] = *reinterpret_cast<const uint32_t *>(&h);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (t < ntiles) {
+            const int64_t rb = t / groups_per_row;
+            const int g = static_cast<int>(t - rb * groups_per_row);
+            const int r = lane & 31;
+            __half *base = x_hat + rb * (row_elems * 32) + (static_cast<int64_t>(g) * 8 * 32 + r) * 8;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {      // instruction j: piece columns 2j and 2j + 1, 32 rows x 16 bytes each
+                const int kp = j * 2 + (lane >> 5);
+                const uint32_t *src = tile + r * kOutPitch + kp * 4;
+                *reinterpret_cast<uint4 *>(base + kp * (32 * 8)) = make_uint4(src[0], src[1], src[2], src[3]);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();      // the tile is refilled in the next iteration
     }
 }
 
@@ -539,7 +573,7 @@ static int launch(const void *x, const float *thr, const float *cb, uint8_t *pac
         const bool codes = packed || codes_u8;
 #define ARCQ_LAUNCH_G64(B, C)                                                                                     \
     hipLaunchKernelGGL((act_quant_g64_kernel<TIN, TOUT, B, C>), dim3(blocks), dim3(64 * kWaves), 0, stream, xin, \
-                       thr, cb, packed, codes_u8, center, scale, code_sum, xo, total_groups, eps, 0, 0, WeightJob{})
+                       thr, cb, packed, codes_u8, center, scale, code_sum, xo, total_groups, eps)
         if (bits == 4) { if (codes) ARCQ_LAUNCH_G64(4, true); else ARCQ_LAUNCH_G64(4, false); }
         else if (bits == 3) { if (codes) ARCQ_LAUNCH_G64(3, true); else ARCQ_LAUNCH_G64(3, false); }
         else { if (codes) ARCQ_LAUNCH_G64(2, true); else ARCQ_LAUNCH_G64(2, false); }
@@ -561,13 +595,13 @@ static int launch_blocked(const void *x, const float *thr, const float *cb, void
 {
     const int groups_per_row = static_cast<int>(cols / 64);
     const int row_blocks = static_cast<int>(rows / 32);
-    const int64_t ntiles = static_cast<int64_t>(row_blocks) * ((groups_per_row + 1) / 2);
+    const int64_t ntiles = static_cast<int64_t>(row_blocks) * groups_per_row;
     const int64_t want = (ntiles + kWaves - 1) / kWaves;
-    const unsigned blocks = static_cast<unsigned>(want < 4096 ? want : 4096) + wj.blocks;
-#define ARCQ_LAUNCH_BLOCKED(B)                                                                                       \
-    hipLaunchKernelGGL((act_quant_g64_kernel<TIN, __half, B, false, true>), dim3(blocks), dim3(64 * kWaves), 0, stream, \
-                       static_cast<const TIN *>(x), thr, cb, nullptr, nullptr, nullptr, nullptr, nullptr,            \
-                       static_cast<__half *>(x_hat), rows * groups_per_row, eps, groups_per_row, row_blocks, wj)
+    const unsigned blocks = static_cast<unsigned>(want < 8192 ? want : 8192) + wj.blocks;
+#define ARCQ_LAUNCH_BLOCKED(B)                                                                                  \
+    hipLaunchKernelGGL((act_quant_blocked2_kernel<TIN, B>), dim3(blocks), dim3(64 * kWaves), 0, stream,        \
+                       static_cast<const TIN *>(x), thr, cb, static_cast<__half *>(x_hat), eps, groups_per_row, \
+                       row_blocks, wj)
     if (bits == 4) ARCQ_LAUNCH_BLOCKED(4);
     else if (bits == 3) ARCQ_LAUNCH_BLOCKED(3);
     else ARCQ_LAUNCH_BLOCKED(2);
