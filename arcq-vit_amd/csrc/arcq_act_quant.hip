@@ -368,7 +368,7 @@ act_quant_small_kernel(const TIN *__restrict__ x, const float *__restrict__ thr,
 template <typename TIN, int BITS>
 __global__ void __launch_bounds__(64 * kWaves)
 act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, const float *__restrict__ cb,
-                          __half *__restrict__ x_hat, float eps, int groups_per_row, int row_blocks, WeightJob wj)
+                          __half *__restrict__ x_hat, float eps, int groups_per_row, int64_t rows, WeightJob wj)
 {
     constexpr int L = 1 << BITS;
     constexpr int kInPitch = Tile<TIN>::stride, kOutPitch = Tile<__half>::stride;     // dwords per tile row
@@ -390,7 +390,7 @@ act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ t
     }
     const int64_t wg = blockIdx.x - wj.blocks;
     const int64_t act_blocks = gridDim.x - wj.blocks;
-    const int64_t ntiles = static_cast<int64_t>(row_blocks) * groups_per_row;
+    const int64_t ntiles = ((rows + 31) / 32) * groups_per_row;
     const int64_t row_elems = static_cast<int64_t>(groups_per_row) * 64;
     uint32_t *tile = tiles[wave];
 
@@ -398,10 +398,12 @@ act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ t
     auto fetch = [&](int64_t t) {          // tile t = (row block t / G, group t % G); zero-fills past the end
         const int64_t rb = t / groups_per_row;
         const int g = static_cast<int>(t - rb * groups_per_row);
-        const TIN *p = x + (rb * 32 + lane / kPieces) * row_elems + g * 64 + (lane % kPieces) * Tile<TIN>::vec;
+        const int64_t r0 = rb * 32 + lane / kPieces;
+        const TIN *p = x + r0 * row_elems + g * 64 + (lane % kPieces) * Tile<TIN>::vec;
 #pragma unroll
-        for (int i = 0; i < kIters; ++i)
-            raw[i] = t < ntiles ? *reinterpret_cast<const uint4 *>(p + i * kRowsPerInstr * row_elems) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < kIters; ++i)         // rows past the tensor's end (a ragged last block) read as zeros
+            raw[i] = (t < ntiles && r0 + i * kRowsPerInstr < rows) ? *reinterpret_cast<const uint4 *>(p + i * kRowsPerInstr * row_elems)
+                                                                   : make_uint4(0, 0, 0, 0);
     };
     fetch(wg * kWaves + wave);
 
@@ -466,12 +468,15 @@ act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ t
             const int64_t rb = t / groups_per_row;
             const int g = static_cast<int>(t - rb * groups_per_row);
             const int r = lane & 31;
-            __half *base = x_hat + rb * (row_elems * 32) + (static_cast<int64_t>(g) * 8 * 32 + r) * 8;
+            const int nrows = static_cast<int>(rows - rb * 32 < 32 ? rows - rb * 32 : 32);     // < 32 in a ragged last block,
+            __half *base = x_hat + rb * (row_elems * 32) + (static_cast<int64_t>(g) * 8 * nrows + r) * 8;   // stored compactly
+            if (r < nrows) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {      // instruction j: piece columns 2j and 2j + 1, 32 rows x 16 bytes each
-                const int kp = j * 2 + (lane >> 5);
-                const uint32_t *src = tile + r * kOutPitch + kp * 4;
-                *reinterpret_cast<uint4 *>(base + kp * (32 * 8)) = make_uint4(src[0], src[1], src[2], src[3]);
+                for (int j = 0; j < 4; ++j) {  // instruction j: piece columns 2j and 2j + 1, nrows x 16 bytes each
+                    const int kp = j * 2 + (lane >> 5);
+                    const uint32_t *src = tile + r * kOutPitch + kp * 4;
+                    *reinterpret_cast<uint4 *>(base + kp * (nrows * 8)) = make_uint4(src[0], src[1], src[2], src[3]);
+                }
             }
         }
         __builtin_amdgcn_wave_barrier();      // the tile is refilled in the next iteration
@@ -594,14 +599,13 @@ static int launch_blocked(const void *x, const float *thr, const float *cb, void
                           int bits, float eps, hipStream_t stream, const WeightJob &wj)
 {
     const int groups_per_row = static_cast<int>(cols / 64);
-    const int row_blocks = static_cast<int>(rows / 32);
-    const int64_t ntiles = static_cast<int64_t>(row_blocks) * groups_per_row;
+    const int64_t ntiles = ((rows + 31) / 32) * groups_per_row;
     const int64_t want = (ntiles + kWaves - 1) / kWaves;
     const unsigned blocks = static_cast<unsigned>(want < 8192 ? want : 8192) + wj.blocks;
 #define ARCQ_LAUNCH_BLOCKED(B)                                                                                  \
     hipLaunchKernelGGL((act_quant_blocked2_kernel<TIN, B>), dim3(blocks), dim3(64 * kWaves), 0, stream,        \
                        static_cast<const TIN *>(x), thr, cb, static_cast<__half *>(x_hat), eps, groups_per_row, \
-                       row_blocks, wj)
+                       rows, wj)
     if (bits == 4) ARCQ_LAUNCH_BLOCKED(4);
     else if (bits == 3) ARCQ_LAUNCH_BLOCKED(3);
     else ARCQ_LAUNCH_BLOCKED(2);
@@ -620,7 +624,6 @@ static int act_quant_blocked_checked(const void *x, int x_dtype, const float *th
     if (!bits_ok(bits)) return fail(ARCQ_ERR_BITS, "arcq_act_quant_blocked: bits must be 2, 3, or 4");
     if (rows < 0 || cols < 0) return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked: bad sizes");
     if (cols % 64 != 0) return fail(ARCQ_ERR_GROUP, "arcq_act_quant_blocked: in_features must be divisible by 64");
-    if (rows % 32 != 0) return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked: rows must be a multiple of 32");
     if (x_dtype != ARCQ_F32 && x_dtype != ARCQ_F16)
         return fail(ARCQ_ERR_DTYPE, "arcq_act_quant_blocked: x must be float32 or float16");
     if (rows * cols == 0 && wj.blocks == 0) return ARCQ_OK;

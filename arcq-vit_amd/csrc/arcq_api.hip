@@ -63,7 +63,7 @@ static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds
             return arcq::launch_status("arcq_linear_otf");
         }
     }
-    // Scratch-only workspaces and whole 32-row blocks: x_hat in the block layout, eight-wave weight-stationary GEMM
+    // Scratch-only workspaces and 512 rows or more: x_hat in the block layout, eight-wave weight-stationary GEMM
     // (bit-identical results; invalid arguments fall through to the entry points below, which report them).
     if (scratch_only && group_size == 64 && arcq::bits_ok(bits) && arcq::otf_blocked_pays(M, N, K) && x != x_hat_ws) {
         // With a weight workspace that pays, its reconstruction rides along in the stage-1 launch.

@@ -353,12 +353,12 @@ ARCQ_API const char *arcq_linear_fused_ws_kernel(int64_t M, int64_t N, int64_t K
 }
 
 // Shapes for which arcq_linear_otf_ws quantizes into the 32-row block layout and multiplies with the eight-wave
-// weight-stationary kernel: whole 32-row blocks from 512 rows on.  Measured against the row-major kernels on the
+// weight-stationary kernel: from 512 rows on.  Measured against the row-major kernels on the
 // twelve DeiT-S / DeiT-B / ViT-L layer shapes it is the fastest on ten and within 3 % (DeiT-B proj, ViT-L fc1) on
 // two.  ARCQ_GEMM_KERNEL pins a row-major kernel, or this one with "slab8" / "prebuilt".
 bool arcq::otf_blocked_pays(int64_t M, int64_t N, int64_t K)
 {
-    if (M < 512 || M % 32 != 0 || N <= 0 || K < 64 || K % 64 != 0 || M * K * 2 >= (int64_t(1) << 32)) return false;
+    if (M < 512 || N <= 0 || K < 64 || K % 64 != 0 || M * K * 2 >= (int64_t(1) << 32)) return false;
     if (M >= (int64_t(1) << 31) - 256 || N >= (int64_t(1) << 31) - 256) return false;
     const char *e = getenv("ARCQ_GEMM_KERNEL");
     if (e) return !strcmp(e, "slab8") || !strcmp(e, "prebuilt");
@@ -408,7 +408,6 @@ int arcq::linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_
     if (group_size != 64) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_fused_blocked: group_size must be 64 (got %d)", group_size);
     if (M < 0 || N < 0 || K < 0) return fail(ARCQ_ERR_SHAPE, "arcq_linear_fused_blocked: negative size");
     if (K % 64 != 0) return fail(ARCQ_ERR_GROUP, "arcq_linear_fused_blocked: in_features must be divisible by group_size");
-    if (M % 32 != 0) return fail(ARCQ_ERR_SHAPE, "arcq_linear_fused_blocked: rows must be a multiple of 32");
     if (y_dtype != ARCQ_F16 && y_dtype != ARCQ_F32)
         return fail(ARCQ_ERR_DTYPE, "arcq_linear_fused_blocked: y must be float16 or float32");
     if (M == 0 || N == 0) return ARCQ_OK;

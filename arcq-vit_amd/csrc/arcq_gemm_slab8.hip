@@ -1,5 +1,6 @@
 // Stages 2+3 fused, weight-stationary kernel for x_hat in the 32-row block layout:
-//   y[M,N] = x_hat[M,K] * w_hat[N,K]^T + bias,   x_hat stored as 16-byte pieces [M/32][K/8][32 rows][8 values].
+//   y[M,N] = x_hat[M,K] * w_hat[N,K]^T + bias,   x_hat stored as 16-byte pieces [M/32][K/8][32 rows][8 values]
+//   (a last block of r < 32 rows as [K/8][r][8]: the tensor takes exactly M*K values).
 //
 // In that layout the MFMA fragment of a 32-row block and k-step (lane = row, 8 consecutive k) is one fully coalesced
 // 16-byte load per lane (512 contiguous bytes per half wave), so x_hat goes from L2 straight into the operand
@@ -98,7 +99,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (tile >= tiles) return;
     const int n_base = (tile % n_slabs) * kSlabN;
-    const int total_blocks = M / 32;
+    const int total_blocks = (M + 31) / 32;
     const int blk0 = (tile / n_slabs) * blocks_per_range;
     const int blk1 = min(total_blocks, blk0 + blocks_per_range);
     // Row blocks of this wave: blk0 + wave, + 8, + 16, ... (one per pass).  Dealing them round-robin instead of in
@@ -179,17 +180,22 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     // x_hat load cursor: the next unit (pass, group) to fetch; it runs two units ahead of the MFMA loop.  A unit is
     // one group of the wave's current 32-row block: four fragments (k-steps) of 16 bytes per lane, 512 contiguous
     // bytes per half wave and k-step.  Past the wave's last block the cursor keeps re-reading a valid block.
+    // A last block of fewer than 32 rows is stored compactly ([K/8][rows][8]): its pieces are `rows` apart instead
+    // of 32, and the lanes past its last row re-read that row (their outputs are not stored).
     int ld_pass = 0, ld_g = 0;
     const char *ld_base;
-    const int lane_off = lh * 2048 + lr * 16;
+    int ld_kstep = 512;                // bytes between the pieces of consecutive k-steps of the current block
     auto set_base = [&](int pass) {
         const int blk = min(blk0 + pass * kWaves + wave, total_blocks - 1);
-        ld_base = reinterpret_cast<const char *>(xb) + static_cast<int64_t>(blk) * K * 64 + lane_off;
+        const int rows = min(32, M - blk * 32);
+        ld_kstep = rows * 16;
+        ld_base = reinterpret_cast<const char *>(xb) + static_cast<int64_t>(blk) * K * 64 + lh * 4 * ld_kstep +
+                  min(lr, rows - 1) * 16;
     };
     auto load_unit = [&](u32x4_t (&r)[4]) {
-        const char *p = ld_base + ld_g * 4096;
+        const char *p = ld_base + ld_g * (8 * ld_kstep);
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) r[kk] = *reinterpret_cast<const u32x4_t *>(p + kk * 512);
+        for (int kk = 0; kk < 4; ++kk) r[kk] = *reinterpret_cast<const u32x4_t *>(p + kk * ld_kstep);
         if (++ld_g == G) {
             ld_g = 0;
             if (ld_pass + 1 < passes) set_base(++ld_pass);
@@ -322,7 +328,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
                     const int cseg = lane & 7;
                     const int row = pblk * 32 + r;
                     const int col = col0 + cseg * kVec;
-                    if (col < N) {
+                    if (row < M && col < N) {
                         const u32x4_t v = *reinterpret_cast<const u32x4_t *>(stage + r * kStageRow + cseg * 16);
                         TOUT *dst = y + static_cast<int64_t>(row) * N + col;
                         if ((N % kVec) == 0 && col + kVec <= N) {
@@ -355,7 +361,7 @@ void launch_slab8_w(const GemmArgs &g, hipStream_t stream, const void *w_hat)
     }
     // One workgroup per CU where possible: split the 32-row blocks into as many ranges as CUs/slabs allow.
     const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
-    const int total_blocks = g.M / 32;
+    const int total_blocks = (g.M + 31) / 32;
     int ranges = 256 / n_slabs;
     if (ranges < 1) ranges = 1;
     if (ranges > total_blocks) ranges = total_blocks;
@@ -379,7 +385,7 @@ void launch_slab8(const GemmArgs &g, hipStream_t stream, const void *w_hat)
 {
     if constexpr (PRE) {
         const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
-        const int total_blocks = g.M / 32;
+        const int total_blocks = (g.M + 31) / 32;
         const int ranges = max(1, min(256 / n_slabs, total_blocks));
         const int64_t units = static_cast<int64_t>((total_blocks + ranges - 1) / ranges) * (g.K / 64);
         if (units >= 256) {
@@ -392,7 +398,7 @@ void launch_slab8(const GemmArgs &g, hipStream_t stream, const void *w_hat)
 
 }  // namespace
 
-// g.x_hat is in the 32-row block layout; g.M must be a positive multiple of 32 and g.K of 64.  w_hat != nullptr:
+// g.x_hat is in the 32-row block layout; g.M must be positive and g.K a positive multiple of 64.  w_hat != nullptr:
 // weights already reconstructed ([N,K] fp16), slab slices are copied from there.
 void launch_gemm_slab8(const GemmArgs &g, const void *w_hat, hipStream_t stream)
 {

@@ -273,7 +273,7 @@ def linear_otf(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Te
 
     With ``scratch=True`` or a ``w_hat_ws`` both workspaces are scratch only: ``y`` is the same bit for bit, but
     ``x_hat_ws`` may afterwards hold ``x_hat`` in the library's 32-row block layout instead of row-major (the
-    faster path for whole 32-row blocks).  Otherwise ``x_hat_ws`` holds ``x_hat`` row-major after the call."""
+    faster path from 512 rows on).  Otherwise ``x_hat_ws`` holds ``x_hat`` row-major after the call."""
     _check(x.is_cuda and packed_w.is_cuda, "x and packed_w must be CUDA tensors")
     _check(x.dim() == 2, "x must have shape [M, K]")
     _check_bits(bits)
@@ -307,7 +307,8 @@ def quantize_activation_blocked(x: torch.Tensor, thresholds: torch.Tensor, codeb
                                 out: Optional[torch.Tensor] = None, weights=None,
                                 w_hat: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Stage 1 (group size 64) with ``x_hat`` written as fp16 in the 32-row block layout
-    ``[M/32, K/8, 32, 8]`` that ``linear_fused_blocked`` reads; same values as ``dequant_activation_hip``.
+    ``[M/32, K/8, 32, 8]`` that ``linear_fused_blocked`` reads (a last block of ``r = M % 32`` rows follows as
+    ``[K/8, r, 8]``); same values as ``dequant_activation_hip``.
 
     ``weights=(packed_w, w_codebook, w_center, w_scale, w_code_sum)`` with ``w_hat`` (fp16, N*K elements): the same
     launch also reconstructs the layer's weights into ``w_hat`` (what ``unpack_weight_hip`` would write)."""
@@ -315,9 +316,10 @@ def quantize_activation_blocked(x: torch.Tensor, thresholds: torch.Tensor, codeb
     _check_bits(bits)
     x = x.contiguous()
     m, k = x.shape
-    _check(m % 32 == 0 and k % 64 == 0, "the block layout needs M divisible by 32 and K by 64")
-    if out is None:
-        out = torch.empty((m // 32, k // 8, 32, 8), dtype=torch.float16, device=x.device)
+    _check(k % 64 == 0, "the block layout needs K divisible by 64")
+    if out is None:      # whole blocks: [M/32, K/8, 32, 8]; a ragged last block is stored compactly behind them: flat
+        shape = (m // 32, k // 8, 32, 8) if m % 32 == 0 else (m * k,)
+        out = torch.empty(shape, dtype=torch.float16, device=x.device)
     else:
         _check(out.is_cuda and out.dtype == torch.float16 and out.is_contiguous() and out.numel() >= m * k,
                "out must be a contiguous float16 CUDA buffer of at least M*K elements")

@@ -158,8 +158,9 @@ const char *arcq_linear_fused_ws_kernel(int64_t M, int64_t N, int64_t K, int hav
  * No counterpart in the reference (its x_hat goes to cuBLAS row-major, FQ/arcq_packed_on_the_fly.py:141-160): these
  * are the two halves arcq_linear_otf_ws is made of when its workspaces are scratch only, exposed so that each can be
  * called, timed and tested on its own.  The layout stores 16-byte pieces of 8 values as
- *     x_hat_blocked[((row / 32) * (K / 8) + k / 8) * 32 + row % 32][k % 8]        (rows a multiple of 32, K of 64),
- * which makes an MFMA operand fragment (32 rows x 8 values) one contiguous 512-byte run.  Values are the ones
+ *     x_hat_blocked[((row / 32) * (K / 8) + k / 8) * 32 + row % 32][k % 8]        (K a multiple of 64),
+ * and a last block of r = rows % 32 rows compactly as [(k / 8) * r + row % 32][k % 8] behind the whole blocks, so the
+ * tensor takes exactly rows * K values.  An MFMA operand fragment (32 rows x 8 values) is one contiguous 512-byte run.  Values are the ones
  * arcq_act_quant writes row-major, bit for bit; arcq_linear_fused_blocked's result equals arcq_linear_fused's on the
  * row-major tensor, bit for bit.  group_size is 64; M * K must stay below 2^31. */
 int arcq_act_quant_blocked(const void *x, int x_dtype, const float *thresholds, const float *codebook,

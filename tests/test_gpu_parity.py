@@ -359,14 +359,20 @@ def test_layer_otf_weight_workspace(cuda, oracle, monkeypatch):
 
 
 def _to_blocked(t):
-    """Row-major [M, K] -> the 32-row block layout [M/32, K/8, 32, 8]."""
+    """Row-major [M, K] -> the 32-row block layout, flat: whole blocks as [M/32, K/8, 32, 8], then a last block of
+    r = M % 32 rows as [K/8, r, 8]."""
     m, k = t.shape
-    return t.reshape(m // 32, 32, k // 8, 8).permute(0, 2, 1, 3).contiguous()
+    full = (m // 32) * 32
+    parts = [t[:full].reshape(m // 32, 32, k // 8, 8).permute(0, 2, 1, 3).reshape(-1)]
+    if full < m:
+        parts.append(t[full:].reshape(m - full, k // 8, 8).permute(1, 0, 2).reshape(-1))
+    return torch.cat(parts).contiguous()
 
 
 @pytest.mark.parametrize("bits", [2, 3, 4])
 @pytest.mark.parametrize("m,k,in_dtype", [(64, 384, torch.float16), (96, 448, torch.float32),    # 7 groups: a half-empty tile
                                           (32, 64, torch.float16),                               # one group per row
+                                          (70, 384, torch.float16), (5, 64, torch.float32),      # a ragged last block
                                           (1024, 1536, torch.float16), (160, 832, torch.float32)])
 def test_stage1_block_layout(cuda, oracle, bits, m, k, in_dtype):
     """arcq_act_quant_blocked writes the values of the row-major stage 1 (and of the oracle), bit for bit, at
@@ -375,14 +381,15 @@ def test_stage1_block_layout(cuda, oracle, bits, m, k, in_dtype):
     x = synth.make_activation(m, k, 43, "gelu").to(in_dtype)
     want = oracle.act_quant_c(x.float().numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)
     got = ops.quantize_activation_blocked(x.to(cuda), thr.to(cuda), cb.to(cuda), bits)
-    assert tuple(got.shape) == (m // 32, k // 8, 32, 8) and got.dtype == torch.float16
+    assert tuple(got.shape) == ((m // 32, k // 8, 32, 8) if m % 32 == 0 else (m * k,)) and got.dtype == torch.float16
+    got = got.reshape(-1)
     assert np.array_equal(_np(got).view(np.uint16), _np(_to_blocked(torch.from_numpy(want))).view(np.uint16))
     if in_dtype == torch.float16:
         assert torch.equal(_to_blocked(ops.dequant_activation_hip(x.to(cuda), thr.to(cuda), cb.to(cuda), 64)), got)
     # a larger out buffer is only written where the layout says
     buf = torch.full((m * k + 64,), -3.0, dtype=torch.float16, device=cuda)
     ops.quantize_activation_blocked(x.to(cuda), thr.to(cuda), cb.to(cuda), bits, out=buf)
-    assert torch.equal(buf[:m * k].view(m // 32, k // 8, 32, 8), got) and bool((buf[m * k:] == -3.0).all())
+    assert torch.equal(buf[:m * k], got) and bool((buf[m * k:] == -3.0).all())
 
 
 @pytest.mark.parametrize("bits,out_dtype", [(4, torch.float16), (3, torch.float32), (2, torch.float16)])
@@ -392,7 +399,8 @@ def test_stage1_block_layout(cuda, oracle, bits, m, k, in_dtype):
                                    (512, 520, 832),       # 13 groups (ring rotation by 1), ragged N
                                    (544, 256, 512),       # 8 groups: last slice of two (ring rotation by 2)
                                    (2112, 1152, 384),     # K in one slice, several passes per wave
-                                   (32, 128, 128)])       # a single row block: seven waves idle
+                                   (1000, 200, 448), (531, 130, 64),      # a ragged last block (8 and 19 rows)
+                                   (32, 128, 128), (7, 64, 128)])         # a single row block: seven waves idle
 def test_fused_gemm_block_layout(cuda, oracle, monkeypatch, bits, out_dtype, m, n, k):
     """arcq_linear_fused_blocked on x_hat in the block layout == arcq_linear_fused on the same x_hat row-major: within
     the fp64 bound, bit-identical to the four-wave weight-stationary kernel (same k order), with and without a weight
@@ -424,7 +432,7 @@ def test_fused_gemm_block_layout(cuda, oracle, monkeypatch, bits, out_dtype, m, 
     # stage 1 with the weight reconstruction carried in its launch, then the GEMM on weights that are ready
     ws2 = torch.full((n * k + 8,), -3.0, dtype=torch.float16, device=cuda)
     xb2 = ops.quantize_activation_blocked(x.to(cuda), thr.to(cuda), cb.to(cuda), bits, weights=w, w_hat=ws2)
-    assert torch.equal(xb2, xb)
+    assert torch.equal(xb2.reshape(-1), xb)
     assert np.array_equal(_np(ws2)[:n * k].view(np.uint16), want_w.reshape(-1).view(np.uint16))
     assert bool((ws2[n * k:] == -3.0).all())
     assert torch.equal(ops.linear_fused_blocked(xb2, m, k, *w, bias, bits, out_dtype=out_dtype, w_hat_ws=ws2,
@@ -434,7 +442,7 @@ def test_fused_gemm_block_layout(cuda, oracle, monkeypatch, bits, out_dtype, m, 
     assert torch.equal(nb + bias, yb)            # the bias is one fp32 addition before the output rounding
 
 
-@pytest.mark.parametrize("m", [1504, 1576])     # whole 32-row blocks (block layout inside) / not (row-major inside)
+@pytest.mark.parametrize("m", [1504, 1576])     # whole 32-row blocks / a last block of 8 rows
 def test_layer_otf_scratch_workspaces(cuda, oracle, monkeypatch, m):
     """arcq_linear_otf_ws (scratch-only workspaces) == arcq_linear_otf bit for bit, whichever layout it uses inside."""
     n, k, bits = 384, 1536, 4
@@ -451,8 +459,7 @@ def test_layer_otf_scratch_workspaces(cuda, oracle, monkeypatch, m):
     assert np.array_equal(_np(xw).view(np.uint16), want_xhat.view(np.uint16))       # row-major without `scratch`
     xs = torch.empty((m, k), dtype=torch.float16, device=cuda)
     assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float16, x_hat_ws=xs, scratch=True), plain)
-    if m % 32 == 0:
-        assert torch.equal(xs.view(m // 32, k // 8, 32, 8), _to_blocked(xw))
+    assert torch.equal(xs.reshape(-1), _to_blocked(xw))        # 512 rows or more: the block layout inside
     ww = torch.zeros(n * k, dtype=torch.float16, device=cuda)
     assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float16, x_hat_ws=xs, w_hat_ws=ww), plain)
     want_w = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, bits, 64, fma=True).astype(np.float16)

@@ -359,7 +359,7 @@ def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
     assert lib.arcq_linear_otf_ws_kernel(12608, 768, 768, 1) == both8                      # two slices, six slabs
     assert lib.arcq_linear_otf_ws_kernel(50432, 4096, 1024, 1) == both8                    # three slices
     assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 1) == both8
-    assert lib.arcq_linear_otf_ws_kernel(1576, 384, 1536, 1) == both                       # 1576 % 32 != 0: row-major
+    assert lib.arcq_linear_otf_ws_kernel(1576, 384, 1536, 1) == both8                      # a ragged last block is fine
     assert lib.arcq_linear_otf_ws_kernel(197, 1152, 384, 1) == b"gemm_splitk_kernel"
     monkeypatch.setenv("ARCQ_GEMM_KERNEL", "stream")
     assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 1) == b"gemm_stream_kernel"
@@ -372,15 +372,14 @@ def test_block_layout_entry_points_validate_before_launching():
     buf = (ctypes.c_char * 256)()
     p = ctypes.addressof(buf) & ~15
     F16 = A._lib.ARCQ_F16
-    assert lib.arcq_act_quant_blocked(p, F16, p, p, p + 64, 33, 64, 4, 1e-6, None) == -4       # rows % 32
-    assert b"multiple of 32" in lib.arcq_last_error()
+    assert lib.arcq_act_quant_blocked(p, F16, p, p, p + 64, -1, 64, 4, 1e-6, None) == -4
     assert lib.arcq_act_quant_blocked(p, F16, p, p, p + 64, 32, 96, 4, 1e-6, None) == -2       # cols % 64
     assert lib.arcq_act_quant_blocked(p, F16, p, p, p + 64, 32, 64, 5, 1e-6, None) == -1       # bits
     assert lib.arcq_act_quant_blocked(p, F16, p, p, None, 32, 64, 4, 1e-6, None) == -3         # NULL output
     assert lib.arcq_act_quant_blocked(p, F16, p, p, p, 32, 64, 4, 1e-6, None) == -6            # in place is not possible
     assert lib.arcq_act_quant_blocked(p, F16, p, p, p + 64, 0, 64, 4, 1e-6, None) == 0         # empty
     args = lambda m, n, k, bits=4, gs=64, ready=0: (p, p, p, p, p, p, None, None, ready, p + 64, F16, m, n, k, bits, gs, None)
-    assert lib.arcq_linear_fused_blocked(*args(33, 8, 64)) == -4
+    assert lib.arcq_linear_fused_blocked(*args(-1, 8, 64)) == -4
     assert lib.arcq_linear_fused_blocked(*args(32, 8, 96)) == -2
     assert lib.arcq_linear_fused_blocked(*args(32, 8, 64, gs=32)) == -6
     assert lib.arcq_linear_fused_blocked(*args(32, 8, 64, bits=1)) == -1
