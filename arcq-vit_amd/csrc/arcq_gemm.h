@@ -24,8 +24,8 @@ void launch_gemm_stream(const GemmArgs &g, hipStream_t stream);
 void launch_gemm_slab(const GemmArgs &g, hipStream_t stream);
 // The same kernel fed from weights reconstructed beforehand into w_hat ([N,K] fp16, 16-byte aligned).
 void launch_gemm_slab_prebuilt(const GemmArgs &g, const void *w_hat, hipStream_t stream);
-// Eight-wave weight-stationary kernel; g.x_hat is in the 32-row block layout ([M/32][K/8][32][8] fp16), g.M a
-// positive, g.K a positive multiple of 64.  w_hat != nullptr: weights already reconstructed ([N,K] fp16).
+// Eight-wave weight-stationary kernel; g.x_hat is in the 32-row block layout ([M/32][K/8][32][8] fp16, a last
+// block of fewer rows stored compactly), g.M positive, g.K a positive multiple of 64.  w_hat != nullptr: weights already reconstructed ([N,K] fp16).
 void launch_gemm_slab8(const GemmArgs &g, const void *w_hat, hipStream_t stream);
 // Whether the whole-layer entry point with scratch-only workspaces runs stage 1 into the block layout and the
 // eight-wave kernel for this shape.
