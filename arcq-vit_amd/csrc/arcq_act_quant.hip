@@ -365,8 +365,8 @@ act_quant_small_kernel(const TIN *__restrict__ x, const float *__restrict__ thr,
 // 1 024 SIMDs leave 158 SIMDs with two tiles (2 x 1 470 instructions), 2 364 half tiles at most three (3 x 740).
 // Data moves through a wave-private LDS tile (rows of the tile = rows of the tensor, odd dword pitch): coalesced
 // 16-byte loads in, every piece column out as one 512-byte run of the block layout.
-template <typename TIN, int BITS>
-__global__ void __launch_bounds__(64 * kWaves)
+template <typename TIN, int BITS, bool BUILDER>
+__global__ void __launch_bounds__(64 * (kWaves + (BUILDER ? 1 : 0)))
 act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ thr, const float *__restrict__ cb,
                           __half *__restrict__ x_hat, float eps, int groups_per_row, int64_t rows, WeightJob wj)
 {
@@ -384,8 +384,23 @@ act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ t
     const int lane = tid & 63;
     const int wave = tid >> 6;
     if (blockIdx.x < wj.blocks) {          // workgroup-uniform: this workgroup rebuilds weights and is done
-        weight_dequant8_block<__half, BITS>(blockIdx.x, lut, wj.packed, wj.cb, wj.center, wj.scale, wj.code_sum, wj.out,
-                                            wj.N, wj.K, 64);
+        if (!BUILDER || wave < kWaves)     // (256 threads per weight block; the fifth wave has nothing to do, and the
+            weight_dequant8_block<__half, BITS, 64 * kWaves>(blockIdx.x, lut, wj.packed, wj.cb, wj.center, wj.scale,
+                                                             wj.code_sum, wj.out, wj.N, wj.K, 64);
+        else                               //  routine's barrier is counted per workgroup: it joins it)
+            __syncthreads();
+        return;
+    }
+    // BUILDER: the workgroup has a fifth wave that owns no tile; it builds the lookup tables while the four tile waves
+    // load their first tile and take its statistics, meets them at the one barrier of the kernel, and is done.  That
+    // takes the table construction (a third of a half tile's instruction chain) off every tile wave's path.  Without
+    // it the four tile waves build the tables together between the two halves of their first tile.
+    float th[L - 1], cbv[L];
+    load_quant_params<BITS>(thr, cb, th, cbv);
+    const BucketScale bq = pick_bucket_scale<BITS>(th);
+    if (BUILDER && wave == kWaves) {
+        build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, lane, 64);
+        __syncthreads();
         return;
     }
     const int64_t wg = blockIdx.x - wj.blocks;
@@ -406,11 +421,7 @@ act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ t
                                                                    : make_uint4(0, 0, 0, 0);
     };
     fetch(wg * kWaves + wave);
-
-    float th[L - 1], cbv[L];
-    load_quant_params<BITS>(thr, cb, th, cbv);
     bool table_ok = false, tables_built = false;
-    BucketScale bq;
     const int row = lane >> 1, half = lane & 1;
 
     for (int64_t tile0 = wg * kWaves; tile0 < ntiles; tile0 += act_blocks * kWaves) {
@@ -442,13 +453,12 @@ act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ t
         }
         float mu, var, s, sum_codes;
         group_stats32x2(xv, eps, mu, var, s);
-        if (!tables_built) {                  // once per workgroup, between the two halves of its first tile
-            bq = pick_bucket_scale<BITS>(th);
-            build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * kWaves);
+        if (!tables_built) {                  // once per workgroup: the builder wave's tables are ready
+            if constexpr (!BUILDER) build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * kWaves);
             __syncthreads();
             table_ok = true;
 #pragma unroll
-            for (int w = 0; w < kWaves; ++w) table_ok = table_ok && (slow_slots[w] == 0);
+            for (int w = 0; w < (BUILDER ? 1 : kWaves); ++w) table_ok = table_ok && (slow_slots[w] == 0);
             tables_built = true;
         }
         group_codes32x2<BITS>(xv, mu, var, s, th, bq, table, lut, table_ok, lane, sum_codes);
@@ -602,10 +612,19 @@ static int launch_blocked(const void *x, const float *thr, const float *cb, void
     const int64_t ntiles = ((rows + 31) / 32) * groups_per_row;
     const int64_t want = (ntiles + kWaves - 1) / kWaves;
     const unsigned blocks = static_cast<unsigned>(want < 8192 ? want : 8192) + wj.blocks;
-#define ARCQ_LAUNCH_BLOCKED(B)                                                                                  \
-    hipLaunchKernelGGL((act_quant_blocked2_kernel<TIN, B>), dim3(blocks), dim3(64 * kWaves), 0, stream,        \
-                       static_cast<const TIN *>(x), thr, cb, static_cast<__half *>(x_hat), eps, groups_per_row, \
-                       rows, wj)
+    // A fifth, table-building wave per workgroup pays while the launch is latency-bound (measured: 5.7 -> 5.3 us for a
+    // few tiles, 11.6 -> 11.2 us for the 2 364 tiles of DeiT-S's K = 384 inputs) and costs occupancy once the chip is
+    // full (ViT-L, 25 216 tiles: 47.6 -> 52.5 us).
+    const bool builder = ntiles <= 4096;
+#define ARCQ_LAUNCH_BLOCKED(B)                                                                                            \
+    do {                                                                                                                  \
+        if (builder)                                                                                                      \
+            hipLaunchKernelGGL((act_quant_blocked2_kernel<TIN, B, true>), dim3(blocks), dim3(64 * (kWaves + 1)), 0, stream, \
+                               static_cast<const TIN *>(x), thr, cb, static_cast<__half *>(x_hat), eps, groups_per_row, rows, wj); \
+        else                                                                                                              \
+            hipLaunchKernelGGL((act_quant_blocked2_kernel<TIN, B, false>), dim3(blocks), dim3(64 * kWaves), 0, stream,   \
+                               static_cast<const TIN *>(x), thr, cb, static_cast<__half *>(x_hat), eps, groups_per_row, rows, wj); \
+    } while (0)
     if (bits == 4) ARCQ_LAUNCH_BLOCKED(4);
     else if (bits == 3) ARCQ_LAUNCH_BLOCKED(3);
     else ARCQ_LAUNCH_BLOCKED(2);

@@ -6,11 +6,12 @@
 
 namespace arcq {
 
-// Work of workgroup number `block` (256 threads) of a launch that reconstructs out[N,K] from packed codes: thread
-// idx = block * 256 + threadIdx.x owns outputs [8 idx, 8 idx + 8) of the flattened tensor.  `lut` is an LDS array of
+// Work of workgroup number `block` (THREADS participating threads, numbered by threadIdx.x) of a launch that
+// reconstructs out[N,K] from packed codes: thread idx = block * THREADS + threadIdx.x owns outputs [8 idx, 8 idx + 8)
+// of the flattened tensor.  `lut` is an LDS array of
 // (1 << BITS) * 64 floats that this call fills with the codebook replicated per lane (conflict-free lookups); every
 // thread of the workgroup must call it (it contains a barrier).
-template <typename TOUT, int BITS>
+template <typename TOUT, int BITS, int THREADS = 256>
 __device__ __forceinline__ void weight_dequant8_block(int64_t block, float *lut, const uint8_t *__restrict__ packed,
                                                       const float *__restrict__ cb, const float *__restrict__ center,
                                                       const float *__restrict__ scale, const float *__restrict__ code_sum,
@@ -25,7 +26,7 @@ __device__ __forceinline__ void weight_dequant8_block(int64_t block, float *lut,
     __syncthreads();
 
     const int64_t chunks_per_row = K / 8;
-    const int64_t idx = block * 256 + threadIdx.x;
+    const int64_t idx = block * THREADS + threadIdx.x;
     if (idx >= N * chunks_per_row) return;
     const int64_t n = idx / chunks_per_row;
     const int64_t k0 = (idx - n * chunks_per_row) * 8;
