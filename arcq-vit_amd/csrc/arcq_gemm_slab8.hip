@@ -112,7 +112,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
 
     // Codes and metadata of one slice: fetched into registers first (for the first slice at the very top of the
     // kernel, so that this latency, the codebook's and the first x_hat units' all overlap), converted afterwards.
-    // Half group number p = round * 512 + tid: consecutive lanes read consecutive pieces of a weight row.
+    // Half group number p = round * threads + tid: consecutive lanes read consecutive pieces of a weight row.
     uint32_t codes[kRounds][BITS];
     float c[kRounds], s[kRounds], m[kRounds];
     auto fetch_slice = [&](int g0) {
