@@ -468,6 +468,30 @@ def test_layer_otf_scratch_workspaces(cuda, oracle, monkeypatch, m):
     assert torch.allclose(y32, plain.float(), rtol=2e-3, atol=2e-3)
 
 
+@pytest.mark.parametrize("m,n,k,bits,out_dtype", [(513, 7, 64, 2, torch.float16),        # one group, N below a vector store
+                                                  (600, 33, 128, 3, torch.float32),
+                                                  (1000, 129, 64, 4, torch.float16),     # second slab one column wide
+                                                  (2048, 40000, 64, 4, torch.float16),   # more slabs than compute units
+                                                  (700, 257, 2560, 3, torch.float32)])   # 40 groups: seven slab slices
+def test_layer_otf_block_layout_odd_shapes(cuda, oracle, monkeypatch, m, n, k, bits, out_dtype):
+    """Whole layer from 512 rows on (block layout, eight-wave GEMM, weights copied or rebuilt in the kernel) against the
+    row-major four-wave kernel on awkward shapes: bit-identical."""
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 61)
+    _, thr = _cb(bits)
+    bias = synth.make_bias(n, 61)
+    x = synth.make_activation(m, k, 61, "ln").to(torch.float16).to(cuda)
+    d = lambda t: t.to(cuda)
+    args = (x, d(thr), d(cb), d(packed), d(cb), d(center), d(scale), d(code_sum), d(bias), bits, 64)
+    monkeypatch.setenv("ARCQ_GEMM_KERNEL", "slab")
+    ref = ops.linear_otf(*args, out_dtype=out_dtype)
+    monkeypatch.delenv("ARCQ_GEMM_KERNEL")
+    ww = torch.empty(n * k, dtype=torch.float16, device=cuda)
+    assert torch.equal(ops.linear_otf(*args, out_dtype=out_dtype, scratch=True), ref)
+    assert torch.equal(ops.linear_otf(*args, out_dtype=out_dtype, w_hat_ws=ww), ref)
+    monkeypatch.setenv("ARCQ_GEMM_KERNEL", "slab8")          # block layout, weights rebuilt inside the GEMM
+    assert torch.equal(ops.linear_otf(*args, out_dtype=out_dtype, w_hat_ws=ww), ref)
+
+
 @pytest.mark.parametrize("bits,in_dtype", [(3, torch.float32), (2, torch.float16)])
 def test_layer_otf_weights_rebuilt_in_stage1_launch(cuda, oracle, monkeypatch, bits, in_dtype):
     """Whole layer in the block layout with a weight workspace (ragged N, seven groups, fp32 / fp16 input): the weights
