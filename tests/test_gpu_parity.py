@@ -167,6 +167,47 @@ def test_stage1_fallback_paths(cuda, oracle):
     check(x, thr, eps=1e-2)
 
 
+def test_stage1_two_lane_fallback_paths(cuda, oracle):
+    """The two-lanes-per-group kernels (small x_hat-only launches, block-layout output) through the same fallbacks:
+    unusable bucket tables and groups outside the guarded range of the fma-based divide; x_hat equals the oracle's."""
+    bits = 4
+    cb, thr = _cb(bits)
+    x = synth.make_activation(70, 128, 9)
+    d = lambda t: t.to(cuda)
+
+    def check(xx, tt):
+        want = oracle.act_quant_c(xx.numpy(), tt, cb, bits, 64)["x_hat"]
+        got = ops.dequant_activation_hip(d(xx), d(tt), d(cb), 64)                   # fp32 in, fp32 out: small kernel
+        assert np.array_equal(_np(got).view(np.uint32), want.view(np.uint32))
+        h = xx.clamp(-6.0e4, 6.0e4).to(torch.float16)      # finite in fp16: an inf group is all NaN, whose bits are free
+        want16 = oracle.act_quant_c(h.float().numpy(), tt, cb, bits, 64)["x_hat"].astype(np.float16)
+        got16 = ops.dequant_activation_hip(d(h), d(tt), d(cb), 64)
+        assert np.array_equal(_np(got16).view(np.uint16), want16.view(np.uint16))
+        blk = ops.quantize_activation_blocked(d(xx), d(tt), d(cb), bits).reshape(-1)   # block layout, fp32 in
+        want_b = oracle.act_quant_c(xx.numpy(), tt, cb, bits, 64)["x_hat"].astype(np.float16)
+        assert np.array_equal(_np(blk).view(np.uint16), _np(_to_blocked(torch.from_numpy(want_b))).view(np.uint16))
+
+    close = thr.clone()
+    close[7] = close[6] + 1e-4
+    check(x, close)
+    unsorted = thr.clone()
+    unsorted[[4, 9]] = unsorted[[9, 4]]
+    check(x, unsorted)
+    far = thr.clone()
+    far[-1] = 9.5
+    check(x, far)
+    tiny = x.clone()
+    tiny[3] *= 1e-30
+    tiny[5] = 0.0
+    check(tiny, thr)
+    huge = x.clone()
+    huge[7] *= 3e18
+    check(huge, thr)
+    const = x.clone()
+    const[11] = 2.5                                   # constant groups: s = sqrt(eps), every t = 0
+    check(const, thr)
+
+
 def test_stage1_empty(cuda):
     cb, thr = _cb(4)
     out = ops.quantize_activation(torch.zeros((0, 128), device=cuda), thr.to(cuda), cb.to(cuda), 4, 64)
