@@ -260,7 +260,7 @@ def test_hip_graph_replay(cuda):
 
 
 # ------------------------------------------------------------------------------------------------
-# full-size, size-independent properties (BASELINE shapes: M = 12608)
+# full-size, size-independent properties (benchmark shapes: M = 12608)
 # ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("bits", [3, 4])
 def test_fullsize_properties(cuda, oracle, bits):
@@ -317,7 +317,7 @@ def test_fullsize_properties(cuda, oracle, bits):
                                         (12608, 1536, 384, 3), (12608, 3072, 768, 4), (12608, 768, 3072, 3),
                                         (50432, 1024, 1024, 3)])
 def test_fullsize_gemm_shapes(cuda, oracle, m, n, k, bits):
-    """The remaining BASELINE layer shapes (DeiT-S proj/fc1/fc2, DeiT-B fc1/fc2, ViT-L proj at batch 256) through
+    """The remaining benchmark layer shapes (DeiT-S proj/fc1/fc2, DeiT-B fc1/fc2, ViT-L proj at batch 256) through
     whichever large-M kernel the dispatcher picks: row permutation and M-split leave rows unchanged (tiles do not
     interact), the result matches a library GEMM on the stage-2 output and, on sampled rows, the fp64 oracle within
     the fp32-accumulation bound."""
