@@ -65,7 +65,9 @@ __device__ __forceinline__ uint32_t code_at(const uint32_t (&w)[BITS], int q)
 // PRE = true: the weights were reconstructed beforehand into a fp16 [N,K] buffer; slab slices are copied,
 // global -> LDS directly, instead of rebuilt.
 // WAVES = 8 or 12 waves per workgroup (two or three per SIMD).
-template <int BITS, typename TOUT, bool PRE, int WAVES>
+// AHEAD = 1 or 2: how many k-steps the LDS reads of the w_hat fragments run ahead of the MFMAs that use them (two
+// where the registers allow it: the LDS round trip under load is longer than one k-step of four MFMAs).
+template <int BITS, typename TOUT, bool PRE, int WAVES, int AHEAD>
 __global__ void __launch_bounds__(64 * WAVES)
 gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw, const float *__restrict__ cb,
                   const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
@@ -216,24 +218,27 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[j][v] = 0.0f;
 
-        // One unit = one group = four k-steps of 4 MFMAs.  Every k-step also issues the LDS reads of the next
-        // k-step's w_hat fragments; k-step 1 fetches the unit two ahead into the ring slot the previous unit used.
-        // `bf[0]` holds the fragments of (gl, k-step 0) on entry and of (gl + 1, k-step 0) on exit.
-        half8_t bf[2][kTJ];
+        // One unit = one group = four k-steps of 4 MFMAs.  Every k-step also issues the LDS reads of the w_hat
+        // fragments needed AHEAD k-steps later; k-step 1 fetches the unit two ahead into the ring slot the previous
+        // unit used.  Slots 0 .. AHEAD - 1 of `bf` hold the fragments of (gl, k-steps 0 .. AHEAD - 1) on entry and of
+        // (gl + 1, the same k-steps) on exit.
+        constexpr int kSlots = 2 * AHEAD;
+        half8_t bf[kSlots][kTJ];
         auto unit = [&](const u32x4_t (&cur_set)[4], u32x4_t (&load_set)[4], int gl) {
             const unsigned char *bsrc = slab_lane + gl * 128;
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
-                const int cur = kk & 1, nxt = cur ^ 1;
+                const int t = kk + AHEAD;           // the k-step whose fragments are read now; t >= 4: of the next group
+                const int off = t < 4 ? t * 16 : 128 + (t - 4) * 16;      // (past the slice on its last unit: unused)
 #pragma unroll
-                for (int j = 0; j < kTJ; ++j)       // kk == 3 reads the next group (past the slice on its last unit: unused)
-                    bf[nxt][j] = *reinterpret_cast<const half8_t *>(bsrc + j * 32 * kPitch + (kk + 1) * 16 + (kk == 3 ? 64 : 0));
+                for (int j = 0; j < kTJ; ++j)
+                    bf[t % kSlots][j] = *reinterpret_cast<const half8_t *>(bsrc + j * 32 * kPitch + off);
                 if (kk == 1) load_unit(load_set);
                 half8_t af;
                 __builtin_memcpy(&af, &cur_set[kk], 16);
 #pragma unroll
                 for (int j = 0; j < kTJ; ++j)
-                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk % kSlots][j], af, acc[j], 0, 0, 0);
 #pragma unroll
                 for (int q = 0; q < kTJ; ++q) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // 1 MFMA
@@ -261,7 +266,10 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
             }
             if (!live) continue;        // (once past its last block a wave stays past it: the ring no longer matters)
 #pragma unroll
-            for (int j = 0; j < kTJ; ++j) bf[0][j] = *reinterpret_cast<const half8_t *>(slab_lane + j * 32 * kPitch);
+            for (int j = 0; j < kTJ; ++j)
+#pragma unroll
+                for (int a = 0; a < AHEAD; ++a)
+                    bf[a][j] = *reinterpret_cast<const half8_t *>(slab_lane + j * 32 * kPitch + a * 16);
             // The ring is walked with fixed register names, three units at a time; every slice but the last has
             // six units, and a last slice that is not a multiple of three rotates the ring back into place.
             for (int gl = 0; gl < ng; gl += 3) {
@@ -294,50 +302,76 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
         constexpr int kBlocksPerChunk = kChunkCols / 32;
         constexpr int kVec = 16 / static_cast<int>(sizeof(TOUT));
         if (live) {
+            // Whole 16-byte pieces everywhere in this slab (wave-uniform): the common case takes no per-piece branch.
+            const bool whole = (N % kVec) == 0 && n_base + kSlabN <= N;
 #pragma unroll
             for (int ch = 0; ch < kChunks; ++ch) {
+                // Bias values first, a batch at a time (the whole chunk with eight waves; one 32-column block with
+                // twelve, which have fewer registers): the compiler cannot tell the bias reads from the staging writes
+                // (both LDS) and would otherwise wait for each read in turn.
+                constexpr int kBiasBatch = WAVES == 8 ? kBlocksPerChunk : 1;
 #pragma unroll
-                for (int jj = 0; jj < kBlocksPerChunk; ++jj) {
-                    const int j = ch * kBlocksPerChunk + jj;
+                for (int jb = 0; jb < kBlocksPerChunk; jb += kBiasBatch) {
+                    float4 bv[kBiasBatch][4];
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int cl = jj * 32 + 8 * q + 4 * lh;            // column inside the chunk
-                        const float4 bv = *reinterpret_cast<const float4 *>(s_bias + j * 32 + 8 * q + 4 * lh);
-                        const float o0 = acc[j][4 * q] + bv.x, o1 = acc[j][4 * q + 1] + bv.y;
-                        const float o2 = acc[j][4 * q + 2] + bv.z, o3 = acc[j][4 * q + 3] + bv.w;
-                        unsigned char *dst = stage + lr * kStageRow + cl * static_cast<int>(sizeof(TOUT));
-                        if constexpr (sizeof(TOUT) == 2) {
-                            const __half2 lo = __floats2half2_rn(o0, o1), hi = __floats2half2_rn(o2, o3);
-                            u32x2_t pk;
-                            pk[0] = *reinterpret_cast<const uint32_t *>(&lo);
-                            pk[1] = *reinterpret_cast<const uint32_t *>(&hi);
-                            *reinterpret_cast<u32x2_t *>(dst) = pk;
-                        } else {
-                            u32x4_t pk;
-                            pk[0] = __float_as_uint(o0); pk[1] = __float_as_uint(o1);
-                            pk[2] = __float_as_uint(o2); pk[3] = __float_as_uint(o3);
-                            *reinterpret_cast<u32x4_t *>(dst) = pk;
+                    for (int jj = 0; jj < kBiasBatch; ++jj)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            bv[jj][q] = *reinterpret_cast<const float4 *>(s_bias + (ch * kBlocksPerChunk + jb + jj) * 32 + 8 * q + 4 * lh);
+#pragma unroll
+                    for (int jj = 0; jj < kBiasBatch; ++jj) {
+                        const int j = ch * kBlocksPerChunk + jb + jj;
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int cl = (jb + jj) * 32 + 8 * q + 4 * lh;            // column inside the chunk
+                            const float o0 = acc[j][4 * q] + bv[jj][q].x, o1 = acc[j][4 * q + 1] + bv[jj][q].y;
+                            const float o2 = acc[j][4 * q + 2] + bv[jj][q].z, o3 = acc[j][4 * q + 3] + bv[jj][q].w;
+                            unsigned char *dst = stage + lr * kStageRow + cl * static_cast<int>(sizeof(TOUT));
+                            if constexpr (sizeof(TOUT) == 2) {
+                                const __half2 lo = __floats2half2_rn(o0, o1), hi = __floats2half2_rn(o2, o3);
+                                u32x2_t pk;
+                                pk[0] = *reinterpret_cast<const uint32_t *>(&lo);
+                                pk[1] = *reinterpret_cast<const uint32_t *>(&hi);
+                                *reinterpret_cast<u32x2_t *>(dst) = pk;
+                            } else {
+                                u32x4_t pk;
+                                pk[0] = __float_as_uint(o0); pk[1] = __float_as_uint(o1);
+                                pk[2] = __float_as_uint(o2); pk[3] = __float_as_uint(o3);
+                                *reinterpret_cast<u32x4_t *>(dst) = pk;
+                            }
                         }
                     }
                 }
                 __builtin_amdgcn_wave_barrier();
-                const int col0 = n_base + ch * kChunkCols;
+                const int col = n_base + ch * kChunkCols + (lane & 7) * kVec;
+                const int row0 = pblk * 32 + (lane >> 3);
+                TOUT *dst0 = y + static_cast<int64_t>(row0) * N + col;
+                constexpr int kStoreBatch = WAVES == 8 ? 4 : 2;       // staged pieces read back before they are stored
 #pragma unroll
-                for (int it = 0; it < 4; ++it) {
-                    const int r = it * 8 + (lane >> 3);
-                    const int cseg = lane & 7;
-                    const int row = pblk * 32 + r;
-                    const int col = col0 + cseg * kVec;
-                    if (row < M && col < N) {
-                        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(stage + r * kStageRow + cseg * 16);
-                        TOUT *dst = y + static_cast<int64_t>(row) * N + col;
-                        if ((N % kVec) == 0 && col + kVec <= N) {
-                            *reinterpret_cast<u32x4_t *>(dst) = v;
-                        } else {
-                            const TOUT *e = reinterpret_cast<const TOUT *>(&v);
+                for (int ib = 0; ib < 4; ib += kStoreBatch) {
+                    u32x4_t v[kStoreBatch];
 #pragma unroll
-                            for (int k = 0; k < kVec; ++k)
-                                if (col + k < N) dst[k] = e[k];
+                    for (int i = 0; i < kStoreBatch; ++i)
+                        v[i] = *reinterpret_cast<const u32x4_t *>(stage + ((ib + i) * 8 + (lane >> 3)) * kStageRow + (lane & 7) * 16);
+                    if (whole) {
+#pragma unroll
+                        for (int i = 0; i < kStoreBatch; ++i)
+                            if (row0 + (ib + i) * 8 < M)
+                                *reinterpret_cast<u32x4_t *>(dst0 + static_cast<int64_t>(ib + i) * 8 * N) = v[i];
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < kStoreBatch; ++i) {
+                            if (row0 + (ib + i) * 8 < M && col < N) {
+                                TOUT *dst = dst0 + static_cast<int64_t>(ib + i) * 8 * N;
+                                if ((N % kVec) == 0 && col + kVec <= N) {
+                                    *reinterpret_cast<u32x4_t *>(dst) = v[i];
+                                } else {
+                                    const TOUT *e = reinterpret_cast<const TOUT *>(&v[i]);
+#pragma unroll
+                                    for (int k = 0; k < kVec; ++k)
+                                        if (col + k < N) dst[k] = e[k];
+                                }
+                            }
                         }
                     }
                 }
@@ -347,12 +381,12 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     }
 }
 
-template <int BITS, typename TOUT, bool PRE, int WAVES>
+template <int BITS, typename TOUT, bool PRE, int WAVES, int AHEAD>
 void launch_slab8_w(const GemmArgs &g, hipStream_t stream, const void *w_hat)
 {
     constexpr int L = 1 << BITS;
     const size_t smem = kSlabBytes + WAVES * kStageTile + L * 64 * sizeof(float) + kSlabN * sizeof(float);
-    auto kernel = gemm_slab8_kernel<BITS, TOUT, PRE, WAVES>;
+    auto kernel = gemm_slab8_kernel<BITS, TOUT, PRE, WAVES, AHEAD>;
     static bool configured = false;   // per instantiation; the attribute is sticky for the process
     if (!configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -389,11 +423,11 @@ void launch_slab8(const GemmArgs &g, hipStream_t stream, const void *w_hat)
         const int ranges = max(1, min(256 / n_slabs, total_blocks));
         const int64_t units = static_cast<int64_t>((total_blocks + ranges - 1) / ranges) * (g.K / 64);
         if (units >= 256) {
-            launch_slab8_w<BITS, TOUT, PRE, 12>(g, stream, w_hat);
+            launch_slab8_w<BITS, TOUT, PRE, 12, 1>(g, stream, w_hat);
             return;
         }
     }
-    launch_slab8_w<BITS, TOUT, PRE, 8>(g, stream, w_hat);
+    launch_slab8_w<BITS, TOUT, PRE, 8, 2>(g, stream, w_hat);
 }
 
 }  // namespace
