@@ -369,7 +369,7 @@ gemm_slab_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, c
                             const u32x4_t v = *reinterpret_cast<const u32x4_t *>(stage + r * kStageRow + cseg * 16);
                             TOUT *dst = y + static_cast<int64_t>(row) * N + col;
                             if ((N % kVec) == 0 && col + kVec <= N) {
-                                *reinterpret_cast<u32x4_t *>(dst) = v;
+                                store_streaming16(dst, v[0], v[1], v[2], v[3]);
                             } else {
                                 const TOUT *e = reinterpret_cast<const TOUT *>(&v);
 #pragma unroll

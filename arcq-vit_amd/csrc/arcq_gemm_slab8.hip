@@ -357,14 +357,14 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
 #pragma unroll
                         for (int i = 0; i < kStoreBatch; ++i)
                             if (row0 + (ib + i) * 8 < M)
-                                *reinterpret_cast<u32x4_t *>(dst0 + static_cast<int64_t>(ib + i) * 8 * N) = v[i];
+                                store_streaming16(dst0 + static_cast<int64_t>(ib + i) * 8 * N, v[i][0], v[i][1], v[i][2], v[i][3]);
                     } else {
 #pragma unroll
                         for (int i = 0; i < kStoreBatch; ++i) {
                             if (row0 + (ib + i) * 8 < M && col < N) {
                                 TOUT *dst = dst0 + static_cast<int64_t>(ib + i) * 8 * N;
                                 if ((N % kVec) == 0 && col + kVec <= N) {
-                                    *reinterpret_cast<u32x4_t *>(dst) = v[i];
+                                    store_streaming16(dst, v[i][0], v[i][1], v[i][2], v[i][3]);
                                 } else {
                                     const TOUT *e = reinterpret_cast<const TOUT *>(&v[i]);
 #pragma unroll
