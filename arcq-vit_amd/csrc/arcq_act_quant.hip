@@ -349,13 +349,13 @@ act_quant_small_kernel(const TIN *__restrict__ x, const float *__restrict__ thr,
                 const __half2 h = __floats2half2_rn(xv[i * 8 + 2 * d], xv[i * 8 + 2 * d + 1]);
                 w[d] = *reinterpret_cast<const uint32_t *>(&h);
             }
-            dst[i] = make_uint4(w[0], w[1], w[2], w[3]);
+            store_writethrough16(dst + i, w[0], w[1], w[2], w[3]);
         }
     } else {
 #pragma unroll
         for (int i = 0; i < kOut; ++i)
-            dst[i] = make_uint4(__float_as_uint(xv[4 * i]), __float_as_uint(xv[4 * i + 1]), __float_as_uint(xv[4 * i + 2]),
-                                __float_as_uint(xv[4 * i + 3]));
+            store_writethrough16(dst + i, __float_as_uint(xv[4 * i]), __float_as_uint(xv[4 * i + 1]),
+                                 __float_as_uint(xv[4 * i + 2]), __float_as_uint(xv[4 * i + 3]));
     }
 }
 
@@ -485,7 +485,7 @@ act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ t
                 for (int j = 0; j < 4; ++j) {  // instruction j: piece columns 2j and 2j + 1, nrows x 16 bytes each
                     const int kp = j * 2 + (lane >> 5);
                     const uint32_t *src = tile + r * kOutPitch + kp * 4;
-                    *reinterpret_cast<uint4 *>(base + kp * (nrows * 8)) = make_uint4(src[0], src[1], src[2], src[3]);
+                    store_writethrough16(base + kp * (nrows * 8), src[0], src[1], src[2], src[3]);
                 }
             }
         }
