@@ -423,10 +423,20 @@ act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ t
     fetch(wg * kWaves + wave);
     bool table_ok = false, tables_built = false;
     const int row = lane >> 1, half = lane & 1;
+    if constexpr (!BUILDER) {
+        // Without a builder wave the four tile waves build the tables first, while their first tile is on its way:
+        // nothing else is live in registers yet (building them between the halves of the first tile, with the tile's
+        // 32 values held, took 169 VGPRs: two waves per SIMD instead of three).
+        build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * kWaves);
+        __syncthreads();
+        table_ok = true;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) table_ok = table_ok && (slow_slots[w] == 0);
+        tables_built = true;
+    }
 
     for (int64_t tile0 = wg * kWaves; tile0 < ntiles; tile0 += act_blocks * kWaves) {
         const int64_t t = tile0 + wave;
-        if (tile0 != wg * kWaves) fetch(t);
         {
             uint32_t *dst = tile + (lane / kPieces) * kInPitch + (lane % kPieces) * 4;
 #pragma unroll
@@ -451,14 +461,12 @@ act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ t
                 }
             }
         }
+        fetch(t + act_blocks * kWaves);       // the wave's next tile (nothing past the end) loads under this one's arithmetic
         float mu, var, s, sum_codes;
         group_stats32x2(xv, eps, mu, var, s);
-        if (!tables_built) {                  // once per workgroup: the builder wave's tables are ready
-            if constexpr (!BUILDER) build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * kWaves);
+        if (BUILDER && !tables_built) {       // once per workgroup: the builder wave's tables are ready
             __syncthreads();
-            table_ok = true;
-#pragma unroll
-            for (int w = 0; w < (BUILDER ? 1 : kWaves); ++w) table_ok = table_ok && (slow_slots[w] == 0);
+            table_ok = (slow_slots[0] == 0);
             tables_built = true;
         }
         group_codes32x2<BITS>(xv, mu, var, s, th, bq, table, lut, table_ok, lane, sum_codes);
@@ -611,11 +619,15 @@ static int launch_blocked(const void *x, const float *thr, const float *cb, void
     const int groups_per_row = static_cast<int>(cols / 64);
     const int64_t ntiles = ((rows + 31) / 32) * groups_per_row;
     const int64_t want = (ntiles + kWaves - 1) / kWaves;
-    const unsigned blocks = static_cast<unsigned>(want < 8192 ? want : 8192) + wj.blocks;
-    // A fifth, table-building wave per workgroup pays while the launch is latency-bound (measured: 5.7 -> 5.3 us for a
-    // few tiles, 11.6 -> 11.2 us for the 2 364 tiles of DeiT-S's K = 384 inputs) and costs occupancy once the chip is
-    // full (ViT-L, 25 216 tiles: 47.6 -> 52.5 us).
-    const bool builder = ntiles <= 4096;
+    // Up to 2 048 tiles (512 workgroups, two per CU) the launch is latency-bound: every wave takes one tile and a fifth
+    // wave per workgroup builds the lookup tables meanwhile (M = 6 304, K = 384: 6.7 us against 7.6 without it).  Beyond
+    // that the grid is what the chip holds at once (1 024 workgroups of four waves, four waves per SIMD), the tables are
+    // built once per workgroup before its first tile, and each wave walks its tiles with the next one's loads in flight
+    // (one workgroup per four tiles, tables rebuilt every time: K = 1 536 at M = 12 608 27-30 us instead of 18-19,
+    // ViT-L's K = 4 096 input 230-258 instead of 171-178).
+    const bool builder = ntiles <= 2048;
+    const int64_t cap = 1024;
+    const unsigned blocks = static_cast<unsigned>(want < cap ? want : cap) + wj.blocks;
 #define ARCQ_LAUNCH_BLOCKED(B)                                                                                            \
     do {                                                                                                                  \
         if (builder)                                                                                                      \
