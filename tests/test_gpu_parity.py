@@ -80,6 +80,13 @@ def test_stage1_bitexact_fp32(cuda, oracle, bits, m, k, kind):
 
 
 @pytest.mark.parametrize("bits", [3, 4])
+def test_stage1_bitexact_large_launch(cuda, oracle, bits):
+    """More 64-group tiles (2 251, the last one a quarter full) than the 512 x 4 waves of the launch: waves walk two
+    tiles, the second prefetched under the first; packed codes, byte codes, metadata and x_hat as the oracle's."""
+    _check_stage1(cuda, oracle, synth.make_activation(9001, 1024, 300 + bits, "gelu"), bits)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
 def test_stage1_fp16_chain_and_inplace(cuda, oracle, bits):
     """fp16 in -> fp16 out, as the on-the-fly layer runs it; fp16 is widened exactly, statistics are
     fp32, x_hat is rounded once to fp16.  In-place (out=x) gives the same bytes."""
