@@ -2,8 +2,8 @@
 //
 // With so few rows a launch cannot fill the chip and its duration is the length of one workgroup's dependent
 // chain: (global load -> dequantize -> MFMA) once per quantization group.  This kernel shortens that chain by
-// splitting K across the waves of a workgroup: a workgroup owns a 32 x 64 or 64 x 64 output tile (32 rows when that
-// still leaves idle compute units), wave w of NW handles the
+// splitting K across the waves of a workgroup: a workgroup owns a 32 x 32, 32 x 64 or 64 x 64 output tile (the
+// smallest that still leaves the grid within the chip), wave w of NW handles the
 // groups g = w, w + NW, w + 2 NW, ... entirely on its own (operands straight from global memory into registers, no
 // barrier inside the loop), and the NW partial tiles are added in LDS in the fixed order w = 0, 1, ..., NW-1, so
 // results do not depend on timing.  Weight reconstruction is the stand-alone stage-2 arithmetic
@@ -25,8 +25,7 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
-constexpr int kSkTile = 64;                    // columns per workgroup (rows: 32 * RB)
-constexpr int kSkPitch = kSkTile * 4 + 16;     // bytes per row of a partial tile in LDS
+// A workgroup's tile is 32 * RB rows x 32 * CB columns; a row of a partial tile in LDS takes 32 * CB * 4 + 16 bytes.
 
 template <int BITS>
 __device__ __forceinline__ void sk_load_codes(const uint8_t *__restrict__ p, uint32_t (&w)[BITS])
@@ -53,14 +52,14 @@ __device__ __forceinline__ uint32_t sk_code_at(const uint32_t (&w)[BITS], int q)
     return v & ((1u << BITS) - 1u);
 }
 
-template <int BITS, int RB>
+template <int BITS, int RB, int CB>
 struct SkOperands {                 // everything one wave needs for one group
     u32x4_t a[RB][4];               // x_hat: RB row blocks x 4 k-steps, 8 halves each
-    uint32_t codes[2][BITS];        // 32 codes of this lane's weight row, per column block
-    float c[2], s[2], m[2];
+    uint32_t codes[CB][BITS];       // 32 codes of this lane's weight row, per column block
+    float c[CB], s[CB], m[CB];
 };
 
-template <int BITS, typename TOUT, int NW, int RB>
+template <int BITS, typename TOUT, int NW, int RB, int CB>
 __global__ void __launch_bounds__(NW * 64)
 gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, const float *__restrict__ cb,
                    const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
@@ -71,6 +70,8 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     float *lut = reinterpret_cast<float *>(smem);                              // [L][64], one copy per lane
     unsigned char *partial = smem + L * 64 * sizeof(float);                    // [NW][RT rows][kSkPitch]
     constexpr int RT = 32 * RB;
+    constexpr int kSkTile = 32 * CB;
+    constexpr int kSkPitch = kSkTile * 4 + 16;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -82,25 +83,25 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     const int64_t pcols = static_cast<int64_t>(K) * BITS / 8;
 
     const __half *a_src[RB];
-    const uint8_t *w_src[2];
-    const float *wc_src[2], *ws_src[2], *wcs_src[2];
+    const uint8_t *w_src[CB];
+    const float *wc_src[CB], *ws_src[CB], *wcs_src[CB];
 #pragma unroll
     for (int i = 0; i < RB; ++i) a_src[i] = a + static_cast<int64_t>(min(m0 + i * 32 + lr, M - 1)) * K + lh * 32;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < CB; ++i) {
         const int n = min(n0 + i * 32 + lr, N - 1);
         w_src[i] = pw + static_cast<int64_t>(n) * pcols + lh * (4 * BITS);
         wc_src[i] = wc + static_cast<int64_t>(n) * G;
         ws_src[i] = ws + static_cast<int64_t>(n) * G;
         wcs_src[i] = wcs + static_cast<int64_t>(n) * G;
     }
-    auto fetch = [&](int g, SkOperands<BITS, RB> &o) {
+    auto fetch = [&](int g, SkOperands<BITS, RB, CB> &o) {
 #pragma unroll
         for (int i = 0; i < RB; ++i)
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) o.a[i][kk] = *reinterpret_cast<const u32x4_t *>(a_src[i] + g * 64 + kk * 8);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < CB; ++i) {
             sk_load_codes<BITS>(w_src[i] + g * (8 * BITS), o.codes[i]);
             o.c[i] = wc_src[i][g];
             o.s[i] = ws_src[i][g];
@@ -108,7 +109,7 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
         }
     };
 
-    SkOperands<BITS, RB> o0, o1;
+    SkOperands<BITS, RB, CB> o0, o1;
     if (wave < G) fetch(wave, o0);             // in flight while the codebook is staged
     if (tid < 64) {
 #pragma unroll
@@ -116,30 +117,30 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     }
     __syncthreads();
 
-    float16_t acc[RB][2];
+    float16_t acc[RB][CB];
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < CB; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
     const char *lut_lane = reinterpret_cast<const char *>(lut) + lane * 4;
-    auto compute = [&](const SkOperands<BITS, RB> &o) {
-        float mg[2];
+    auto compute = [&](const SkOperands<BITS, RB, CB> &o) {
+        float mg[CB];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) mg[j] = o.m[j] * 0.015625f;        // S/64, exact
-        float wv[2][32];          // all 64 table lookups are issued before the first is used
+        for (int j = 0; j < CB; ++j) mg[j] = o.m[j] * 0.015625f;       // S/64, exact
+        float wv[CB][32];         // all table lookups are issued before the first is used
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < CB; ++j)
 #pragma unroll
             for (int q = 0; q < 32; ++q)
                 wv[j][q] = *reinterpret_cast<const float *>(lut_lane + (sk_code_at<BITS>(o.codes[j], q) << 8));
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
-            half8_t bf[2];
+            half8_t bf[CB];
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < CB; ++j)
 #pragma unroll
                 for (int q = 0; q < 8; ++q)
                     bf[j][q] = static_cast<_Float16>(fma_f32(wv[j][kk * 8 + q] - mg[j], o.s[j], o.c[j]));
@@ -148,7 +149,7 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
                 half8_t af;
                 __builtin_memcpy(&af, &o.a[i][kk], 16);
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < CB; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af, acc[i][j], 0, 0, 0);
             }
         }
@@ -170,7 +171,7 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < CB; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 f32x4_t v;
@@ -187,20 +188,25 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     const int waves_used = min(NW, G);                     // the others hold zeros; skipping them changes nothing
     for (int w = 0; w < waves_used; ++w) {
         const unsigned char *src = partial + w * (RT * kSkPitch) + row * kSkPitch + col * 4;
+        if constexpr (E % 4 == 0) {
 #pragma unroll
-        for (int e = 0; e < E; e += 4) {
-            const f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + e * 4);
-            sum[e] += v[0]; sum[e + 1] += v[1]; sum[e + 2] += v[2]; sum[e + 3] += v[3];
+            for (int e = 0; e < E; e += 4) {
+                const f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + e * 4);
+                sum[e] += v[0]; sum[e + 1] += v[1]; sum[e + 2] += v[2]; sum[e + 3] += v[3];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) sum[e] += *reinterpret_cast<const float *>(src + e * 4);
         }
     }
     const int gr = m0 + row, gc = n0 + col;
     if (gr < M && gc < N) {
         TOUT *dst = y + static_cast<int64_t>(gr) * N + gc;
-        if (gc + E <= N && (N % E) == 0) {
+        constexpr int BYTES = E * static_cast<int>(sizeof(TOUT));
+        if (gc + E <= N && (N % E) == 0 && BYTES % 8 == 0) {
             TOUT out[E];
 #pragma unroll
             for (int e = 0; e < E; ++e) out[e] = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
-            constexpr int BYTES = E * static_cast<int>(sizeof(TOUT));
             if constexpr (BYTES % 16 == 0) {
 #pragma unroll
                 for (int b = 0; b < BYTES; b += 16)
@@ -217,14 +223,16 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     }
 }
 
-template <int BITS, typename TOUT, int RB>
+template <int BITS, typename TOUT, int RB, int CB>
 static void launch_splitk_rb(const GemmArgs &g, hipStream_t stream)
 {
     constexpr int NW = 8;
     constexpr int L = 1 << BITS;
     constexpr int RT = 32 * RB;
+    constexpr int kSkTile = 32 * CB;
+    constexpr int kSkPitch = kSkTile * 4 + 16;
     const size_t smem = L * 64 * sizeof(float) + static_cast<size_t>(NW) * RT * kSkPitch;
-    auto kernel = gemm_splitk_kernel<BITS, TOUT, NW, RB>;
+    auto kernel = gemm_splitk_kernel<BITS, TOUT, NW, RB, CB>;
     static bool configured = false;   // per instantiation; the attribute is sticky for the process
     if (!configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -241,9 +249,15 @@ static void launch_splitk_t(const GemmArgs &g, hipStream_t stream)
 {
     // 32-row tiles while the grid still fits the chip: more workgroups in flight and half the row-strided x_hat
     // loads per wave; 64-row tiles otherwise (the weights are then rebuilt half as often).
-    const int64_t tiles32 = static_cast<int64_t>((g.N + kSkTile - 1) / kSkTile) * ((g.M + 31) / 32);
-    if (tiles32 <= 256) launch_splitk_rb<BITS, TOUT, 1>(g, stream);
-    else launch_splitk_rb<BITS, TOUT, 2>(g, stream);
+    // 32 x 32 tiles while the grid stays within about one and a half workgroups per CU: a wave then rebuilds 32 weight
+    // rows per group instead of 64 and the chain a launch this small waits for is a third shorter (M = 197:
+    // 384 x 1536 11.9 -> 8.0 us, 384 x 384 5.0 -> 3.8, 1024 x 1024 10.0 -> 6.9; 1536 x 384, 336 tiles, 5.2 -> 4.8;
+    // equal at 504 tiles, slower beyond).  Same k order per output: bit-identical.
+    const int64_t tiles32 = static_cast<int64_t>((g.N + 63) / 64) * ((g.M + 31) / 32);
+    const int64_t tiles32x32 = static_cast<int64_t>((g.N + 31) / 32) * ((g.M + 31) / 32);
+    if (tiles32x32 <= 400) launch_splitk_rb<BITS, TOUT, 1, 1>(g, stream);
+    else if (tiles32 <= 256) launch_splitk_rb<BITS, TOUT, 1, 2>(g, stream);
+    else launch_splitk_rb<BITS, TOUT, 2, 2>(g, stream);
 }
 
 void launch_gemm_splitk(const GemmArgs &g, hipStream_t stream)
