@@ -2,7 +2,7 @@
 // (FQ/arcq_packed_on_the_fly.py:137-161 end to end).
 //
 // At batch 1 every kernel of the layer costs about as much as an empty launch, so the number of launches is
-// what matters.  A workgroup owns a tile of RT rows x 64 output columns.  It first quantizes the activations
+// what matters.  A workgroup owns a tile of RT rows x 32 or 64 output columns.  It first quantizes the activations
 // of its RT rows (all K/64 groups; one group per lane, the same arithmetic as the stand-alone stage-1 kernel,
 // arcq_act_quant_core.h) and keeps x_hat as fp16 in LDS; the column tiles of a row tile repeat that work, on
 // compute units that would otherwise idle.  Then it runs the split-K product of gemm_splitk_kernel: wave w
@@ -21,8 +21,8 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kOsWaves = 8;
-constexpr int kOsCols = 64;                    // output columns per workgroup
-constexpr int kOsRedPitch = kOsCols * 4 + 16;  // bytes per row of a partial tile
+// Output columns per workgroup: 32 * CB (CB = 1 or 2); a row of a partial tile takes 32 * CB * 4 + 16 bytes.
+__host__ __device__ constexpr int os_red_pitch(int cb) { return 32 * cb * 4 + 16; }
 constexpr int kOsGroupPitch = 144;             // bytes per group of an x_hat row in LDS (128 + 16 pad)
 
 __host__ __device__ inline int os_row_pitch(int G) { return G * kOsGroupPitch + 16; }
@@ -52,10 +52,10 @@ __device__ __forceinline__ uint32_t os_code_at(const uint32_t (&w)[BITS], int q)
     return v & ((1u << BITS) - 1u);
 }
 
-template <int BITS>
+template <int BITS, int CB>
 struct OsWeights {                  // what one wave needs of the weights for one group
-    uint32_t codes[2][BITS];        // 32 codes of this lane's weight row, per 32-column block
-    float c[2], s[2], m[2];
+    uint32_t codes[CB][BITS];       // 32 codes of this lane's weight row, per 32-column block
+    float c[CB], s[CB], m[CB];
 };
 
 // The lane's E consecutive inputs (a whole group, or half of one when two lanes share a group): raw 16-byte loads
@@ -92,7 +92,7 @@ __device__ __forceinline__ void os_convert_group(const OsGroupRegs<TIN, E> &r, f
 }
 
 // RB = 32-row blocks per workgroup tile (1 or 2); LPG = lanes per quantization group in stage 1 (1 or 2).
-template <typename TIN, int BITS, typename TOUT, int RB, int LPG>
+template <typename TIN, int BITS, typename TOUT, int RB, int LPG, int CB>
 __global__ void __launch_bounds__(kOsWaves * 64)
 otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, const float *__restrict__ a_cb,
                  const uint8_t *__restrict__ pw, const float *__restrict__ w_cb,
@@ -102,6 +102,8 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
 {
     constexpr int L = 1 << BITS;
     constexpr int RT = 32 * RB;
+    constexpr int kOsCols = 32 * CB;
+    constexpr int kOsRedPitch = os_red_pitch(CB);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     // [x_hat tile | partial tiles] [activation LUT] [weight LUT] [buckets] [per-wave flags]; the partial tiles of
     // the reduction follow the x_hat tile (partial_off == tile_bytes) or, when K is too long for both, reuse its space
@@ -125,26 +127,26 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     const int64_t pcols = static_cast<int64_t>(K) * BITS / 8;
 
     // ---- weights of this wave's first group: requested now, used after stage 1 ---------------------------
-    const uint8_t *w_src[2];
-    const float *wc_src[2], *ws_src[2], *wcs_src[2];
+    const uint8_t *w_src[CB];
+    const float *wc_src[CB], *ws_src[CB], *wcs_src[CB];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < CB; ++j) {
         const int n = min(n0 + j * 32 + lr, N - 1);
         w_src[j] = pw + static_cast<int64_t>(n) * pcols + lh * (4 * BITS);
         wc_src[j] = wc + static_cast<int64_t>(n) * G;
         ws_src[j] = ws + static_cast<int64_t>(n) * G;
         wcs_src[j] = wcs + static_cast<int64_t>(n) * G;
     }
-    auto fetch_w = [&](int g, OsWeights<BITS> &o) {
+    auto fetch_w = [&](int g, OsWeights<BITS, CB> &o) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < CB; ++j) {
             os_load_codes<BITS>(w_src[j] + g * (8 * BITS), o.codes[j]);
             o.c[j] = wc_src[j][g];
             o.s[j] = ws_src[j][g];
             o.m[j] = wcs_src[j][g];
         }
     };
-    OsWeights<BITS> o0, o1;
+    OsWeights<BITS, CB> o0, o1;
     if (wave < G) fetch_w(wave, o0);
 
     // ---- stage 1: x_hat of the RT rows into LDS -----------------------------------------------------------
@@ -236,32 +238,32 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     __syncthreads();
 
     // ---- stages 2+3: split-K product, wave w takes groups w, w+8, ... --------------------------------------
-    float16_t acc[RB][2];
+    float16_t acc[RB][CB];
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < CB; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
     const char *lut_lane = reinterpret_cast<const char *>(w_lut) + lane * 4;
     const unsigned char *a_lane = xt + lr * row_pitch + lh * 64;
-    auto compute = [&](int g, const OsWeights<BITS> &o) {
-        float mg[2];
+    auto compute = [&](int g, const OsWeights<BITS, CB> &o) {
+        float mg[CB];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) mg[j] = o.m[j] * 0.015625f;        // S/64, exact
+        for (int j = 0; j < CB; ++j) mg[j] = o.m[j] * 0.015625f;       // S/64, exact
         const unsigned char *a_g = a_lane + g * kOsGroupPitch;
-        float wv[2][32];          // all 64 table lookups are issued before the first is used
+        float wv[CB][32];         // all table lookups are issued before the first is used
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < CB; ++j)
 #pragma unroll
             for (int q = 0; q < 32; ++q)
                 wv[j][q] = *reinterpret_cast<const float *>(lut_lane + (os_code_at<BITS>(o.codes[j], q) << 8));
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
-            half8_t bf[2];
+            half8_t bf[CB];
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < CB; ++j)
 #pragma unroll
                 for (int q = 0; q < 8; ++q)
                     bf[j][q] = static_cast<_Float16>(fma_f32(wv[j][kk * 8 + q] - mg[j], o.s[j], o.c[j]));
@@ -269,7 +271,7 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
             for (int i = 0; i < RB; ++i) {
                 const half8_t af = *reinterpret_cast<const half8_t *>(a_g + i * 32 * row_pitch + kk * 16);
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < CB; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af, acc[i][j], 0, 0, 0);
             }
         }
@@ -288,7 +290,7 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < CB; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 f32x4_t v;
@@ -296,7 +298,7 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
                 *reinterpret_cast<f32x4_t *>(mine + (i * 32 + lr) * kOsRedPitch + (j * 32 + 8 * q + 4 * lh) * 4) = v;
             }
     __syncthreads();
-    constexpr int E = RT * kOsCols / (kOsWaves * 64);      // outputs per thread, consecutive in a row (8 or 4)
+    constexpr int E = RT * kOsCols / (kOsWaves * 64);      // outputs per thread, consecutive in a row (8, 4 or 2)
     constexpr int TPR = kOsCols / E;
     const int row = tid / TPR, col = (tid % TPR) * E;
     float sum[E];
@@ -305,10 +307,15 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     const int waves_used = min(kOsWaves, G);
     for (int w = 0; w < waves_used; ++w) {
         const unsigned char *src = partial + w * (RT * kOsRedPitch) + row * kOsRedPitch + col * 4;
+        if constexpr (E % 4 == 0) {
 #pragma unroll
-        for (int e = 0; e < E; e += 4) {
-            const f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + e * 4);
-            sum[e] += v[0]; sum[e + 1] += v[1]; sum[e + 2] += v[2]; sum[e + 3] += v[3];
+            for (int e = 0; e < E; e += 4) {
+                const f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + e * 4);
+                sum[e] += v[0]; sum[e + 1] += v[1]; sum[e + 2] += v[2]; sum[e + 3] += v[3];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) sum[e] += *reinterpret_cast<const float *>(src + e * 4);
         }
     }
     const int gr = m0 + row, gc = n0 + col;
@@ -335,11 +342,13 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     }
 }
 
-template <typename TIN, int BITS, typename TOUT, int RB, int LPG>
+template <typename TIN, int BITS, typename TOUT, int RB, int LPG, int CB>
 static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
 {
     constexpr int L = 1 << BITS;
     constexpr int RT = 32 * RB;
+    constexpr int kOsCols = 32 * CB;
+    constexpr int kOsRedPitch = os_red_pitch(CB);
     const int G = a.K / 64;
     const int xhat_bytes = RT * os_row_pitch(G);
     const int partial_bytes = kOsWaves * RT * kOsRedPitch;
@@ -348,7 +357,7 @@ static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
     // Both regions side by side while they fit 160 KB of LDS; else the partial tiles reuse the x_hat tile's space.
     const int partial_off = (tile_bytes + partial_bytes + tables <= 160 * 1024) ? tile_bytes : 0;
     const size_t smem = (partial_off ? tile_bytes + partial_bytes : (tile_bytes > partial_bytes ? tile_bytes : partial_bytes)) + tables;
-    auto kernel = otf_small_kernel<TIN, BITS, TOUT, RB, LPG>;
+    auto kernel = otf_small_kernel<TIN, BITS, TOUT, RB, LPG, CB>;
     static int configured = 0;        // per instantiation: largest dynamic LDS size requested so far
     if (static_cast<int>(smem) > configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -365,8 +374,17 @@ template <typename TIN, int BITS, typename TOUT>
 static void launch_os_rb(const OtfSmallArgs &a, hipStream_t stream)
 {
     // Two lanes per group while the 32-row tile is at most eight 32-group tiles: half the chain, no extra round.
-    if (32 * (a.K / 64) <= 8 * 32) launch_os<TIN, BITS, TOUT, 1, 2>(a, stream);
-    else launch_os<TIN, BITS, TOUT, 1, 1>(a, stream);
+    // 32-column tiles while their grid fits the chip in one wave of workgroups: half the weight rows to rebuild per wave
+    // and half the reduction, at the price of twice as many workgroups repeating stage 1 (M = 197, K = 384:
+    // N = 1152, 252 tiles, 8.9 -> 8.0 us; N = 384 8.7 -> 7.6; N = 1536, 336 tiles, 8.7-9.4 -> 10.0).  Bit-identical.
+    const bool narrow = static_cast<int64_t>((a.N + 31) / 32) * ((a.M + 31) / 32) <= 256;
+    if (32 * (a.K / 64) <= 8 * 32) {
+        if (narrow) launch_os<TIN, BITS, TOUT, 1, 2, 1>(a, stream);
+        else launch_os<TIN, BITS, TOUT, 1, 2, 2>(a, stream);
+    } else {
+        if (narrow) launch_os<TIN, BITS, TOUT, 1, 1, 1>(a, stream);
+        else launch_os<TIN, BITS, TOUT, 1, 1, 2>(a, stream);
+    }
 }
 
 template <typename TIN, typename TOUT>
@@ -386,7 +404,7 @@ bool otf_small_supported(int64_t M, int64_t N, int64_t K, bool any_supported)
 {
     if (!(M < 512 && K >= 64 && K % 64 == 0 && K <= 1536)) return false;
     if (any_supported || K <= 512) return true;
-    return K <= 768 && ((N + kOsCols - 1) / kOsCols) * ((M + 31) / 32) <= 256;
+    return K <= 768 && ((N + 63) / 64) * ((M + 31) / 32) <= 256;
 }
 
 void launch_otf_small(const OtfSmallArgs &a, hipStream_t stream)
