@@ -425,6 +425,7 @@ def _to_blocked(t):
                                           (2752, 1536, torch.float16),     # 2 064 tiles: no builder wave, one tile per wave
                                           (6000, 1536, torch.float16),     # 4 512 tiles on 1 024 workgroups: waves walk 1-2 tiles, ragged end
                                           (4500, 1024, torch.float32),     # fp32 input without the builder wave
+                                          (9001, 1024, torch.float32),     # fp32 input, waves walk 1-2 tiles, ragged end
                                           (12608, 1536, torch.float16)])   # the benchmark's largest stage 1: 2-3 tiles per wave
 def test_stage1_block_layout(cuda, oracle, bits, m, k, in_dtype):
     """arcq_act_quant_blocked writes the values of the row-major stage 1 (and of the oracle), bit for bit, at
