@@ -306,6 +306,9 @@ act_quant_small_kernel(const TIN *__restrict__ x, const float *__restrict__ thr,
     float th[L - 1], cbv[L];
     load_quant_params<BITS>(thr, cb, th, cbv);
     const BucketScale bq = pick_bucket_scale<BITS>(th);
+    // The tables are built while the inputs are still on their way: their latency and the build's overlap (-0.2 us).
+    build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * kWaves);
+    __syncthreads();
 
     float xv[32];
     if constexpr (sizeof(TIN) == 2) {
@@ -327,8 +330,6 @@ act_quant_small_kernel(const TIN *__restrict__ x, const float *__restrict__ thr,
     }
     float mu, var, s, sum_codes;
     group_stats32x2(xv, eps, mu, var, s);
-    build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * kWaves);
-    __syncthreads();
     bool table_ok = true;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) table_ok = table_ok && (slow_slots[w] == 0);
