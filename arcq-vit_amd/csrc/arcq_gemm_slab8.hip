@@ -20,6 +20,10 @@
 
 #include <type_traits>
 
+#ifndef ARCQ_SPLIT_DEFAULT
+#define ARCQ_SPLIT_DEFAULT 1
+#endif
+
 namespace arcq {
 namespace {
 
@@ -76,6 +80,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
 {
     constexpr int L = 1 << BITS;
     constexpr int kWaves = WAVES;
+    constexpr bool SPLIT = ARCQ_SPLIT_DEFAULT && WAVES == 8;     // left-over blocks are dealt in halves
     constexpr int kThreads = 64 * WAVES;
     constexpr int kStageBytes = kWaves * kStageTile;
     constexpr int kRounds = kSlabN * kHalves / kThreads;       // half groups per thread and slice
@@ -117,7 +122,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     // Half group number p = round * threads + tid: consecutive lanes read consecutive pieces of a weight row.
     uint32_t codes[kRounds][BITS];
     float c[kRounds], s[kRounds], m[kRounds];
-    auto fetch_slice = [&](int g0) {
+    auto fetch_slice = [&](int g0) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < kRounds; ++r) {
             const int p = r * kThreads + tid;
@@ -141,7 +146,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     if (tid < kSlabN) s_bias[tid] = (bias && n_base + tid < N) ? bias[n_base + tid] : 0.0f;
     // PRE: one direct global -> LDS load per slab row (lanes 0..47 carry the row's 48 16-byte pieces, the hardware
     // writes lane l's piece at the wave-uniform LDS base + 16 l); the caller waits for vmcnt and the barrier.
-    auto copy_slice = [&](int g0, int ng) {
+    auto copy_slice = [&](int g0, int ng) __attribute__((always_inline)) {
         const bool active = lane < 8 * ng;
         for (int row = wave; row < kSlabN; row += kWaves) {
             const int n = min(n_base + row, N - 1);
@@ -151,7 +156,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
                     (__attribute__((address_space(3))) void *)(slab + row * kPitch), 16, 0, 0);
         }
     };
-    auto dequant_slice = [&](int ng) {
+    auto dequant_slice = [&](int ng) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < kRounds; ++r) {
             const int p = r * kThreads + tid;
@@ -187,8 +192,34 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     int ld_pass = 0, ld_g = 0;
     const char *ld_base;
     int ld_kstep = 512;                // bytes between the pieces of consecutive k-steps of the current block
+    // Blocks of a pass.  A full pass gives every wave one block (32 rows x the slab's 128 columns).  A pass with fewer
+    // blocks than waves (the last one of a workgroup) splits as many blocks as there are spare waves into two halves
+    // of 64 columns: waves 0 .. W-1 take whole blocks, the pairs after them one block each.  A half keeps the k order
+    // of every output it computes, so results do not depend on how a block was dealt.  In a workgroup of one pass
+    // this always pays (5 blocks on 8 waves: the busiest SIMD multiplies 9 units per slice instead of 12; proj / fc2
+    // of DeiT-S 9.2 -> 8.4 and 25.3 -> 22.7 us); after full passes only while at most two blocks are split (10 blocks:
+    // 12.6 -> 11.8 us; with three or four, six or eight waves fetch the same x_hat at once: 19 blocks 19.3 -> 21.0).
+    auto assign = [&](int pass, int &blk, int &jb, int &nj) {
+        const int base = blk0 + pass * kWaves;
+        const int nb = min(kWaves, blk1 - base);
+        int S = (SPLIT && nb > 0) ? min(nb, kWaves - nb) : 0;
+        if (passes > 1 && S > 2) S = 0;          // (measured: see launch_slab8)
+        const int W = nb - S;
+        if (wave < W || !SPLIT) {
+            blk = base + wave;
+            jb = 0;
+            nj = kTJ;
+        } else {
+            const int i = (wave - W) >> 1;
+            blk = i < S ? base + W + i : blk1;
+            jb = ((wave - W) & 1) * (kTJ / 2);
+            nj = kTJ / 2;
+        }
+    };
     auto set_base = [&](int pass) {
-        const int blk = min(blk0 + pass * kWaves + wave, total_blocks - 1);
+        int ablk, ajb, anj;
+        assign(pass, ablk, ajb, anj);
+        const int blk = min(ablk, total_blocks - 1);
         const int rows = min(32, M - blk * 32);
         ld_kstep = rows * 16;
         ld_base = reinterpret_cast<const char *>(xb) + static_cast<int64_t>(blk) * K * 64 + lh * 4 * ld_kstep +
@@ -209,12 +240,14 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     load_unit(r0);
     load_unit(r1);
 
-    for (int pass = 0; pass < passes; ++pass) {
-        const int pblk = blk0 + pass * kWaves + wave;
-        const bool live = pblk < blk1;           // a wave past its last block only keeps the barriers company
-        float16_t acc[kTJ];
+    // One pass of one wave over NJ of the slab's four 32-column tiles, starting at tile jb.  Every wave of the
+    // workgroup runs this once per pass, whatever its NJ: the barriers inside are the same in every instantiation.
+    auto run_pass = [&](auto njc, const int pass, const int pblk, const int jb, const bool live) __attribute__((always_inline)) {
+        constexpr int NJ = decltype(njc)::value;
+        const unsigned char *slab_wave = slab_lane + jb * 32 * kPitch;
+        float16_t acc[NJ];
 #pragma unroll
-        for (int j = 0; j < kTJ; ++j)
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[j][v] = 0.0f;
 
@@ -223,24 +256,24 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
         // unit used.  Slots 0 .. AHEAD - 1 of `bf` hold the fragments of (gl, k-steps 0 .. AHEAD - 1) on entry and of
         // (gl + 1, the same k-steps) on exit.
         constexpr int kSlots = 2 * AHEAD;
-        half8_t bf[kSlots][kTJ];
+        half8_t bf[kSlots][NJ];
         auto unit = [&](const u32x4_t (&cur_set)[4], u32x4_t (&load_set)[4], int gl) {
-            const unsigned char *bsrc = slab_lane + gl * 128;
+            const unsigned char *bsrc = slab_wave + gl * 128;
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
                 const int t = kk + AHEAD;           // the k-step whose fragments are read now; t >= 4: of the next group
                 const int off = t < 4 ? t * 16 : 128 + (t - 4) * 16;      // (past the slice on its last unit: unused)
 #pragma unroll
-                for (int j = 0; j < kTJ; ++j)
+                for (int j = 0; j < NJ; ++j)
                     bf[t % kSlots][j] = *reinterpret_cast<const half8_t *>(bsrc + j * 32 * kPitch + off);
                 if (kk == 1) load_unit(load_set);
                 half8_t af;
                 __builtin_memcpy(&af, &cur_set[kk], 16);
 #pragma unroll
-                for (int j = 0; j < kTJ; ++j)
+                for (int j = 0; j < NJ; ++j)
                     acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk % kSlots][j], af, acc[j], 0, 0, 0);
 #pragma unroll
-                for (int q = 0; q < kTJ; ++q) {
+                for (int q = 0; q < NJ; ++q) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // 1 MFMA
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 // 1 LDS read
                     if (kk == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // 1 global load
@@ -266,10 +299,10 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
             }
             if (!live) continue;        // (once past its last block a wave stays past it: the ring no longer matters)
 #pragma unroll
-            for (int j = 0; j < kTJ; ++j)
+            for (int j = 0; j < NJ; ++j)
 #pragma unroll
                 for (int a = 0; a < AHEAD; ++a)
-                    bf[a][j] = *reinterpret_cast<const half8_t *>(slab_lane + j * 32 * kPitch + a * 16);
+                    bf[a][j] = *reinterpret_cast<const half8_t *>(slab_wave + j * 32 * kPitch + a * 16);
             // The ring is walked with fixed register names, three units at a time; every slice but the last has
             // six units, and a last slice that is not a multiple of three rotates the ring back into place.
             for (int gl = 0; gl < ng; gl += 3) {
@@ -298,7 +331,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
         // ---- epilogue of this pass: the 32 x 128 block leaves in chunks of 128 bytes per row through the wave's
         // private staging tile (LDS operations of one wave execute in order: no wait is needed between them) ----
         constexpr int kChunkCols = 128 / static_cast<int>(sizeof(TOUT));     // 64 (fp16) / 32 (fp32)
-        constexpr int kChunks = kSlabN / kChunkCols;
+        constexpr int kChunks = NJ * 32 / kChunkCols;
         constexpr int kBlocksPerChunk = kChunkCols / 32;
         constexpr int kVec = 16 / static_cast<int>(sizeof(TOUT));
         if (live) {
@@ -311,19 +344,19 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
                 // (both LDS) and would otherwise wait for each read in turn.
                 constexpr int kBiasBatch = WAVES == 8 ? kBlocksPerChunk : 1;
 #pragma unroll
-                for (int jb = 0; jb < kBlocksPerChunk; jb += kBiasBatch) {
+                for (int cb = 0; cb < kBlocksPerChunk; cb += kBiasBatch) {
                     float4 bv[kBiasBatch][4];
 #pragma unroll
                     for (int jj = 0; jj < kBiasBatch; ++jj)
 #pragma unroll
                         for (int q = 0; q < 4; ++q)
-                            bv[jj][q] = *reinterpret_cast<const float4 *>(s_bias + (ch * kBlocksPerChunk + jb + jj) * 32 + 8 * q + 4 * lh);
+                            bv[jj][q] = *reinterpret_cast<const float4 *>(s_bias + (jb + ch * kBlocksPerChunk + cb + jj) * 32 + 8 * q + 4 * lh);
 #pragma unroll
                     for (int jj = 0; jj < kBiasBatch; ++jj) {
-                        const int j = ch * kBlocksPerChunk + jb + jj;
+                        const int j = ch * kBlocksPerChunk + cb + jj;
 #pragma unroll
                         for (int q = 0; q < 4; ++q) {
-                            const int cl = (jb + jj) * 32 + 8 * q + 4 * lh;            // column inside the chunk
+                            const int cl = (cb + jj) * 32 + 8 * q + 4 * lh;            // column inside the chunk
                             const float o0 = acc[j][4 * q] + bv[jj][q].x, o1 = acc[j][4 * q + 1] + bv[jj][q].y;
                             const float o2 = acc[j][4 * q + 2] + bv[jj][q].z, o3 = acc[j][4 * q + 3] + bv[jj][q].w;
                             unsigned char *dst = stage + lr * kStageRow + cl * static_cast<int>(sizeof(TOUT));
@@ -343,7 +376,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
                     }
                 }
                 __builtin_amdgcn_wave_barrier();
-                const int col = n_base + ch * kChunkCols + (lane & 7) * kVec;
+                const int col = n_base + jb * 32 + ch * kChunkCols + (lane & 7) * kVec;
                 const int row0 = pblk * 32 + (lane >> 3);
                 TOUT *dst0 = y + static_cast<int64_t>(row0) * N + col;
                 constexpr int kStoreBatch = WAVES == 8 ? 4 : 2;       // staged pieces read back before they are stored
@@ -378,6 +411,14 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
                 __builtin_amdgcn_wave_barrier();
             }
         }
+    };
+
+    for (int pass = 0; pass < passes; ++pass) {
+        int pblk, jb, nj;
+        assign(pass, pblk, jb, nj);
+        const bool live = pblk < blk1;           // a wave without a block only keeps the barriers company
+        if (!SPLIT || nj == kTJ) run_pass(std::integral_constant<int, kTJ>{}, pass, pblk, jb, live);
+        else run_pass(std::integral_constant<int, kTJ / 2>{}, pass, pblk, jb, live);
     }
 }
 
