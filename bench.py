@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch of each fused-GEMM kernel at the default workload (average over the layer shapes it serves),
 # from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a plain 256 MiB
 # copy (factors 2.00 and 1.00).  Summary: profiles/deit_small_w4a4_bs64_packed_linears.md.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): {"gemm_slab8_kernel<copy>": 48.2e6}}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): {"gemm_slab8_kernel<copy>": 48.1e6}}
 
 
 def parse_args():
