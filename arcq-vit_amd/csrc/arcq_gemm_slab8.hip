@@ -80,7 +80,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
 {
     constexpr int L = 1 << BITS;
     constexpr int kWaves = WAVES;
-    constexpr bool SPLIT = ARCQ_SPLIT_DEFAULT && WAVES == 8;     // left-over blocks are dealt in halves
+    constexpr bool SPLIT = ARCQ_SPLIT_DEFAULT;                   // left-over blocks are dealt in halves
     constexpr int kThreads = 64 * WAVES;
     constexpr int kStageBytes = kWaves * kStageTile;
     constexpr int kRounds = kSlabN * kHalves / kThreads;       // half groups per thread and slice
