@@ -20,11 +20,12 @@ from .packed_convert import (  # noqa: F401
     convert_arcq_linear_to_packed,
     count_packed_linear,
     load_packed_state_dict,
+    share_buffers,
     to_on_the_fly,
 )
 from .packed_fast_linear import ARCQPackedLinearFast  # noqa: F401
 from .packed_linear import ARCQPackedLinear, _quantize_weight_reference, infer_packed_hparams  # noqa: F401
-from .packed_on_the_fly import ARCQPackedLinearOnTheFly  # noqa: F401
+from .packed_on_the_fly import ARCQPackedLinearOnTheFly, clear_workspaces  # noqa: F401
 from .quant_source import FrozenARCQQuantizer, QuantLinearPCARCQ  # noqa: F401
 
 __all__ = [
@@ -33,5 +34,5 @@ __all__ = [
     "unpack_weight_hip", "linear_fused", "linear_otf", "pack_codes_py", "unpack_codes_py",
     "ARCQPackedLinear", "ARCQPackedLinearOnTheFly", "ARCQPackedLinearFast", "QuantLinearPCARCQ",
     "FrozenARCQQuantizer", "convert_arcq_linear_to_packed", "count_packed_linear", "to_on_the_fly",
-    "load_packed_state_dict", "infer_packed_hparams",
+    "load_packed_state_dict", "infer_packed_hparams", "share_buffers", "clear_workspaces",
 ]

@@ -47,6 +47,27 @@ def to_on_the_fly(model: nn.Module) -> nn.Module:
     return model
 
 
+def share_buffers(model: nn.Module, max_rows: int = 0) -> nn.Module:
+    """Give every on-the-fly layer of ``model`` (already on its device) the two scratch buffers its forward uses,
+    shared by all layers: ``_weight_buffer``, one flat fp16 tensor for the largest ``out_features * in_features``
+    (what scripts/benchmark_arcq_on_the_fly.py:182-191 sets up), and, when ``max_rows`` is given, ``_x_hat_buffer``
+    for ``max_rows`` tokens of the widest input (so that forwards allocate nothing and the buffer's lifetime is
+    the model's).  Layers run one after another on a stream, which makes the sharing safe."""
+    layers = [m for m in model.modules() if isinstance(m, ARCQPackedLinearOnTheFly)]
+    if not layers:
+        return model
+    dev = layers[0].packed_weight_codes.device
+    w = torch.zeros(max(m.out_features * m.in_features for m in layers), dtype=torch.float16, device=dev)
+    xh = None
+    if max_rows > 0:
+        xh = torch.zeros(int(max_rows) * max(m.in_features for m in layers), dtype=torch.float16, device=dev)
+    for m in layers:
+        m._weight_buffer = w
+        if xh is not None:
+            m._x_hat_buffer = xh
+    return model
+
+
 def packed_layer_prefixes(state_dict: Dict[str, torch.Tensor]) -> List[str]:
     """Prefixes (with trailing dot) of all packed layers in a flat state dict."""
     tail = "packed_weight_codes"

@@ -22,12 +22,17 @@ import torch.nn as nn
 
 from . import ops
 
-# One reusable fp16 x_hat workspace per (device, stream): layers run back to back on a stream, and
-# stream order makes the reuse safe.  Grown on demand, never shrunk.
+# Fallback fp16 x_hat workspace, one per (device, stream), for layers that were given no ``_x_hat_buffer``: layers
+# run back to back on a stream, and stream order makes the reuse safe.  Grown on demand; ``clear_workspaces()``
+# releases them.  Never used while a HIP graph is being captured: memory allocated during a capture belongs to
+# that graph's private pool, so a capture gets a buffer of its own (kept alive by the graph's pool) instead of
+# leaving one in this cache for a later capture to find.
 _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
 def _workspace(device: torch.device, numel: int) -> torch.Tensor:
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(max(numel, 1), dtype=torch.float16, device=device)
     key = (device.index if device.index is not None else torch.cuda.current_device(),
            torch.cuda.current_stream(device).cuda_stream)
     ws = _workspaces.get(key)
@@ -35,6 +40,11 @@ def _workspace(device: torch.device, numel: int) -> torch.Tensor:
         ws = torch.empty(max(numel, 1), dtype=torch.float16, device=device)
         _workspaces[key] = ws
     return ws
+
+
+def clear_workspaces() -> None:
+    """Drop the fallback x_hat workspaces (they are re-created on demand)."""
+    _workspaces.clear()
 
 
 class ARCQPackedLinearOnTheFly(nn.Module):
@@ -105,7 +115,9 @@ class ARCQPackedLinearOnTheFly(nn.Module):
         if x2.dtype not in (torch.float16, torch.float32):
             x2 = x2.to(torch.float16)
         x2 = x2.contiguous()
-        ws = _workspace(x2.device, x2.numel())
+        ws = getattr(self, "_x_hat_buffer", None)       # a buffer the model owns (packed_convert.share_buffers)
+        if ws is None or ws.numel() < x2.numel() or ws.device != x2.device:
+            ws = _workspace(x2.device, x2.numel())
         bias = self.bias_tensor if self.bias_tensor.numel() > 0 else None
         w_ws = getattr(self, "_weight_buffer", None)
         if w_ws is not None and (not w_ws.is_cuda or w_ws.dtype != torch.float16 or not w_ws.is_contiguous()

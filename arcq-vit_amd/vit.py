@@ -14,7 +14,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .packed_convert import convert_arcq_linear_to_packed, to_on_the_fly
+from .packed_convert import convert_arcq_linear_to_packed, share_buffers, to_on_the_fly
 from .quant_source import QuantLinearPCARCQ
 from .synth import MODEL_DIMS, SEED, quantile_codebook
 
@@ -93,10 +93,13 @@ class VisionTransformer(nn.Module):
 
 
 def build_fakequant_vit(model: str, bits: int, group_size: int = 64, seed: int = SEED,
-                        num_classes: int = 1000) -> VisionTransformer:
+                        num_classes: int = 1000, depth: Optional[int] = None) -> VisionTransformer:
     """Random-init ViT whose block linears are ``QuantLinearPCARCQ`` with quantile codebooks
-    (weights N(0, 0.02^2), as timm's trunc_normal_(std=.02) init; biases N(0, 0.01^2))."""
-    cfg = MODEL_DIMS[model]
+    (weights N(0, 0.02^2), as timm's trunc_normal_(std=.02) init; biases N(0, 0.01^2)).
+    ``depth`` overrides the model's number of blocks (a shallower model of the same widths)."""
+    cfg = dict(MODEL_DIMS[model])
+    if depth is not None:
+        cfg["depth"] = int(depth)
     cb = quantile_codebook(bits)
 
     def make(i: int, o: int, b: bool) -> nn.Module:
@@ -118,14 +121,18 @@ def build_fakequant_vit(model: str, bits: int, group_size: int = 64, seed: int =
 
 
 def build_packed_vit(model: str, bits: int, group_size: int = 64, seed: int = SEED, num_classes: int = 1000,
-                     device: str = "cuda", half_chain: bool = True) -> VisionTransformer:
+                     device: str = "cuda", half_chain: bool = True, depth: Optional[int] = None,
+                     shared_buffers: bool = False, max_rows: int = 0) -> VisionTransformer:
     """Fake-quant ViT -> packed (``convert_arcq_linear_to_packed``) -> on-the-fly layers -> device,
     the sequence of scripts/benchmark_arcq_on_the_fly.py:88-199.  ``half_chain`` casts the
-    floating-point rest of the model to fp16 (packed metadata stays fp32)."""
-    vit = build_fakequant_vit(model, bits, group_size, seed, num_classes)
+    floating-point rest of the model to fp16 (packed metadata stays fp32).  ``shared_buffers`` gives all
+    layers one weight scratch buffer (:182-191 there) and, with ``max_rows`` tokens, one x_hat buffer."""
+    vit = build_fakequant_vit(model, bits, group_size, seed, num_classes, depth)
     convert_arcq_linear_to_packed(vit, runtime_code_format="packed")
     to_on_the_fly(vit)
     vit = vit.to(device)
     if half_chain:
         vit = vit.half()
+    if shared_buffers:
+        share_buffers(vit, max_rows)
     return vit.eval()
