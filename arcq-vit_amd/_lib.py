@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libarcq_hip.so")
 
 ARCQ_F32 = 0
 ARCQ_F16 = 1
+ARCQ_STATIC_SCRATCH_BYTES = 40 * 1024 * 1024
 
 _c_i64 = ctypes.c_int64
 _c_int = ctypes.c_int
@@ -37,6 +38,8 @@ _SIGNATURES = {
                              _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
     "arcq_linear_otf_ws": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                            _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
+    "arcq_linear_otf_static": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                               _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
     "arcq_act_quant_blocked": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32, _c_ptr],
     "arcq_act_quant_blocked_with_weights": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32,
                                             _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr],

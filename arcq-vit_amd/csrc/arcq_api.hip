@@ -5,6 +5,8 @@
 
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "arcq_common.h"
 #include "arcq_gemm.h"
 
@@ -104,4 +106,60 @@ ARCQ_API int arcq_linear_otf_ws(const void *x, int x_dtype, const float *a_thres
 {
     return linear_otf_impl(x, x_dtype, a_thresholds, a_codebook, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias,
                            x_hat_ws, w_hat_ws, true, y, y_dtype, M, N, K, bits, group_size, stream);
+}
+
+// ---- the same layer for callers that cannot allocate --------------------------------------------------------
+// Both scratch buffers of arcq_linear_otf_ws live in a file-scope device array instead of caller memory.  Every GPU
+// the library runs on holds its own copy of the array (at its own address) until the process ends.
+static __device__ __align__(256) unsigned char scratch[ARCQ_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+unsigned char *g_scratch_ptr[kMaxDevices];        // device address of `scratch` on each device, once resolved
+}
+
+ARCQ_API int arcq_linear_otf_static(const void *x, int x_dtype, const float *a_thresholds, const float *a_codebook,
+                                    const uint8_t *packed_w, const float *w_codebook,
+                                    const float *w_center, const float *w_scale, const float *w_code_sum,
+                                    const float *bias, void *y, int y_dtype,
+                                    int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
+{
+    if (M < 0 || N < 0 || K < 0) return arcq::fail(ARCQ_ERR_SHAPE, "arcq_linear_otf_static: negative size");
+    // Layout of the array: [w_hat: N*K fp16, rounded up to 256 bytes][x_hat: M*K fp16].
+    const int64_t limit = ARCQ_STATIC_SCRATCH_BYTES;
+    if (K > limit || N > limit || M > limit)
+        return arcq::fail(ARCQ_ERR_SHAPE, "arcq_linear_otf_static: sizes exceed the static scratch of %lld bytes",
+                          static_cast<long long>(limit));
+    const int64_t w_bytes = (N * K * 2 + 255) / 256 * 256;
+    const int64_t x_bytes = M * K * 2;
+    if (w_bytes + x_bytes > limit)
+        return arcq::fail(ARCQ_ERR_SHAPE,
+                          "arcq_linear_otf_static: 2*N*K + 2*M*K = %lld bytes of scratch needed, the static scratch holds "
+                          "%lld; use arcq_linear_otf_ws with caller-owned workspaces",
+                          static_cast<long long>(w_bytes + x_bytes), static_cast<long long>(limit));
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return arcq::fail(static_cast<int>(e), "arcq_linear_otf_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices)
+        return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_static: device index %d not supported", dev);
+    unsigned char *base;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (!g_scratch_ptr[dev]) {
+            // In host code the array's name is only a handle: its device address has to be asked for, once per
+            // device, with that device current.
+            void *p = nullptr;
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !p)
+                return arcq::fail(e != hipSuccess ? static_cast<int>(e) : ARCQ_ERR_NULL,
+                                  "arcq_linear_otf_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+            g_scratch_ptr[dev] = static_cast<unsigned char *>(p);
+        }
+        base = g_scratch_ptr[dev];
+    }
+    // Nothing in the array has to start at zero: stage 1 writes every x_hat value and the weight reconstruction every
+    // w_hat value before the GEMM reads them.
+    return linear_otf_impl(x, x_dtype, a_thresholds, a_codebook, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias,
+                           base + w_bytes, base, true, y, y_dtype, M, N, K, bits, group_size, stream);
 }

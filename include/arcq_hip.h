@@ -181,6 +181,21 @@ int arcq_linear_fused_blocked(const void *x_hat_blocked,
                               const float *bias, void *w_hat_ws, int w_hat_ready, void *y, int y_dtype,
                               int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
 
+/* arcq_linear_otf_ws for callers that cannot allocate device memory or lend workspaces (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The two
+ * scratch buffers come from a static device array of ARCQ_STATIC_SCRATCH_BYTES inside the library, of which every GPU
+ * the library runs on holds its own copy until the process ends; the call itself allocates and frees nothing.  It
+ * needs 2*N*K (rounded up to 256) + 2*M*K bytes of it and returns ARCQ_ERR_SHAPE beyond that (the limit covers every
+ * DeiT-Small layer at batch 64).  y equals arcq_linear_otf_ws's bit for bit.  All calls on one GPU share that GPU's
+ * array: calls that overlap on one GPU (different streams, or threads) race; calls on one stream are ordered.  The
+ * first call on a device looks up the array's address; make it outside a graph capture. */
+#define ARCQ_STATIC_SCRATCH_BYTES (40 * 1024 * 1024)
+int arcq_linear_otf_static(const void *x, int x_dtype, const float *a_thresholds, const float *a_codebook,
+                           const uint8_t *packed_w, const float *w_codebook,
+                           const float *w_center, const float *w_scale, const float *w_code_sum,
+                           const float *bias, void *y, int y_dtype,
+                           int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
+
 /* Kernels arcq_linear_otf_ws runs after stage 1 for these sizes: "gemm_slab8_kernel", or "gemm_slab8_kernel<copy>"
  * (weights rebuilt in the stage-1 launch, copied by the GEMM), when it takes the block layout, else
  * arcq_linear_fused_ws_kernel's answer.  A profiling aid with no counterpart in the reference. */
