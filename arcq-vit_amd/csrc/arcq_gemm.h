@@ -27,6 +27,10 @@ void launch_gemm_slab_prebuilt(const GemmArgs &g, const void *w_hat, hipStream_t
 // Eight-wave weight-stationary kernel; g.x_hat is in the 32-row block layout ([M/32][K/8][32][8] fp16, a last
 // block of fewer rows stored compactly), g.M positive, g.K a positive multiple of 64.  w_hat != nullptr: weights already reconstructed ([N,K] fp16).
 void launch_gemm_slab8(const GemmArgs &g, const void *w_hat, hipStream_t stream);
+// The same with two row blocks per wave and pass (wave tile 64 x 128); weights must be reconstructed already.
+void launch_gemm_pair(const GemmArgs &g, const void *w_hat, hipStream_t stream);
+// Whether launch_gemm_pair is the kernel of choice for this shape.
+bool gemm_pair_pays(const GemmArgs &g);
 // Whether the whole-layer entry point with scratch-only workspaces runs stage 1 into the block layout and the
 // eight-wave kernel for this shape.
 bool otf_blocked_pays(int64_t M, int64_t N, int64_t K);

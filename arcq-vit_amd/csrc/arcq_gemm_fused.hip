@@ -367,8 +367,13 @@ bool arcq::otf_blocked_pays(int64_t M, int64_t N, int64_t K)
 
 ARCQ_API const char *arcq_linear_otf_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace)
 {
-    if (otf_blocked_pays(M, N, K))
-        return (have_workspace && blocked_uses_workspace(N, K)) ? "gemm_slab8_kernel<copy>" : "gemm_slab8_kernel";
+    if (otf_blocked_pays(M, N, K)) {
+        if (!(have_workspace && blocked_uses_workspace(N, K))) return "gemm_slab8_kernel";
+        GemmArgs g{};
+        g.M = static_cast<int>(M), g.N = static_cast<int>(N), g.K = static_cast<int>(K);
+        const char *e = getenv("ARCQ_PAIR");
+        return (e ? e[0] == '1' : gemm_pair_pays(g)) ? "gemm_pair_kernel" : "gemm_slab8_kernel<copy>";
+    }
     return arcq_linear_fused_ws_kernel(M, N, K, have_workspace);
 }
 

@@ -1,0 +1,352 @@
+// Stages 2+3 on weights reconstructed beforehand, x_hat in the 32-row block layout: the eight-wave weight-stationary
+// kernel with TWO row blocks per wave and pass (wave tile 64 rows x 128 columns = 2 x 4 MFMA blocks).
+//
+//   y[M,N] = x_hat[M,K] * w_hat[N,K]^T + bias,   x_hat as 16-byte pieces [M/32][K/8][32 rows][8 values]
+//   (a last block of r < 32 rows as [K/8][r][8]),  w_hat [N,K] fp16 row-major.
+//
+// Operand budget of a CU per MFMA time (32 clocks, four SIMDs): LDS delivers 4 KB, the vector memory path 2 KB.  With
+// one row block per wave every w_hat fragment read from LDS (1 KB) feeds a single MFMA, i.e. the LDS runs at its limit;
+// with two row blocks it feeds two, and an x_hat fragment (from L2, one coalesced 16-byte load per lane) still feeds
+// four.  The pass structure, slab slices copied global -> LDS, k order inside a group and operand roles are those of
+// gemm_slab8_kernel, so results are bit-identical to it (every output accumulates its k-steps in the same order).
+//
+// x_hat fragments live in eight 16-byte slots per lane (k-step x row block): the slot of k-step kk is refilled with
+// the next group's k-step kk right after the MFMAs that consumed it, so every load has four k-steps (32 MFMAs) to
+// arrive.  Left-over blocks of a workgroup (fewer than sixteen) are dealt as pairs, single blocks and column halves.
+#include "arcq_common.h"
+#include "arcq_gemm.h"
+
+#include <stdlib.h>
+#include <type_traits>
+
+namespace arcq {
+namespace {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kSlabN = 128;                 // columns per slab
+constexpr int kTJ = kSlabN / 32;            // 4 column blocks
+constexpr int kStageRow = 144;              // bytes per staged output row: 128 + 16 pad
+constexpr int kStageTile = 32 * kStageRow;  // 4608 B per wave
+
+// WAVES waves per workgroup and SG groups per K slice of the slab.  (8, 6) is one workgroup per CU.  (Two workgroups of
+// four waves per CU with three-group slices, 70 KB of LDS each, so that one multiplies while the other copies a slice
+// or writes a block out, measured 35-45 % slower on every shape: 466 against 342 us at 50 432 x 3 072 x 1 024.)
+template <int WAVES, int SG> struct PairCfg {
+    static constexpr int kPieces = SG * 8 + 1;            // 16-byte pieces per slab row, one of them padding
+    static constexpr int kPitch = kPieces * 16;           // (conflict-free 16-byte fragment reads)
+    static constexpr int kSlabBytes = kSlabN * kPitch;
+    static constexpr int kSmem = kSlabBytes + WAVES * kStageTile + kSlabN * static_cast<int>(sizeof(float)) + 64;
+};
+
+template <typename TOUT, int WAVES, int SG>
+__global__ void __launch_bounds__(64 * WAVES)
+gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K,
+                 int row_ranges, int blocks_per_range, const __half *__restrict__ w_hat)
+{
+    constexpr int kWaves = WAVES;
+    constexpr int kSliceGroups = SG;
+    constexpr int kPieces = PairCfg<WAVES, SG>::kPieces;
+    constexpr int kPitch = PairCfg<WAVES, SG>::kPitch;
+    constexpr int kSlabBytes = PairCfg<WAVES, SG>::kSlabBytes;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    unsigned char *slab = smem;
+    float *s_bias = reinterpret_cast<float *>(smem + kSlabBytes + kWaves * kStageTile);      // [128]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int lr = lane & 31;
+    const int lh = lane >> 5;
+    const int G = K / 64;
+
+    // Tile = (row range, slab), slab fastest; each XCD (workgroups are dealt to the 8 XCDs round-robin) takes a
+    // contiguous run of tiles so that the slabs sharing a row range read x_hat through one L2.
+    const int n_slabs = (N + kSlabN - 1) / kSlabN;
+    const int tiles = n_slabs * row_ranges;
+    const int per_xcd = (tiles + 7) / 8;
+    const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (tile >= tiles) return;
+    const int n_base = (tile % n_slabs) * kSlabN;
+    const int total_blocks = (M + 31) / 32;
+    const int blk0 = (tile / n_slabs) * blocks_per_range;
+    const int blk1 = min(total_blocks, blk0 + blocks_per_range);
+    const int nblk = blk1 - blk0;
+    const int full_passes = nblk / (2 * kWaves);       // every wave multiplies a pair of blocks
+    const int rest = nblk - full_passes * 2 * kWaves;  // 0 .. 15 blocks for one more pass
+    const int passes = full_passes + (rest > 0 ? 1 : 0);
+    const int slices = (G + kSliceGroups - 1) / kSliceGroups;
+
+    const unsigned char *slab_lane = slab + lr * kPitch + lh * 64;
+    unsigned char *stage = smem + kSlabBytes + wave * kStageTile;
+
+    if (tid < kSlabN) s_bias[tid] = (bias && n_base + tid < N) ? bias[n_base + tid] : 0.0f;
+    // Direct global -> LDS loads: the slab is filled as one flat run of 16-byte pieces (piece p = row * kPieces +
+    // column; the hardware writes lane l's piece at the wave-uniform LDS base + 16 l), 64 pieces per instruction
+    // whatever the row length; padding pieces and the columns past a short last slice are skipped.  The caller
+    // waits for vmcnt and the barrier.
+    auto copy_slice = [&](int g0, int ng) __attribute__((always_inline)) {
+        for (int p0 = wave * 64; p0 < kSlabN * kPieces; p0 += kWaves * 64) {
+            const int p = p0 + lane;
+            const int row = p / kPieces, col = p - row * kPieces;
+            const int n = min(n_base + row, N - 1);
+            if (col < 8 * ng && row < kSlabN)
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void *)(w_hat + static_cast<int64_t>(n) * K + g0 * 64 + col * 8),
+                    (__attribute__((address_space(3))) void *)(slab + p0 * 16), 16, 0, 0);
+        }
+    };
+
+    // One pass of one wave: NB row blocks (first block b0) times NJ of the slab's four 32-column tiles, from tile jb.
+    // Every wave of the workgroup runs this once per pass, whatever its NB and NJ: the barriers are the same in every
+    // instantiation.  live == false: the wave has no block in this pass and only keeps the barriers company.
+    auto run_pass = [&](auto nbc, auto njc, const int pass, const int b0, const int jb, const bool live) __attribute__((always_inline)) {
+        constexpr int NB = decltype(nbc)::value;
+        constexpr int NJ = decltype(njc)::value;
+        const unsigned char *slab_wave = slab_lane + jb * 32 * kPitch;
+        float16_t acc[NB][NJ];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[nb][j][v] = 0.0f;
+
+        // x_hat fragments: lane (lr, lh) reads, for k-step kk of group g, piece 8 g + 4 lh + kk of row lr of its block
+        // (k = 64 g + 32 lh + 8 kk ... + 7).  A last block of fewer than 32 rows is stored compactly: its pieces are
+        // `rows` apart instead of 32, and the lanes past its last row re-read that row (their outputs are not stored).
+        const char *xbase[NB];
+        int kstep[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int blk = min(b0 + nb, total_blocks - 1);
+            const int rows = min(32, M - blk * 32);
+            kstep[nb] = rows * 16;
+            xbase[nb] = reinterpret_cast<const char *>(xb) + static_cast<int64_t>(blk) * K * 64 + lh * 4 * kstep[nb] +
+                        min(lr, rows - 1) * 16;
+        }
+        // The first group's fragments, requested in the order in which the loop below refills the slots (the scheduling
+        // barriers pin it).  The compiler's wait-count bookkeeping merges this state with the loop's own at the top of
+        // the group loop and waits for the stricter of the two: with the loads in any other order here (left alone it
+        // reverses them) that is vmcnt(0) in every iteration, i.e. no load is ever left in flight across a group.
+        u32x4_t xs[4][NB];
+        if (live) {
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                    xs[kk][nb] = *reinterpret_cast<const u32x4_t *>(xbase[nb] + kk * kstep[nb]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+        }
+
+        for (int sl = 0; sl < slices; ++sl) {
+            const int g0 = sl * kSliceGroups;
+            const int ng = min(kSliceGroups, G - g0);
+            if (!(slices == 1 && pass > 0)) {
+                __syncthreads();      // every wave is done reading the previous slice
+                copy_slice(g0, ng);
+                __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the slice has landed in LDS
+                asm volatile("" ::: "memory");
+                __syncthreads();
+            }
+            if (!live) continue;
+            half8_t bf[2][NJ];
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) bf[0][j] = *reinterpret_cast<const half8_t *>(slab_wave + j * 32 * kPitch);
+            for (int gl = 0; gl < ng; ++gl) {
+                // The group whose fragments the slots are refilled with: the next one, or (past the last) the last one
+                // again -- lines this wave has just read, so those loads hit L1 and nobody waits for them.
+                const int gn = min(g0 + gl + 1, G - 1);
+                const unsigned char *bsrc = slab_wave + gl * 128;
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk) {
+                    // w_hat fragments of the next k-step (of the next group after the fourth; past the slice after
+                    // its last one: read and never used)
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j)
+                        bf[(kk + 1) & 1][j] = *reinterpret_cast<const half8_t *>(bsrc + j * 32 * kPitch + (kk + 1) * 16 + (kk == 3 ? 64 : 0));
+                    half8_t af[NB];
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) __builtin_memcpy(&af[nb], &xs[kk][nb], 16);
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j)
+                            acc[nb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk & 1][j], af[nb], acc[nb][j], 0, 0, 0);
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb)
+                        xs[kk][nb] = *reinterpret_cast<const u32x4_t *>(xbase[nb] + (gn * 8 + kk) * kstep[nb]);
+#pragma unroll
+                    for (int q = 0; q < NB * NJ; ++q) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                     // 1 MFMA
+                        if (q < NJ) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);         // 1 LDS read
+                        if (q >= NB * NJ - NB) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // 1 global load
+                    }
+                }
+            }
+        }
+
+        // ---- epilogue of this pass: each 32 x (32 NJ) block leaves in chunks of 128 bytes per row through the wave's
+        // private staging tile (LDS operations of one wave execute in order: no wait is needed between them) ----
+        constexpr int kChunkCols = 128 / static_cast<int>(sizeof(TOUT));     // 64 (fp16) / 32 (fp32)
+        constexpr int kChunks = NJ * 32 / kChunkCols;
+        constexpr int kBlocksPerChunk = kChunkCols / 32;
+        constexpr int kVec = 16 / static_cast<int>(sizeof(TOUT));
+        if (live) {
+            // Whole 16-byte pieces everywhere in this slab (wave-uniform): the common case takes no per-piece branch.
+            const bool whole = (N % kVec) == 0 && n_base + kSlabN <= N;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const int pblk = b0 + nb;
+#pragma unroll
+                for (int ch = 0; ch < kChunks; ++ch) {
+                    // Bias values first: the compiler cannot tell the bias reads from the staging writes (both LDS)
+                    // and would otherwise wait for each read in turn.
+                    float4 bv[kBlocksPerChunk][4];
+#pragma unroll
+                    for (int jj = 0; jj < kBlocksPerChunk; ++jj)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            bv[jj][q] = *reinterpret_cast<const float4 *>(s_bias + (jb + ch * kBlocksPerChunk + jj) * 32 + 8 * q + 4 * lh);
+#pragma unroll
+                    for (int jj = 0; jj < kBlocksPerChunk; ++jj) {
+                        const int j = ch * kBlocksPerChunk + jj;
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int cl = jj * 32 + 8 * q + 4 * lh;            // column inside the chunk
+                            const float o0 = acc[nb][j][4 * q] + bv[jj][q].x, o1 = acc[nb][j][4 * q + 1] + bv[jj][q].y;
+                            const float o2 = acc[nb][j][4 * q + 2] + bv[jj][q].z, o3 = acc[nb][j][4 * q + 3] + bv[jj][q].w;
+                            unsigned char *dst = stage + lr * kStageRow + cl * static_cast<int>(sizeof(TOUT));
+                            if constexpr (sizeof(TOUT) == 2) {
+                                const __half2 lo = __floats2half2_rn(o0, o1), hi = __floats2half2_rn(o2, o3);
+                                u32x2_t pk;
+                                pk[0] = *reinterpret_cast<const uint32_t *>(&lo);
+                                pk[1] = *reinterpret_cast<const uint32_t *>(&hi);
+                                *reinterpret_cast<u32x2_t *>(dst) = pk;
+                            } else {
+                                u32x4_t pk;
+                                pk[0] = __float_as_uint(o0); pk[1] = __float_as_uint(o1);
+                                pk[2] = __float_as_uint(o2); pk[3] = __float_as_uint(o3);
+                                *reinterpret_cast<u32x4_t *>(dst) = pk;
+                            }
+                        }
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                    const int col = n_base + jb * 32 + ch * kChunkCols + (lane & 7) * kVec;
+                    const int row0 = pblk * 32 + (lane >> 3);
+                    TOUT *dst0 = y + static_cast<int64_t>(row0) * N + col;
+                    u32x4_t v[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        v[i] = *reinterpret_cast<const u32x4_t *>(stage + (i * 8 + (lane >> 3)) * kStageRow + (lane & 7) * 16);
+                    if (whole) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            if (row0 + i * 8 < M)
+                                store_streaming16(dst0 + static_cast<int64_t>(i) * 8 * N, v[i][0], v[i][1], v[i][2], v[i][3]);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            if (row0 + i * 8 < M && col < N) {
+                                TOUT *dst = dst0 + static_cast<int64_t>(i) * 8 * N;
+                                if ((N % kVec) == 0 && col + kVec <= N) {
+                                    store_streaming16(dst, v[i][0], v[i][1], v[i][2], v[i][3]);
+                                } else {
+                                    const TOUT *e = reinterpret_cast<const TOUT *>(&v[i]);
+#pragma unroll
+                                    for (int k = 0; k < kVec; ++k)
+                                        if (col + k < N) dst[k] = e[k];
+                                }
+                            }
+                        }
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+        }
+    };
+
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I4 = std::integral_constant<int, 4>;
+    for (int pass = 0; pass < full_passes; ++pass)
+        run_pass(I2{}, I4{}, pass, blk0 + pass * 2 * kWaves + 2 * wave, 0, true);
+    if (rest > 0) {
+        const int base = blk0 + full_passes * 2 * kWaves;
+        if (rest >= kWaves) {
+            // rest - 8 pairs in front, single blocks behind them: pairs + (8 - pairs) waves, 2 pairs + 8 - pairs = rest blocks
+            const int pairs = rest - kWaves;
+            if (wave < pairs) run_pass(I2{}, I4{}, full_passes, base + 2 * wave, 0, true);
+            else run_pass(I1{}, I4{}, full_passes, base + 2 * pairs + (wave - pairs), 0, true);
+        } else {
+            // Fewer blocks than waves: as many as there are spare waves are split into two halves of 64 columns (after
+            // full passes only while at most two are split: more waves than that fetching the same x_hat at once cost
+            // more than the shorter pass gains).  A half keeps the k order of every output it computes.
+            int S = min(rest, kWaves - rest);
+            if (passes > 1 && S > 2) S = 0;
+            const int W = rest - S;
+            if (wave < W) {
+                run_pass(I1{}, I4{}, full_passes, base + wave, 0, true);
+            } else {
+                const int i = (wave - W) >> 1;
+                const bool live = i < S;
+                run_pass(I1{}, I2{}, full_passes, live ? base + W + i : base, ((wave - W) & 1) * 2, live);
+            }
+        }
+    }
+}
+
+template <typename TOUT, int WAVES, int SG>
+void launch_pair_t(const GemmArgs &g, hipStream_t stream, const void *w_hat, int ranges, int blocks_per_range)
+{
+    auto kernel = gemm_pair_kernel<TOUT, WAVES, SG>;
+    constexpr int kSmem = PairCfg<WAVES, SG>::kSmem;
+    // (Setting the attribute is cheap and idempotent; done on every call so that it holds on every device.)
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+    const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
+    const int tiles = n_slabs * ranges;
+    hipLaunchKernelGGL(kernel, dim3(8 * ((tiles + 7) / 8)), dim3(64 * WAVES), kSmem, stream,
+                       static_cast<const __half *>(g.x_hat), g.bias, static_cast<TOUT *>(g.y), g.M, g.N, g.K, ranges,
+                       blocks_per_range, static_cast<const __half *>(w_hat));
+}
+
+}  // namespace
+
+// Row ranges of the weight-stationary kernels: `slots` workgroups on the chip at once (one or two per CU).
+static void pair_ranges(const GemmArgs &g, int slots, int &ranges, int &blocks_per_range)
+{
+    const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
+    const int total_blocks = (g.M + 31) / 32;
+    ranges = slots / n_slabs;
+    if (ranges < 1) ranges = 1;
+    if (ranges > total_blocks) ranges = total_blocks;
+    blocks_per_range = (total_blocks + ranges - 1) / ranges;
+    ranges = (total_blocks + blocks_per_range - 1) / blocks_per_range;
+}
+
+// Whether the two-blocks-per-wave kernel is the one to run for this shape (weights already reconstructed).
+// Measured against gemm_slab8_kernel on the twelve DeiT-S / DeiT-B / ViT-L layer shapes: 8-17 % faster wherever K spans
+// several slab slices and a workgroup has at least eight row blocks (DeiT-B qkv 65.7 -> 54.1 us, fc1 85.2 -> 73.0,
+// ViT-L qkv 358 -> 325, fc2 444 -> 414), equal within 3 % on the single-slice shapes (K = 384), where the eight-wave
+// kernel's finer dealing of 15-19 blocks matters as much as the halved LDS traffic, and on five-block workgroups.
+bool gemm_pair_pays(const GemmArgs &g)
+{
+    int ranges, per;
+    pair_ranges(g, 256, ranges, per);
+    return g.K > 6 * 64 && per >= 8;
+}
+
+// g.x_hat is in the 32-row block layout; w_hat [N,K] fp16 holds the reconstructed weights.
+void launch_gemm_pair(const GemmArgs &g, const void *w_hat, hipStream_t stream)
+{
+    int ranges, per;
+    pair_ranges(g, 256, ranges, per);
+    if (g.y_f16) launch_pair_t<__half, 8, 6>(g, stream, w_hat, ranges, per);
+    else launch_pair_t<float, 8, 6>(g, stream, w_hat, ranges, per);
+}
+
+}  // namespace arcq

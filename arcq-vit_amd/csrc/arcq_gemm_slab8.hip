@@ -18,6 +18,7 @@
 #include "arcq_common.h"
 #include "arcq_gemm.h"
 
+#include <stdlib.h>
 #include <type_traits>
 
 #ifndef ARCQ_SPLIT_DEFAULT
@@ -478,6 +479,11 @@ void launch_slab8(const GemmArgs &g, hipStream_t stream, const void *w_hat)
 void launch_gemm_slab8(const GemmArgs &g, const void *w_hat, hipStream_t stream)
 {
     if (w_hat) {
+        const char *e = getenv("ARCQ_PAIR");           // tuning aid: 0 / 1 pin the choice
+        if (e ? e[0] == '1' : gemm_pair_pays(g)) {
+            launch_gemm_pair(g, w_hat, stream);
+            return;
+        }
         if (g.y_f16) launch_slab8<4, __half, true>(g, stream, w_hat);
         else launch_slab8<4, float, true>(g, stream, w_hat);
         return;

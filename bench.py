@@ -101,7 +101,8 @@ class Layer:
     # that are ready; other shapes: arcq_act_quant and arcq_linear_fused_ws.
     def mode(self, lib, m):
         name = lib.arcq_linear_otf_ws_kernel(m, self.n, self.k, 1)
-        return "copy" if name == b"gemm_slab8_kernel<copy>" else "blocked" if b"slab8" in name else "rowmajor"
+        return ("copy" if name in (b"gemm_slab8_kernel<copy>", b"gemm_pair_kernel") else
+                "blocked" if b"slab8" in name else "rowmajor")
 
     def call_act(self, lib, x, ws, stream):
         from arcq_vit_amd._lib import ARCQ_F16

@@ -196,9 +196,10 @@ int arcq_linear_otf_static(const void *x, int x_dtype, const float *a_thresholds
                            const float *bias, void *y, int y_dtype,
                            int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
 
-/* Kernels arcq_linear_otf_ws runs after stage 1 for these sizes: "gemm_slab8_kernel", or "gemm_slab8_kernel<copy>"
- * (weights rebuilt in the stage-1 launch, copied by the GEMM), when it takes the block layout, else
- * arcq_linear_fused_ws_kernel's answer.  A profiling aid with no counterpart in the reference. */
+/* Kernels arcq_linear_otf_ws runs after stage 1 for these sizes: "gemm_slab8_kernel", or, with the weights rebuilt
+ * in the stage-1 launch and copied by the GEMM, "gemm_slab8_kernel<copy>" or "gemm_pair_kernel" (two row blocks per
+ * wave), when it takes the block layout, else arcq_linear_fused_ws_kernel's answer.  A profiling aid with no
+ * counterpart in the reference. */
 const char *arcq_linear_otf_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace);
 
 /* ---- index-space linears (no reconstruction, product-table gather) ---------

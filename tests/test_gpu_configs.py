@@ -99,9 +99,9 @@ def test_benchmarked_layer_call_fullsize(cuda, oracle, name, k, n, bits):
     path = _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1).decode()
     a = oracle.act_quant_c(x.float().numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)
     w16 = oracle.weight_dequant_c(pw.numpy(), cb, wc, ws, wcs, bits, 64, fma=True).astype(np.float16)
-    if "slab8" in path:           # stage 1 wrote the block layout, the stage-1 launch rebuilt the weights
+    if "slab8" in path or "pair" in path:       # stage 1 wrote the block layout
         assert np.array_equal(_np(x_ws).view(np.uint16), _np(_to_blocked(torch.from_numpy(a))).view(np.uint16)), path
-    if path.endswith("<copy>"):
+    if path.endswith("<copy>") or "pair" in path:       # the stage-1 launch rebuilt the weights
         assert np.array_equal(_np(w_ws).view(np.uint16), w16.reshape(-1).view(np.uint16)), path
     rows = torch.randint(0, m, (64,), generator=torch.Generator().manual_seed(3))
     rows[0], rows[1] = 0, m - 1
