@@ -100,26 +100,29 @@ gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, 
         }
     };
 
-    // One pass of one wave: NB row blocks (first block b0) times NJ of the slab's four 32-column tiles, from tile jb.
-    // Every wave of the workgroup runs this once per pass, whatever its NB and NJ: the barriers are the same in every
-    // instantiation.  live == false: the wave has no block in this pass and only keeps the barriers company.
-    auto run_pass = [&](auto nbc, auto njc, const int pass, const int b0, const int jb, const bool live) __attribute__((always_inline)) {
-        constexpr int NB = decltype(nbc)::value;
-        constexpr int NJ = decltype(njc)::value;
-        const unsigned char *slab_wave = slab_lane + jb * 32 * kPitch;
-        float16_t acc[NB][NJ];
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-            for (int j = 0; j < NJ; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[nb][j][v] = 0.0f;
+    // The same copy for the one place where it runs under other LDS traffic (the write-out of a pass): issued from
+    // inline assembly, because the compiler orders every LDS read behind a pending global -> LDS load it knows of
+    // (it cannot tell that the staging tile and the slab are disjoint) and would wait for the slice right away.
+    // The caller waits for vmcnt(0) and a barrier before anybody reads the slab.
+    auto copy_slice_unseen = [&](int g0, int ng) __attribute__((always_inline)) {
+        for (int p0 = wave * 64; p0 < kSlabN * kPieces; p0 += kWaves * 64) {
+            const int p = p0 + lane;
+            const int row = p / kPieces, col = p - row * kPieces;
+            const int n = min(n_base + row, N - 1);
+            const __half *src = w_hat + static_cast<int64_t>(n) * K + g0 * 64 + col * 8;
+            const uint32_t lds = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+                (__attribute__((address_space(3))) unsigned char *)(slab + p0 * 16))));      // wave-uniform
+            if (col < 8 * ng && row < kSlabN)
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds) : "memory", "m0");
+        }
+    };
 
-        // x_hat fragments: lane (lr, lh) reads, for k-step kk of group g, piece 8 g + 4 lh + kk of row lr of its block
-        // (k = 64 g + 32 lh + 8 kk ... + 7).  A last block of fewer than 32 rows is stored compactly: its pieces are
-        // `rows` apart instead of 32, and the lanes past its last row re-read that row (their outputs are not stored).
-        const char *xbase[NB];
-        int kstep[NB];
+    // x_hat fragments: lane (lr, lh) reads, for k-step kk of group g, piece 8 g + 4 lh + kk of row lr of its block
+    // (k = 64 g + 32 lh + 8 kk ... + 7).  A last block of fewer than 32 rows is stored compactly: its pieces are
+    // `rows` apart instead of 32, and the lanes past its last row re-read that row (their outputs are not stored).
+    // Address of this lane's first piece of block b0 + nb (group 0, k-step 0) and the distance between k-steps.
+    auto set_blocks = [&](auto nbc, const int b0, const char *(&xbase)[decltype(nbc)::value], int (&kstep)[decltype(nbc)::value]) __attribute__((always_inline)) {
+        constexpr int NB = decltype(nbc)::value;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             const int blk = min(b0 + nb, total_blocks - 1);
@@ -128,144 +131,159 @@ gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, 
             xbase[nb] = reinterpret_cast<const char *>(xb) + static_cast<int64_t>(blk) * K * 64 + lh * 4 * kstep[nb] +
                         min(lr, rows - 1) * 16;
         }
-        // The first group's fragments, requested in the order in which the loop below refills the slots (the scheduling
-        // barriers pin it).  The compiler's wait-count bookkeeping merges this state with the loop's own at the top of
-        // the group loop and waits for the stricter of the two: with the loads in any other order here (left alone it
-        // reverses them) that is vmcnt(0) in every iteration, i.e. no load is ever left in flight across a group.
-        u32x4_t xs[4][NB];
-        if (live) {
+    };
+    // The first group's fragments, requested in the order in which the group loop refills the slots (the scheduling
+    // barriers pin it).  The compiler's wait-count bookkeeping merges this state with the loop's own at the top of the
+    // group loop and waits for the stricter of the two: with the loads in any other order here (left alone it
+    // reverses them) that is vmcnt(0) in every iteration, i.e. no load is ever left in flight across a group.
+    auto first_fragments = [&](auto nbc, u32x4_t (&xs)[4][decltype(nbc)::value], const char *const (&xbase)[decltype(nbc)::value],
+                               const int (&kstep)[decltype(nbc)::value]) __attribute__((always_inline)) {
+        constexpr int NB = decltype(nbc)::value;
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk)
+        for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                    xs[kk][nb] = *reinterpret_cast<const u32x4_t *>(xbase[nb] + kk * kstep[nb]);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-        }
-
-        for (int sl = 0; sl < slices; ++sl) {
-            const int g0 = sl * kSliceGroups;
-            const int ng = min(kSliceGroups, G - g0);
-            if (!(slices == 1 && pass > 0)) {
-                __syncthreads();      // every wave is done reading the previous slice
-                copy_slice(g0, ng);
-                __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the slice has landed in LDS
-                asm volatile("" ::: "memory");
-                __syncthreads();
+            for (int nb = 0; nb < NB; ++nb) {
+                xs[kk][nb] = *reinterpret_cast<const u32x4_t *>(xbase[nb] + kk * kstep[nb]);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            if (!live) continue;
-            half8_t bf[2][NJ];
+    };
+    auto fill_slice = [&](int g0, int ng) __attribute__((always_inline)) {
+        __syncthreads();      // every wave is done reading the previous slice
+        copy_slice(g0, ng);
+        __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the slice has landed in LDS
+        asm volatile("" ::: "memory");
+        __syncthreads();
+    };
+
+    // The groups [g0, g0 + ng) of the resident slice times NB row blocks and NJ column tiles from tile jb.  Slot kk is
+    // refilled, right after the MFMAs that read it, with k-step kk of the next group; after the last group of the
+    // tensor (g == G - 1) with group 0 of the blocks at xnext (the wave's next pass, or any valid address).
+    auto multiply_slice = [&](auto nbc, auto njc, float16_t (&acc)[decltype(nbc)::value][decltype(njc)::value],
+                              u32x4_t (&xs)[4][decltype(nbc)::value], const char *const (&xbase)[decltype(nbc)::value],
+                              const int (&kstep)[decltype(nbc)::value], const char *const (&xnext)[decltype(nbc)::value],
+                              const int (&knext)[decltype(nbc)::value], const int g0, const int ng, const int jb) __attribute__((always_inline)) {
+        constexpr int NB = decltype(nbc)::value;
+        constexpr int NJ = decltype(njc)::value;
+        const unsigned char *slab_wave = slab_lane + jb * 32 * kPitch;
+        half8_t bf[2][NJ];
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) bf[0][j] = *reinterpret_cast<const half8_t *>(slab_wave + j * 32 * kPitch);
-            for (int gl = 0; gl < ng; ++gl) {
-                // The group whose fragments the slots are refilled with: the next one, or (past the last) the last one
-                // again -- lines this wave has just read, so those loads hit L1 and nobody waits for them.
-                const int gn = min(g0 + gl + 1, G - 1);
-                const unsigned char *bsrc = slab_wave + gl * 128;
+        for (int j = 0; j < NJ; ++j) bf[0][j] = *reinterpret_cast<const half8_t *>(slab_wave + j * 32 * kPitch);
+        for (int gl = 0; gl < ng; ++gl) {
+            const bool wrap = g0 + gl + 1 >= G;
+            const char *rbase[NB];
+            int rstep[NB];
 #pragma unroll
-                for (int kk = 0; kk < 4; ++kk) {
-                    // w_hat fragments of the next k-step (of the next group after the fourth; past the slice after
-                    // its last one: read and never used)
+            for (int nb = 0; nb < NB; ++nb) {
+                rstep[nb] = wrap ? knext[nb] : kstep[nb];
+                rbase[nb] = wrap ? xnext[nb] : xbase[nb] + (g0 + gl + 1) * 8 * kstep[nb];
+            }
+            const unsigned char *bsrc = slab_wave + gl * 128;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                // w_hat fragments of the next k-step (of the next group after the fourth; past the slice after its
+                // last one: read and never used)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+                    bf[(kk + 1) & 1][j] = *reinterpret_cast<const half8_t *>(bsrc + j * 32 * kPitch + (kk + 1) * 16 + (kk == 3 ? 64 : 0));
+                half8_t af[NB];
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) __builtin_memcpy(&af[nb], &xs[kk][nb], 16);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                     for (int j = 0; j < NJ; ++j)
-                        bf[(kk + 1) & 1][j] = *reinterpret_cast<const half8_t *>(bsrc + j * 32 * kPitch + (kk + 1) * 16 + (kk == 3 ? 64 : 0));
-                    half8_t af[NB];
+                        acc[nb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk & 1][j], af[nb], acc[nb][j], 0, 0, 0);
 #pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) __builtin_memcpy(&af[nb], &xs[kk][nb], 16);
+                for (int nb = 0; nb < NB; ++nb)
+                    xs[kk][nb] = *reinterpret_cast<const u32x4_t *>(rbase[nb] + kk * rstep[nb]);
 #pragma unroll
-                    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                        for (int j = 0; j < NJ; ++j)
-                            acc[nb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk & 1][j], af[nb], acc[nb][j], 0, 0, 0);
-#pragma unroll
-                    for (int nb = 0; nb < NB; ++nb)
-                        xs[kk][nb] = *reinterpret_cast<const u32x4_t *>(xbase[nb] + (gn * 8 + kk) * kstep[nb]);
-#pragma unroll
-                    for (int q = 0; q < NB * NJ; ++q) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                     // 1 MFMA
-                        if (q < NJ) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);         // 1 LDS read
-                        if (q >= NB * NJ - NB) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // 1 global load
-                    }
+                for (int q = 0; q < NB * NJ; ++q) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                     // 1 MFMA
+                    if (q < NJ) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);         // 1 LDS read
+                    if (q >= NB * NJ - NB) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // 1 global load
                 }
             }
         }
+    };
 
-        // ---- epilogue of this pass: each 32 x (32 NJ) block leaves in chunks of 128 bytes per row through the wave's
-        // private staging tile (LDS operations of one wave execute in order: no wait is needed between them) ----
+    // The NB blocks from b0 (32 x 32 NJ values each, columns from tile jb) leave in chunks of 128 bytes per row through
+    // the wave's private staging tile (LDS operations of one wave execute in order: no wait is needed between them).
+    auto write_out = [&](auto nbc, auto njc, const float16_t (&acc)[decltype(nbc)::value][decltype(njc)::value],
+                         const int b0, const int jb) __attribute__((always_inline)) {
+        constexpr int NB = decltype(nbc)::value;
+        constexpr int NJ = decltype(njc)::value;
         constexpr int kChunkCols = 128 / static_cast<int>(sizeof(TOUT));     // 64 (fp16) / 32 (fp32)
         constexpr int kChunks = NJ * 32 / kChunkCols;
         constexpr int kBlocksPerChunk = kChunkCols / 32;
         constexpr int kVec = 16 / static_cast<int>(sizeof(TOUT));
-        if (live) {
-            // Whole 16-byte pieces everywhere in this slab (wave-uniform): the common case takes no per-piece branch.
-            const bool whole = (N % kVec) == 0 && n_base + kSlabN <= N;
+        // Whole 16-byte pieces everywhere in this slab (wave-uniform): the common case takes no per-piece branch.
+        const bool whole = (N % kVec) == 0 && n_base + kSlabN <= N;
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                const int pblk = b0 + nb;
+        for (int nb = 0; nb < NB; ++nb) {
+            const int pblk = b0 + nb;
 #pragma unroll
-                for (int ch = 0; ch < kChunks; ++ch) {
-                    // Bias values first: the compiler cannot tell the bias reads from the staging writes (both LDS)
-                    // and would otherwise wait for each read in turn.
-                    float4 bv[kBlocksPerChunk][4];
+            for (int ch = 0; ch < kChunks; ++ch) {
+                // Bias values first: the compiler cannot tell the bias reads from the staging writes (both LDS) and
+                // would otherwise wait for each read in turn.
+                float4 bv[kBlocksPerChunk][4];
 #pragma unroll
-                    for (int jj = 0; jj < kBlocksPerChunk; ++jj)
+                for (int jj = 0; jj < kBlocksPerChunk; ++jj)
 #pragma unroll
-                        for (int q = 0; q < 4; ++q)
-                            bv[jj][q] = *reinterpret_cast<const float4 *>(s_bias + (jb + ch * kBlocksPerChunk + jj) * 32 + 8 * q + 4 * lh);
+                    for (int q = 0; q < 4; ++q)
+                        bv[jj][q] = *reinterpret_cast<const float4 *>(s_bias + (jb + ch * kBlocksPerChunk + jj) * 32 + 8 * q + 4 * lh);
 #pragma unroll
-                    for (int jj = 0; jj < kBlocksPerChunk; ++jj) {
-                        const int j = ch * kBlocksPerChunk + jj;
+                for (int jj = 0; jj < kBlocksPerChunk; ++jj) {
+                    const int j = ch * kBlocksPerChunk + jj;
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const int cl = jj * 32 + 8 * q + 4 * lh;            // column inside the chunk
-                            const float o0 = acc[nb][j][4 * q] + bv[jj][q].x, o1 = acc[nb][j][4 * q + 1] + bv[jj][q].y;
-                            const float o2 = acc[nb][j][4 * q + 2] + bv[jj][q].z, o3 = acc[nb][j][4 * q + 3] + bv[jj][q].w;
-                            unsigned char *dst = stage + lr * kStageRow + cl * static_cast<int>(sizeof(TOUT));
-                            if constexpr (sizeof(TOUT) == 2) {
-                                const __half2 lo = __floats2half2_rn(o0, o1), hi = __floats2half2_rn(o2, o3);
-                                u32x2_t pk;
-                                pk[0] = *reinterpret_cast<const uint32_t *>(&lo);
-                                pk[1] = *reinterpret_cast<const uint32_t *>(&hi);
-                                *reinterpret_cast<u32x2_t *>(dst) = pk;
-                            } else {
-                                u32x4_t pk;
-                                pk[0] = __float_as_uint(o0); pk[1] = __float_as_uint(o1);
-                                pk[2] = __float_as_uint(o2); pk[3] = __float_as_uint(o3);
-                                *reinterpret_cast<u32x4_t *>(dst) = pk;
-                            }
+                    for (int q = 0; q < 4; ++q) {
+                        const int cl = jj * 32 + 8 * q + 4 * lh;            // column inside the chunk
+                        const float o0 = acc[nb][j][4 * q] + bv[jj][q].x, o1 = acc[nb][j][4 * q + 1] + bv[jj][q].y;
+                        const float o2 = acc[nb][j][4 * q + 2] + bv[jj][q].z, o3 = acc[nb][j][4 * q + 3] + bv[jj][q].w;
+                        unsigned char *dst = stage + lr * kStageRow + cl * static_cast<int>(sizeof(TOUT));
+                        if constexpr (sizeof(TOUT) == 2) {
+                            const __half2 lo = __floats2half2_rn(o0, o1), hi = __floats2half2_rn(o2, o3);
+                            u32x2_t pk;
+                            pk[0] = *reinterpret_cast<const uint32_t *>(&lo);
+                            pk[1] = *reinterpret_cast<const uint32_t *>(&hi);
+                            *reinterpret_cast<u32x2_t *>(dst) = pk;
+                        } else {
+                            u32x4_t pk;
+                            pk[0] = __float_as_uint(o0); pk[1] = __float_as_uint(o1);
+                            pk[2] = __float_as_uint(o2); pk[3] = __float_as_uint(o3);
+                            *reinterpret_cast<u32x4_t *>(dst) = pk;
                         }
                     }
-                    __builtin_amdgcn_wave_barrier();
-                    const int col = n_base + jb * 32 + ch * kChunkCols + (lane & 7) * kVec;
-                    const int row0 = pblk * 32 + (lane >> 3);
-                    TOUT *dst0 = y + static_cast<int64_t>(row0) * N + col;
-                    u32x4_t v[4];
+                }
+                __builtin_amdgcn_wave_barrier();
+                const int col = n_base + jb * 32 + ch * kChunkCols + (lane & 7) * kVec;
+                const int row0 = pblk * 32 + (lane >> 3);
+                TOUT *dst0 = y + static_cast<int64_t>(row0) * N + col;
+                u32x4_t v[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    v[i] = *reinterpret_cast<const u32x4_t *>(stage + (i * 8 + (lane >> 3)) * kStageRow + (lane & 7) * 16);
+                if (whole) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
-                        v[i] = *reinterpret_cast<const u32x4_t *>(stage + (i * 8 + (lane >> 3)) * kStageRow + (lane & 7) * 16);
-                    if (whole) {
+                        if (row0 + i * 8 < M)
+                            store_streaming16(dst0 + static_cast<int64_t>(i) * 8 * N, v[i][0], v[i][1], v[i][2], v[i][3]);
+                } else {
 #pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            if (row0 + i * 8 < M)
-                                store_streaming16(dst0 + static_cast<int64_t>(i) * 8 * N, v[i][0], v[i][1], v[i][2], v[i][3]);
-                    } else {
+                    for (int i = 0; i < 4; ++i) {
+                        if (row0 + i * 8 < M && col < N) {
+                            TOUT *dst = dst0 + static_cast<int64_t>(i) * 8 * N;
+                            if ((N % kVec) == 0 && col + kVec <= N) {
+                                store_streaming16(dst, v[i][0], v[i][1], v[i][2], v[i][3]);
+                            } else {
+                                const TOUT *e = reinterpret_cast<const TOUT *>(&v[i]);
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            if (row0 + i * 8 < M && col < N) {
-                                TOUT *dst = dst0 + static_cast<int64_t>(i) * 8 * N;
-                                if ((N % kVec) == 0 && col + kVec <= N) {
-                                    store_streaming16(dst, v[i][0], v[i][1], v[i][2], v[i][3]);
-                                } else {
-                                    const TOUT *e = reinterpret_cast<const TOUT *>(&v[i]);
-#pragma unroll
-                                    for (int k = 0; k < kVec; ++k)
-                                        if (col + k < N) dst[k] = e[k];
-                                }
+                                for (int k = 0; k < kVec; ++k)
+                                    if (col + k < N) dst[k] = e[k];
                             }
                         }
                     }
-                    __builtin_amdgcn_wave_barrier();
                 }
+                __builtin_amdgcn_wave_barrier();
             }
         }
     };
@@ -273,15 +291,95 @@ gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, 
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
     using I4 = std::integral_constant<int, 4>;
-    for (int pass = 0; pass < full_passes; ++pass)
-        run_pass(I2{}, I4{}, pass, blk0 + pass * 2 * kWaves + 2 * wave, 0, true);
+
+    // ---- full passes: every wave multiplies a pair of blocks.  The fragment slots run on from one pass into the next
+    // (the last group of a pass refills them with the first group of the wave's next pair), and when K spans several
+    // slices the first slice of the next pass is requested before this pass's blocks are written out, so both
+    // latencies pass under the write-out. ----
+    if (full_passes > 0) {
+        float16_t acc[2][4];
+        u32x4_t xs[4][2];
+        const char *xcur[2], *xnxt[2];
+        int kcur[2], knxt[2];
+        set_blocks(I2{}, blk0 + 2 * wave, xcur, kcur);
+        first_fragments(I2{}, xs, xcur, kcur);
+        fill_slice(0, min(kSliceGroups, G));
+        for (int pass = 0; pass < full_passes; ++pass) {
+            const bool more = pass + 1 < full_passes;
+            const int b0 = blk0 + pass * 2 * kWaves + 2 * wave;
+            if (more) {
+                set_blocks(I2{}, b0 + 2 * kWaves, xnxt, knxt);
+            } else {          // nothing follows: re-read this pair's last group (lines the wave has just read)
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+                    knxt[nb] = kcur[nb];
+                    xnxt[nb] = xcur[nb] + (G - 1) * 8 * kcur[nb];
+                }
+            }
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[nb][j][v] = 0.0f;
+            for (int sl = 0; sl < slices; ++sl) {
+                const int g0 = sl * kSliceGroups;
+                multiply_slice(I2{}, I4{}, acc, xs, xcur, kcur, xnxt, knxt, g0, min(kSliceGroups, G - g0), 0);
+                if (sl + 1 < slices) fill_slice(g0 + kSliceGroups, min(kSliceGroups, G - g0 - kSliceGroups));
+            }
+            const bool refill = slices > 1 && more;
+            if (refill) {
+                __syncthreads();      // every wave is done reading the last slice
+                copy_slice_unseen(0, kSliceGroups);
+            }
+            write_out(I2{}, I4{}, acc, b0, 0);
+            if (refill) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+                asm volatile("" ::: "memory");
+                __syncthreads();
+            }
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) {
+                xcur[nb] = xnxt[nb];
+                kcur[nb] = knxt[nb];
+            }
+        }
+    }
+
+    // ---- the left-over blocks (fewer than sixteen): one more pass, dealt as pairs, single blocks and column halves.
+    // Every wave runs it exactly once, whatever its share: the barriers inside are the same in every instantiation. ----
+    auto last_pass = [&](auto nbc, auto njc, const int b0, const int jb, const bool live) __attribute__((always_inline)) {
+        constexpr int NB = decltype(nbc)::value;
+        constexpr int NJ = decltype(njc)::value;
+        float16_t acc[NB][NJ];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[nb][j][v] = 0.0f;
+        const char *xbase[NB], *xlast[NB];
+        int kstep[NB];
+        set_blocks(nbc, b0, xbase, kstep);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) xlast[nb] = xbase[nb] + (G - 1) * 8 * kstep[nb];
+        u32x4_t xs[4][NB];
+        if (live) first_fragments(nbc, xs, xbase, kstep);
+        for (int sl = 0; sl < slices; ++sl) {
+            const int g0 = sl * kSliceGroups;
+            const int ng = min(kSliceGroups, G - g0);
+            if (!(slices == 1 && full_passes > 0)) fill_slice(g0, ng);      // (a single slice is still resident)
+            if (live) multiply_slice(nbc, njc, acc, xs, xbase, kstep, xlast, kstep, g0, ng, jb);
+        }
+        if (live) write_out(nbc, njc, acc, b0, jb);
+    };
     if (rest > 0) {
         const int base = blk0 + full_passes * 2 * kWaves;
         if (rest >= kWaves) {
             // rest - 8 pairs in front, single blocks behind them: pairs + (8 - pairs) waves, 2 pairs + 8 - pairs = rest blocks
             const int pairs = rest - kWaves;
-            if (wave < pairs) run_pass(I2{}, I4{}, full_passes, base + 2 * wave, 0, true);
-            else run_pass(I1{}, I4{}, full_passes, base + 2 * pairs + (wave - pairs), 0, true);
+            if (wave < pairs) last_pass(I2{}, I4{}, base + 2 * wave, 0, true);
+            else last_pass(I1{}, I4{}, base + 2 * pairs + (wave - pairs), 0, true);
         } else {
             // Fewer blocks than waves: as many as there are spare waves are split into two halves of 64 columns (after
             // full passes only while at most two are split: more waves than that fetching the same x_hat at once cost
@@ -290,11 +388,11 @@ gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, 
             if (passes > 1 && S > 2) S = 0;
             const int W = rest - S;
             if (wave < W) {
-                run_pass(I1{}, I4{}, full_passes, base + wave, 0, true);
+                last_pass(I1{}, I4{}, base + wave, 0, true);
             } else {
                 const int i = (wave - W) >> 1;
                 const bool live = i < S;
-                run_pass(I1{}, I2{}, full_passes, live ? base + W + i : base, ((wave - W) & 1) * 2, live);
+                last_pass(I1{}, I2{}, live ? base + W + i : base, ((wave - W) & 1) * 2, live);
             }
         }
     }

@@ -495,6 +495,42 @@ def test_fused_gemm_block_layout(cuda, oracle, monkeypatch, bits, out_dtype, m, 
     assert torch.equal(nb + bias, yb)            # the bias is one fp32 addition before the output rounding
 
 
+@pytest.mark.parametrize("bits,out_dtype", [(4, torch.float16), (3, torch.float32)])
+@pytest.mark.parametrize("m,n,k", [(8960 + 7, 4096, 128),     # 8 ranges of 35-36 blocks: two full passes of pairs, 3-4 left (halves), ragged last block
+                                   (10496, 4000, 192),        # 41 blocks per range: two full passes, 1 pair + 7 single blocks; ragged N
+                                   (7936, 4096, 64),          # 31 blocks: one full pass, 7 pairs + 1 single block
+                                   (4096, 4096, 448),         # 16 blocks, two slices: exactly one full pass, nothing left
+                                   (3000, 1000, 832),         # 94 blocks over 32 ranges: 3 per workgroup (no full pass), three slices, ragged M and N
+                                   (12608, 768, 768),         # DeiT-B proj: 10 blocks per workgroup: 2 pairs + 6 singles, two slices
+                                   (6400, 2304, 1024)])       # 200 blocks over 14 ranges of 15: 7 pairs + 1 single, three slices
+def test_fused_gemm_pair_kernel(cuda, oracle, monkeypatch, bits, out_dtype, m, n, k):
+    """gemm_pair_kernel (two row blocks per wave and pass, weights ready in a workspace) against gemm_slab8_kernel on
+    the same operands: bit-identical (same k order per output), whichever way a workgroup's blocks fall into pairs,
+    single blocks and column halves; sampled rows against the fp64 oracle."""
+    cb, packed, center, scale, code_sum = _packed_weight(oracle, n, k, bits, 61)
+    _, thr = _cb(bits)
+    x = synth.make_activation(m, k, 61, "gelu" if k > n else "ln").to(torch.float16)
+    bias = synth.make_bias(n, 61).to(cuda)
+    w = [t.to(cuda) for t in (packed, cb, center, scale, code_sum)]
+    ws = torch.empty(n * k, dtype=torch.float16, device=cuda)
+    xb = ops.quantize_activation_blocked(x.to(cuda), thr.to(cuda), cb.to(cuda), bits, weights=w, w_hat=ws)
+    monkeypatch.setenv("ARCQ_PAIR", "0")
+    ref = ops.linear_fused_blocked(xb, m, k, *w, bias, bits, out_dtype=out_dtype, w_hat_ws=ws, w_hat_ready=True)
+    monkeypatch.setenv("ARCQ_PAIR", "1")
+    y = ops.linear_fused_blocked(xb, m, k, *w, bias, bits, out_dtype=out_dtype, w_hat_ws=ws, w_hat_ready=True)
+    monkeypatch.delenv("ARCQ_PAIR")
+    assert torch.equal(y, ref)
+    rows = torch.randint(0, m, (40,), generator=torch.Generator().manual_seed(2))
+    rows[0], rows[1] = 0, m - 1
+    a = oracle.act_quant_c(x[rows].float().numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)
+    w16 = oracle.weight_dequant_c(packed.numpy(), cb, center, scale, code_sum, bits, 64, fma=True).astype(np.float16)
+    y64, mag = oracle.linear_f64_c(a, w16, _np(bias))
+    tol = _gemm_tol(mag, k)
+    if out_dtype == torch.float16:
+        tol = tol + np.abs(y64) * 2.0 ** -11 + 2.0 ** -25
+    assert np.all(np.abs(_np(y[rows.to(cuda)]).astype(np.float64) - y64) <= tol)
+
+
 @pytest.mark.parametrize("m", [1504, 1576])     # whole 32-row blocks / a last block of 8 rows
 def test_layer_otf_scratch_workspaces(cuda, oracle, monkeypatch, m):
     """arcq_linear_otf_ws (scratch-only workspaces) == arcq_linear_otf bit for bit, whichever layout it uses inside."""
