@@ -48,7 +48,7 @@ _SIGNATURES = {
     "arcq_linear_forward_packed": [_c_ptr] * 11 + [_c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_ptr],
     "arcq_linear_forward_u8": [_c_ptr] * 11 + [_c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
 }
-EXPORTED_SYMBOLS = ("arcq_version", "arcq_last_error", "arcq_linear_fused_kernel",
+EXPORTED_SYMBOLS = ("arcq_version", "arcq_last_error", "arcq_reload_tuning", "arcq_linear_fused_kernel",
                     "arcq_linear_fused_ws_kernel", "arcq_linear_otf_ws_kernel") + tuple(_SIGNATURES)
 
 _lib = None
@@ -75,6 +75,8 @@ def load() -> ctypes.CDLL:
             lib.arcq_version.argtypes = []
             lib.arcq_last_error.restype = ctypes.c_char_p
             lib.arcq_last_error.argtypes = []
+            lib.arcq_reload_tuning.restype = None
+            lib.arcq_reload_tuning.argtypes = []
             lib.arcq_linear_fused_kernel.restype = ctypes.c_char_p
             lib.arcq_linear_fused_kernel.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64]
             lib.arcq_linear_fused_ws_kernel.restype = ctypes.c_char_p
@@ -95,3 +97,8 @@ def check(rc: int) -> None:
     if rc != 0:
         msg = load().arcq_last_error().decode("utf-8", "replace")
         raise RuntimeError(msg or f"libarcq_hip call failed with code {rc}")
+
+
+def reload_tuning() -> None:
+    """Make the library read its ``ARCQ_*`` tuning variables again (it reads them once per process)."""
+    load().arcq_reload_tuning()

@@ -30,7 +30,46 @@ int launch_status(const char *what)
     return fail(static_cast<int>(e), "%s: launch failed: %s", what, hipGetErrorString(e));
 }
 
+namespace {
+struct TuningStore {
+    char gemm_kernel[32], otf_fused[8], pair[8];
+    Tuning view;
+};
+TuningStore g_tuning;
+std::once_flag g_tuning_once;
+std::mutex g_tuning_mutex;
+
+void read_tuning()
+{
+    auto grab = [](const char *name, char *buf, size_t n) -> const char * {
+        const char *e = getenv(name);
+        if (!e) return nullptr;
+        strncpy(buf, e, n - 1);
+        buf[n - 1] = 0;
+        return buf;
+    };
+    std::lock_guard<std::mutex> lock(g_tuning_mutex);
+    g_tuning.view.gemm_kernel = grab("ARCQ_GEMM_KERNEL", g_tuning.gemm_kernel, sizeof(g_tuning.gemm_kernel));
+    g_tuning.view.otf_fused = grab("ARCQ_OTF_FUSED", g_tuning.otf_fused, sizeof(g_tuning.otf_fused));
+    g_tuning.view.pair = grab("ARCQ_PAIR", g_tuning.pair, sizeof(g_tuning.pair));
+}
+}  // namespace
+
+const Tuning &tuning()
+{
+    std::call_once(g_tuning_once, read_tuning);
+    return g_tuning.view;
+}
+
 }  // namespace arcq
+
+// Reads the ARCQ_* tuning variables again (they are otherwise read once per process).  Not safe against calls
+// running in other threads at the same moment; a hook for tests and tuning scripts.
+ARCQ_API void arcq_reload_tuning(void)
+{
+    (void)arcq::tuning();
+    arcq::read_tuning();
+}
 
 ARCQ_API int arcq_version(void) { return ARCQ_VERSION; }
 
@@ -51,7 +90,7 @@ static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds
     // is plainly valid; anything else goes through the two entry points below, which report what is wrong.
     // ARCQ_OTF_FUSED=0 switches the single-launch path off, =2 takes it for every shape the kernel can run (tuning aids).
     {
-        const char *e = getenv("ARCQ_OTF_FUSED");
+        const char *e = arcq::tuning().otf_fused;
         const bool enabled = !(e && e[0] == '0');
         if (enabled && group_size == 64 && arcq::bits_ok(bits) && M > 0 && N > 0 && N < (int64_t(1) << 30) &&
             arcq::otf_small_supported(M, N, K, e && e[0] == '2') && x && x != x_hat_ws && a_thresholds && a_codebook && packed_w &&

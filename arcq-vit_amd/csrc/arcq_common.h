@@ -6,6 +6,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <atomic>
+
 #include "arcq_hip.h"
 
 #define ARCQ_API extern "C" __attribute__((visibility("default")))
@@ -16,6 +18,15 @@ namespace arcq {
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 // Turns hipGetLastError() after a launch into the ABI's return value.
 int launch_status(const char *what);
+
+// Tuning switches from the environment (ARCQ_GEMM_KERNEL, ARCQ_OTF_FUSED, ARCQ_PAIR), read once per process;
+// arcq_reload_tuning() reads them again.  nullptr = not set.
+struct Tuning {
+    const char *gemm_kernel;   // "stream" | "slab" | "small" | "splitk" | "slab8" | "prebuilt"
+    const char *otf_fused;     // "0" | "2"
+    const char *pair;          // "0" | "1"
+};
+const Tuning &tuning();
 
 __host__ __device__ inline bool bits_ok(int bits) { return bits == 2 || bits == 3 || bits == 4; }
 __host__ __device__ inline int64_t packed_cols(int64_t length, int bits) { return (length * bits + 7) / 8; }
@@ -80,6 +91,20 @@ __device__ __forceinline__ void store_writethrough16(void *p, uint32_t a, uint32
     // The two wait states keep the next VALU instruction from overwriting the data registers while the store still
     // reads them (the compiler inserts them for its own wide stores; it does not look inside an asm statement).
     asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+}
+
+// Raises a kernel's dynamic LDS limit, once per device and kernel (the attribute belongs to the device's copy of
+// the code object).  Kernel is the kernel's address as a template argument, so every kernel has its own record.
+template <auto Kernel>
+inline void allow_dynamic_lds(int bytes)
+{
+    static std::atomic<uint64_t> done{0};          // one bit per device index (mod 64: at worst a redundant call)
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const uint64_t bit = uint64_t(1) << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return;
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    done.fetch_or(bit, std::memory_order_release);
 }
 
 __device__ __forceinline__ float to_float(float v) { return v; }

@@ -207,10 +207,10 @@ static void launch_out(const void *x_hat, const uint8_t *pw, const float *cb, co
 
 using namespace arcq;
 
-// Tuning aid: ARCQ_GEMM_KERNEL=stream|slab|small|splitk pins the kernel choice (looked up on every call).
+// Tuning aid: ARCQ_GEMM_KERNEL=stream|slab|small|splitk pins the kernel choice (read once per process).
 static int forced_kernel()
 {
-    const char *e = getenv("ARCQ_GEMM_KERNEL");
+    const char *e = tuning().gemm_kernel;
     if (!e) return 0;
     if (!strcmp(e, "stream")) return 1;
     if (!strcmp(e, "slab")) return 2;
@@ -325,7 +325,7 @@ ARCQ_API int arcq_linear_fused(const void *x_hat,
 static bool workspace_pays(int64_t M, int64_t N, int64_t K)
 {
     if (M < 512 || K < 64 || K % 64 != 0 || M * K * 2 >= (int64_t(1) << 32)) return false;
-    const char *e = getenv("ARCQ_GEMM_KERNEL");
+    const char *e = tuning().gemm_kernel;
     if (e) return !strcmp(e, "prebuilt");
     // Measured: copying beats both fused kernels when few slabs (N <= 1024) meet a K of three or more slab slices,
     // i.e. when up to 256 / slabs workgroups per slab would each rebuild the same long weight rows (fc2 of DeiT-S:
@@ -340,7 +340,7 @@ static bool workspace_pays(int64_t M, int64_t N, int64_t K)
 static bool workspace_pays_blocked(int64_t N, int64_t K)
 {
     if (K < 64 || K % 64 != 0) return false;
-    const char *e = getenv("ARCQ_GEMM_KERNEL");
+    const char *e = tuning().gemm_kernel;
     if (e && !strcmp(e, "prebuilt")) return true;
     const int64_t slabs = (N + 127) / 128, slices = (K / 64 + 5) / 6;
     return slices >= 3 || (slices == 2 && slabs <= 8);
@@ -360,7 +360,7 @@ bool arcq::otf_blocked_pays(int64_t M, int64_t N, int64_t K)
 {
     if (M < 512 || N <= 0 || K < 64 || K % 64 != 0 || M * K * 2 >= (int64_t(1) << 32)) return false;
     if (M >= (int64_t(1) << 31) - 256 || N >= (int64_t(1) << 31) - 256) return false;
-    const char *e = getenv("ARCQ_GEMM_KERNEL");
+    const char *e = tuning().gemm_kernel;
     if (e) return !strcmp(e, "slab8") || !strcmp(e, "prebuilt");
     return true;
 }
@@ -371,7 +371,7 @@ ARCQ_API const char *arcq_linear_otf_ws_kernel(int64_t M, int64_t N, int64_t K, 
         if (!(have_workspace && blocked_uses_workspace(N, K))) return "gemm_slab8_kernel";
         GemmArgs g{};
         g.M = static_cast<int>(M), g.N = static_cast<int>(N), g.K = static_cast<int>(K);
-        const char *e = getenv("ARCQ_PAIR");
+        const char *e = tuning().pair;
         return (e ? e[0] == '1' : gemm_pair_pays(g)) ? "gemm_pair_kernel" : "gemm_slab8_kernel<copy>";
     }
     return arcq_linear_fused_ws_kernel(M, N, K, have_workspace);
@@ -387,7 +387,7 @@ ARCQ_API const char *arcq_linear_otf_ws_kernel(int64_t M, int64_t N, int64_t K, 
 bool arcq::blocked_uses_workspace(int64_t N, int64_t K)
 {
     if (N <= 0 || K < 64 || K % 64 != 0) return false;
-    const char *e = getenv("ARCQ_GEMM_KERNEL");
+    const char *e = tuning().gemm_kernel;
     if (e) return !strcmp(e, "prebuilt");
     return true;
 }

@@ -403,8 +403,7 @@ void launch_pair_t(const GemmArgs &g, hipStream_t stream, const void *w_hat, int
 {
     auto kernel = gemm_pair_kernel<TOUT, WAVES, SG>;
     constexpr int kSmem = PairCfg<WAVES, SG>::kSmem;
-    // (Setting the attribute is cheap and idempotent; done on every call so that it holds on every device.)
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+    allow_dynamic_lds<gemm_pair_kernel<TOUT, WAVES, SG>>(kSmem);
     const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
     const int tiles = n_slabs * ranges;
     hipLaunchKernelGGL(kernel, dim3(8 * ((tiles + 7) / 8)), dim3(64 * WAVES), kSmem, stream,

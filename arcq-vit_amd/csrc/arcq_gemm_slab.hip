@@ -391,12 +391,7 @@ static void launch_slab(const GemmArgs &g, hipStream_t stream, const void *w_hat
     constexpr int L = 1 << BITS;
     const size_t smem = kSlabBytes + kStageBytes + L * 64 * sizeof(float) + kSlabN * sizeof(float);
     auto kernel = gemm_slab_kernel<BITS, TOUT, PRE>;
-    static bool configured = false;   // per instantiation; the attribute is sticky for the process
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  static_cast<int>(smem));
-        configured = true;
-    }
+    allow_dynamic_lds<gemm_slab_kernel<BITS, TOUT, PRE>>(static_cast<int>(smem));
     // One workgroup per CU where possible: split the 32-row blocks into as many ranges as CUs/slabs allow.
     const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
     const int total_blocks = (g.M + 31) / 32;

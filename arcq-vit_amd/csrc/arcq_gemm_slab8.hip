@@ -429,12 +429,7 @@ void launch_slab8_w(const GemmArgs &g, hipStream_t stream, const void *w_hat)
     constexpr int L = 1 << BITS;
     const size_t smem = kSlabBytes + WAVES * kStageTile + L * 64 * sizeof(float) + kSlabN * sizeof(float);
     auto kernel = gemm_slab8_kernel<BITS, TOUT, PRE, WAVES, AHEAD>;
-    static bool configured = false;   // per instantiation; the attribute is sticky for the process
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  static_cast<int>(smem));
-        configured = true;
-    }
+    allow_dynamic_lds<gemm_slab8_kernel<BITS, TOUT, PRE, WAVES, AHEAD>>(static_cast<int>(smem));
     // One workgroup per CU where possible: split the 32-row blocks into as many ranges as CUs/slabs allow.
     const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
     const int total_blocks = (g.M + 31) / 32;
@@ -479,7 +474,7 @@ void launch_slab8(const GemmArgs &g, hipStream_t stream, const void *w_hat)
 void launch_gemm_slab8(const GemmArgs &g, const void *w_hat, hipStream_t stream)
 {
     if (w_hat) {
-        const char *e = getenv("ARCQ_PAIR");           // tuning aid: 0 / 1 pin the choice
+        const char *e = tuning().pair;           // tuning aid: 0 / 1 pin the choice
         if (e ? e[0] == '1' : gemm_pair_pays(g)) {
             launch_gemm_pair(g, w_hat, stream);
             return;

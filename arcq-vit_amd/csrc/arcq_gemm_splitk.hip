@@ -233,12 +233,7 @@ static void launch_splitk_rb(const GemmArgs &g, hipStream_t stream)
     constexpr int kSkPitch = kSkTile * 4 + 16;
     const size_t smem = L * 64 * sizeof(float) + static_cast<size_t>(NW) * RT * kSkPitch;
     auto kernel = gemm_splitk_kernel<BITS, TOUT, NW, RB, CB>;
-    static bool configured = false;   // per instantiation; the attribute is sticky for the process
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  static_cast<int>(smem));
-        configured = true;
-    }
+    allow_dynamic_lds<gemm_splitk_kernel<BITS, TOUT, NW, RB, CB>>(static_cast<int>(smem));
     const dim3 grid((g.N + kSkTile - 1) / kSkTile, (g.M + RT - 1) / RT);
     hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), smem, stream, static_cast<const __half *>(g.x_hat), g.pw, g.cb, g.wc,
                        g.ws, g.wcs, g.bias, static_cast<TOUT *>(g.y), g.M, g.N, g.K);

@@ -330,12 +330,7 @@ static void launch_ti(const GemmArgs &g, hipStream_t stream)
     const size_t stage_bytes = size_t(4 * WM) * (4 / WM) * 32 * (64 * sizeof(TOUT) + 16);       // epilogue staging
     const size_t smem = main_bytes > stage_bytes ? main_bytes : stage_bytes;
     auto kernel = gemm_stream_kernel<BITS, TOUT, TI, WM>;
-    static bool configured = false;   // per instantiation; the attribute is sticky for the process
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  static_cast<int>(smem));
-        configured = true;
-    }
+    allow_dynamic_lds<gemm_stream_kernel<BITS, TOUT, TI, WM>>(static_cast<int>(smem));
     const int tiles = ((g.N + kBN - 1) / kBN) * ((g.M + BM - 1) / BM);
     dim3 grid(8 * ((tiles + 7) / 8));
     hipLaunchKernelGGL(kernel, grid, dim3(256 * WM), smem, stream, static_cast<const __half *>(g.x_hat), g.pw, g.cb,

@@ -358,12 +358,7 @@ static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
     const int partial_off = (tile_bytes + partial_bytes + tables <= 160 * 1024) ? tile_bytes : 0;
     const size_t smem = (partial_off ? tile_bytes + partial_bytes : (tile_bytes > partial_bytes ? tile_bytes : partial_bytes)) + tables;
     auto kernel = otf_small_kernel<TIN, BITS, TOUT, RB, LPG, CB>;
-    static int configured = 0;        // per instantiation: largest dynamic LDS size requested so far
-    if (static_cast<int>(smem) > configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  static_cast<int>(smem));
-        configured = static_cast<int>(smem);
-    }
+    allow_dynamic_lds<otf_small_kernel<TIN, BITS, TOUT, RB, LPG, CB>>(160 * 1024);      // (the size varies with K: allow the CU's whole LDS)
     const dim3 grid((a.N + kOsCols - 1) / kOsCols, (a.M + RT - 1) / RT);
     hipLaunchKernelGGL(kernel, grid, dim3(kOsWaves * 64), smem, stream, static_cast<const TIN *>(a.x), a.a_thr, a.a_cb,
                        a.pw, a.w_cb, a.wc, a.ws, a.wcs, a.bias, static_cast<__half *>(a.x_hat_ws),

@@ -68,8 +68,10 @@ def infer_packed_hparams(packed_weight_codes: torch.Tensor, weight_center: torch
                          weight_codebook: torch.Tensor) -> Dict[str, int]:
     """Hyper-parameters are not stored in a packed ``state_dict``; recover them from shapes.
 
-    ``N = packed.shape[0]``, ``G = center.shape[1]``, ``bits = log2(len(codebook))``,
-    ``K = packed.shape[1]*8 // bits``, ``gs = K // G``.
+    ``N = packed.shape[0]``, ``G = center.shape[1]``, ``bits = log2(len(codebook))``; ``K`` is the
+    row length whose packed size ``ceil(K*bits/8)`` equals ``packed.shape[1]`` and which ``G``
+    divides (a row of 3-bit codes can end inside a byte, so up to three lengths share a packed size;
+    a shape that leaves more than one of them is rejected as ambiguous), ``gs = K // G``.
     """
     levels = int(weight_codebook.numel())
     bits = levels.bit_length() - 1
@@ -77,9 +79,14 @@ def infer_packed_hparams(packed_weight_codes: torch.Tensor, weight_center: torch
         raise ValueError(f"weight_codebook has {levels} entries; expected 4, 8 or 16")
     n, pcols = packed_weight_codes.shape
     groups = int(weight_center.shape[1])
-    k = (pcols * 8) // bits
-    if groups == 0 or k % groups != 0 or (k * bits + 7) // 8 != pcols:
-        raise ValueError(f"inconsistent packed shapes: packed={tuple(packed_weight_codes.shape)} groups={groups}")
+    k_max = (pcols * 8) // bits
+    fits = [k for k in range(k_max, max(k_max - 8, 0), -1)
+            if (k * bits + 7) // 8 == pcols and groups > 0 and k % groups == 0]
+    if len(fits) != 1:
+        raise ValueError(f"{'ambiguous' if fits else 'inconsistent'} packed shapes: "
+                         f"packed={tuple(packed_weight_codes.shape)} groups={groups} bits={bits} "
+                         f"(candidate in_features: {fits})")
+    k = fits[0]
     return {"in_features": k, "out_features": int(n), "bits": bits, "group_size": k // groups}
 
 

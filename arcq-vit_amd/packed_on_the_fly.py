@@ -9,9 +9,16 @@ never exists in HBM.  ``_weight_buffer`` (the flat fp16 scratch the reference's 
 between all layers, scripts/benchmark_arcq_on_the_fly.py:182-191, read at :148-158) is honoured as
 an optional workspace: when it is set and the shape is one where rebuilding the weight once beats
 rebuilding it per row tile, the library reconstructs the weight into it and the GEMM copies from
-there; the result is bit-identical either way.  Differences a caller can observe: the input
-tensor is never overwritten (the reference overwrites a contiguous fp16 input) and statistics are
-taken in fp32 even for fp16 input.
+there; the result is bit-identical either way.
+
+Differences from the reference module that a caller can observe (all on the side of more accuracy;
+for these cases "same indices as the reference" is not pinned by any test):
+  * the input tensor is never overwritten (the reference overwrites a contiguous fp16 input);
+  * group statistics are taken in fp32 even for fp16 input (the Triton kernel reduces in fp16);
+  * an fp32 input is quantized from its fp32 values (the reference first casts x to fp16, :139);
+  * the bias is added in fp32 before the one output rounding (the reference rounds the bias to fp16);
+  * ``model.half()`` leaves the fp32 metadata (codebooks, thresholds, center/scale/code_sum, bias)
+    at their fp32 values (the reference's half chain leaves them rounded to fp16).
 """
 from __future__ import annotations
 
@@ -20,7 +27,8 @@ from typing import Dict, Optional, Tuple
 import torch
 import torch.nn as nn
 
-from . import ops
+from . import _lib, ops
+from ._lib import ARCQ_F16, ARCQ_F32
 
 # Fallback fp16 x_hat workspace, one per (device, stream), for layers that were given no ``_x_hat_buffer``: layers
 # run back to back on a stream, and stream order makes the reuse safe.  Grown on demand; ``clear_workspaces()``
@@ -80,6 +88,23 @@ class ARCQPackedLinearOnTheFly(nn.Module):
         else:
             self.register_buffer("bias_tensor", torch.empty(0))
         self.out_dtype = torch.float16
+        self._prep = None
+
+    def _prepare(self):
+        """Validated, fp32-contiguous views of the buffers and their raw pointers, built once and reused by every
+        forward until the buffers move (``_apply``, ``load_state_dict``) or are replaced."""
+        a = [ops._f32c(self.activation_thresholds), ops._f32c(self.activation_codebook)]
+        w = [self.packed_weight_codes.contiguous(), ops._f32c(self.weight_codebook), ops._f32c(self.weight_center),
+             ops._f32c(self.weight_scale), ops._f32c(self.weight_code_sum)]
+        bias = ops._f32c(self.bias_tensor) if self.bias_tensor.numel() > 0 else None
+        keep = a + w + [bias]
+        self._prep = (keep, tuple(0 if t is None else t.data_ptr() for t in keep), self.packed_weight_codes.data_ptr(),
+                      self.packed_weight_codes.device)
+        return self._prep
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self._prep = None
+        return super()._load_from_state_dict(*args, **kwargs)
 
     @classmethod
     def from_packed(cls, packed_layer: nn.Module) -> "ARCQPackedLinearOnTheFly":
@@ -98,6 +123,7 @@ class ARCQPackedLinearOnTheFly(nn.Module):
         # then widens these buffers again, scripts/benchmark_arcq_on_the_fly.py:63-85, which leaves
         # them rounded to fp16.)  Device moves still apply; dtype changes of these buffers do not.
         keep = {n: self._buffers[n] for n in self._FP32_BUFFERS if self._buffers.get(n) is not None}
+        self._prep = None
         super()._apply(fn, *args, **kwargs)
         for name, orig in keep.items():
             new = self._buffers[name]
@@ -115,19 +141,28 @@ class ARCQPackedLinearOnTheFly(nn.Module):
         if x2.dtype not in (torch.float16, torch.float32):
             x2 = x2.to(torch.float16)
         x2 = x2.contiguous()
+        m = x2.shape[0]
+        prep = self._prep
+        if prep is None or prep[2] != self.packed_weight_codes.data_ptr():
+            prep = self._prepare()
+        if prep[3] != x2.device:
+            raise RuntimeError("x and the layer's buffers must be on the same device")
         ws = getattr(self, "_x_hat_buffer", None)       # a buffer the model owns (packed_convert.share_buffers)
         if ws is None or ws.numel() < x2.numel() or ws.device != x2.device:
             ws = _workspace(x2.device, x2.numel())
-        bias = self.bias_tensor if self.bias_tensor.numel() > 0 else None
         w_ws = getattr(self, "_weight_buffer", None)
         if w_ws is not None and (not w_ws.is_cuda or w_ws.dtype != torch.float16 or not w_ws.is_contiguous()
                                  or w_ws.numel() < self.out_features * self.in_features):
             raise ValueError("_weight_buffer must be a contiguous float16 CUDA tensor of at least "
                              "out_features * in_features elements")
-        y = ops.linear_otf(x2, self.activation_thresholds, self.activation_codebook, self.packed_weight_codes,
-                           self.weight_codebook, self.weight_center, self.weight_scale, self.weight_code_sum,
-                           bias, self.bits, self.group_size, out_dtype=self.out_dtype, x_hat_ws=ws,
-                           w_hat_ws=w_ws, scratch=True)
+        y = torch.empty((m, self.out_features), dtype=self.out_dtype, device=x2.device)
+        p = prep[1]
+        with torch.cuda.device(x2.device):
+            _lib.check(_lib.load().arcq_linear_otf_ws(
+                x2.data_ptr(), ARCQ_F16 if x2.dtype == torch.float16 else ARCQ_F32, p[0], p[1], p[2], p[3], p[4], p[5],
+                p[6], p[7], ws.data_ptr(), 0 if w_ws is None else w_ws.data_ptr(), y.data_ptr(),
+                ARCQ_F16 if self.out_dtype == torch.float16 else ARCQ_F32, m, self.out_features, self.in_features,
+                self.bits, self.group_size, torch.cuda.current_stream().cuda_stream))
         return y.reshape(*original_shape[:-1], self.out_features)
 
     def estimated_persistent_mb(self) -> float:

@@ -57,6 +57,10 @@ extern "C" {
 
 int arcq_version(void);
 const char *arcq_last_error(void);
+/* The library reads its tuning variables (ARCQ_GEMM_KERNEL, ARCQ_OTF_FUSED, ARCQ_PAIR: they pin kernel choices for
+ * experiments; results are the same bits either way) once per process; this reads them again.  A hook for tests
+ * and tuning scripts with no counterpart in the reference; do not call it while other threads are inside the library. */
+void arcq_reload_tuning(void);
 
 /* ---- bit packing --------------------------------------------------------
  * Replaces pack_codes_cuda / unpack_codes_cuda / unpack_codes_u8_cuda,

@@ -28,3 +28,36 @@ def cuda():
     from arcq_vit_amd import _lib
     _lib.load()  # raises if the HIP library is not built: GPU tests must not pass without it
     return torch.device("cuda:0")
+
+
+@pytest.fixture(autouse=True)
+def _arcq_tuning_env(monkeypatch):
+    """The library reads its ARCQ_* tuning variables once per process: re-read them whenever a test changes one
+    through ``monkeypatch``, and once more after the test's changes have been undone."""
+    import os
+    from arcq_vit_amd import _lib
+    touched = []
+
+    def reload():
+        if os.path.exists(_lib.LIB_PATH):
+            _lib.reload_tuning()
+
+    orig_set, orig_del = monkeypatch.setenv, monkeypatch.delenv
+
+    def setenv(name, value, *a, **k):
+        orig_set(name, value, *a, **k)
+        if name.startswith("ARCQ_"):
+            touched.append(name)
+            reload()
+
+    def delenv(name, *a, **k):
+        orig_del(name, *a, **k)
+        if name.startswith("ARCQ_"):
+            touched.append(name)
+            reload()
+
+    monkeypatch.setenv, monkeypatch.delenv = setenv, delenv
+    yield
+    if touched:
+        monkeypatch.undo()
+        reload()

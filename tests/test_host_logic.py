@@ -276,6 +276,15 @@ def test_three_bit_conversion_sizes():
     assert hp == {"in_features": 384, "out_features": 16, "bits": 3, "group_size": 64}
     with pytest.raises(ValueError):
         A.infer_packed_hparams(layer.packed_weight_codes, layer.weight_center, torch.zeros(5))
+    # 3-bit rows that end inside a byte: K = 35 in groups of 7 packs into ceil(105 / 8) = 14 bytes, and so would 36 and
+    # 37 (the number of groups decides); K = 6, 7 or 8 in ONE group all pack into 3 bytes and cannot be told apart
+    cb8 = torch.zeros(8)
+    hp = A.infer_packed_hparams(torch.zeros(4, 14, dtype=torch.uint8), torch.zeros(4, 5), cb8)
+    assert hp == {"in_features": 35, "out_features": 4, "bits": 3, "group_size": 7}
+    with pytest.raises(ValueError, match="ambiguous"):
+        A.infer_packed_hparams(torch.zeros(4, 3, dtype=torch.uint8), torch.zeros(4, 1), cb8)
+    with pytest.raises(ValueError, match="inconsistent"):
+        A.infer_packed_hparams(torch.zeros(4, 14, dtype=torch.uint8), torch.zeros(4, 11), cb8)
 
 
 def test_fake_quant_source_matches_oracle(oracle):
@@ -356,9 +365,14 @@ def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
     assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 0) == b"gemm_slab8_kernel"
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 1) == both8
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 0) == b"gemm_slab8_kernel"
-    assert lib.arcq_linear_otf_ws_kernel(12608, 768, 768, 1) == both8                      # two slices, six slabs
-    assert lib.arcq_linear_otf_ws_kernel(50432, 4096, 1024, 1) == both8                    # three slices
+    pair = b"gemm_pair_kernel"        # several slices and at least eight row blocks per workgroup: two blocks per wave
+    assert lib.arcq_linear_otf_ws_kernel(12608, 768, 768, 1) == pair                       # two slices, six slabs
+    assert lib.arcq_linear_otf_ws_kernel(50432, 4096, 1024, 1) == pair                     # three slices
+    assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 1) == pair
+    assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 0) == b"gemm_slab8_kernel"      # (needs the weights ready)
+    monkeypatch.setenv("ARCQ_PAIR", "0")
     assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 1) == both8
+    monkeypatch.delenv("ARCQ_PAIR")
     assert lib.arcq_linear_otf_ws_kernel(1576, 384, 1536, 1) == both8                      # a ragged last block is fine
     assert lib.arcq_linear_otf_ws_kernel(197, 1152, 384, 1) == b"gemm_splitk_kernel"
     monkeypatch.setenv("ARCQ_GEMM_KERNEL", "stream")
