@@ -3,16 +3,20 @@
 
 Workload (the headline configuration): the 48 packed linears of DeiT-Small (12 blocks x qkv 384->1152,
 proj 384->384, fc1 384->1536, fc2 1536->384), W4A4, group size 64, fp16 activations in and out,
-batch 64 (M = 64*197 = 12608 tokens).  One step = one pass over all 48 layers: stage 1 (activation
-group-residual quantize + reconstruct) and the fused unpack+GEMM for each.  Inputs (one synthetic
-activation tensor per layer shape, packed weights of 48 distinct random layers) are resident in HBM
-before the timed region starts.
+batch 64 (M = 64*197 = 12608 tokens).  One step = one pass over all 48 layers through
+arcq_linear_otf_ws: stage 1 (activation group-residual quantize + reconstruct, with the layer's fp16
+weights reconstructed by extra workgroups of the same launch) and an fp16 MFMA GEMM + bias on them.
+Inputs (one synthetic activation tensor per layer shape, packed weights of 48 distinct random layers)
+are resident in HBM before the timed region starts.
 
-Prints ONE JSON line.  ``value`` is images/s of that step.  ``roofline`` is for the dominant kernel,
-the fused GEMM: algorithmic flops (2*M*N*K summed over the 48 launches of a step) divided by the
-time of those launches alone, measured here with HIP events on the launch stream in a GEMM-only
-loop.  ``cpu_baseline`` times the oracle's restatement of the reference's fake-quant CPU path
-(quantize + reconstruct activation and weight, fp32 matmul) on a bounded sample on this host.
+Prints ONE JSON line.  ``value`` is images/s of that step (packed linears only: no attention,
+LayerNorm or GELU; ``model_forward`` times the whole skeleton model next to it).  ``roofline`` is for
+the dominant kernel, the GEMM: algorithmic flops (2*M*N*K) of its launches divided by their time
+alone, measured here with HIP events on the launch stream in a GEMM-only loop; ``roofline.layer`` is
+the whole step against the same peaks; ``roofline.weights_rebuilt_inside_gemm`` the variant that
+dequantizes inside the GEMM.  ``cpu_baseline`` times the oracle's restatement of the reference's
+fake-quant CPU path (quantize + reconstruct activation and weight, fp32 matmul) on a bounded sample
+on this host.
 """
 from __future__ import annotations
 
@@ -28,22 +32,39 @@ if ROOT not in sys.path:
 
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
-# HBM bytes per launch of each fused-GEMM kernel at the default workload (average over the layer shapes it serves),
-# from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a plain 256 MiB
-# copy (factors 2.00 and 1.00).  Summary: profiles/deit_small_w4a4_bs64_packed_linears.md.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {("deit_small", 4, 64): {"gemm_slab8_kernel<copy>": 48.1e6}}
+PROFILE_NAMES = {("deit_small", 4, 64): "deit_small_w4a4_bs64_packed_linears.md",
+                 ("deit_base", 4, 64): "deit_base_w4a4_bs64_packed_linears.md",
+                 ("vit_large", 3, 256): "vit_large_w3a3_bs256_packed_linears.md"}
+
+
+def profiled_traffic(model, bits, batch, kernel):
+    """HBM bytes per launch of `kernel` (average over the layer shapes it serves) as the committed rocprofv3 summary
+    of this workload states it: two --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a
+    plain 256 MiB copy.  The summary holds one line `traffic_bytes_per_launch[<kernel>] = <bytes>` per kernel; None
+    when there is no summary or no such line."""
+    import re
+    name = PROFILE_NAMES.get((model, bits, batch))
+    if not name:
+        return None
+    try:
+        text = open(os.path.join(ROOT, "profiles", name)).read()
+    except OSError:
+        return None
+    m = re.search(r"traffic_bytes_per_launch\[" + re.escape(kernel) + r"\]\s*=\s*([0-9.eE+]+)", text)
+    return float(m.group(1)) if m else None
 
 
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--model", default="deit_small")
     ap.add_argument("--bits", type=int, default=4)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bs1", action="store_true")
+    ap.add_argument("--no-model", action="store_true", help="skip the model_forward block (whole ViT forward)")
     ap.add_argument("--eager", action="store_true",
                     help="launch every kernel from Python instead of replaying one HIP graph per step")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -128,6 +149,18 @@ class Layer:
             self.code_sum.data_ptr(), self.bias.data_ptr(), Layer.W_WS.data_ptr() if mode == "copy" else 0,
             1 if mode == "copy" else 0, y.data_ptr(), ARCQ_F16, m, self.n, self.k, self.bits, 64, stream)
 
+    def call_gemm_rebuild_inside(self, lib, ws, y, m, stream):
+        """The fused GEMM with the weights reconstructed inside the kernel (no weight workspace at all)."""
+        from arcq_vit_amd._lib import ARCQ_F16
+        if self.mode(lib, m) == "rowmajor":
+            return lib.arcq_linear_fused(ws.data_ptr(), self.packed.data_ptr(), self.cb.data_ptr(), self.center.data_ptr(),
+                                         self.scale.data_ptr(), self.code_sum.data_ptr(), self.bias.data_ptr(),
+                                         y.data_ptr(), ARCQ_F16, m, self.n, self.k, self.bits, 64, stream)
+        return lib.arcq_linear_fused_blocked(
+            ws.data_ptr(), self.packed.data_ptr(), self.cb.data_ptr(), self.center.data_ptr(), self.scale.data_ptr(),
+            self.code_sum.data_ptr(), self.bias.data_ptr(), 0, 0, y.data_ptr(), ARCQ_F16, m, self.n, self.k, self.bits,
+            64, stream)
+
     def act_args(self, x, ws, stream):
         from arcq_vit_amd._lib import ARCQ_F16
         m = x.shape[0]
@@ -205,6 +238,12 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
             if rc:
                 _lib.check(rc)
 
+    def step_gemm_inside():
+        for l in layers:
+            rc = l.call_gemm_rebuild_inside(lib, ws, y, m, stream)
+            if rc:
+                _lib.check(rc)
+
     if use_graph:
         # One HIP graph per step (the reference does this for bs <= 1,
         # scripts/benchmark_arcq_on_the_fly.py:223-231).  A launch through ctypes costs ~10 us of host
@@ -219,6 +258,8 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
                         rc = lib.arcq_linear_otf_ws(*l.otf_args(x, ws, y, sp))
                     elif kind == "act":
                         rc = l.call_act(lib, x, ws, sp)
+                    elif kind == "inside":
+                        rc = l.call_gemm_rebuild_inside(lib, ws, y, m, sp)
                     else:
                         rc = l.call_gemm(lib, ws, y, m, sp)
                     if rc:
@@ -226,11 +267,15 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
             return g.replay
         step_full()
         torch.cuda.synchronize()
+        step_gemm_inside()
+        torch.cuda.synchronize()
         step_full, step_act, step_gemm = capture("full"), capture("act"), capture("gemm")
+        step_gemm_inside = capture("inside")
 
     t_full = time_loop(step_full, steps, warmup)
     t_gemm = time_loop(step_gemm, steps, warmup)
     t_act = time_loop(step_act, steps, warmup)
+    t_inside = time_loop(step_gemm_inside, steps, warmup)
 
     # The fused entry point picks one of several kernels per shape; time each kernel's launches on their own so that
     # the roofline figure belongs to one kernel (the one with the largest share of the step).
@@ -265,6 +310,8 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
         "gemm_us_per_launch": t_gemm / steps / len(layers) * 1e6,
         "gemm_tflops": flops * steps / t_gemm / 1e12,
         "gemm_gbs": gemm_bytes * steps / t_gemm / 1e9,
+        "gemm_rebuild_inside_us_per_launch": t_inside / steps / len(layers) * 1e6,
+        "gemm_rebuild_inside_tflops": flops * steps / t_inside / 1e12,
         "act_ms_per_step": t_act / steps * 1e3,
         "act_us_per_launch": t_act / steps / len(layers) * 1e6,
         "act_gbs": act_bytes * steps / t_act / 1e9,
@@ -316,11 +363,13 @@ def cold_cache_bs1(model, bits, steps, warmup, dev, footprint_bytes=512 << 20):
             "hbm_frac": nbytes * n / t / 1e9 / PEAK_HBM_GBS}
 
 
-def cpu_baseline(layers, inputs, batch, budget_s=20.0):
-    """Oracle restatement of QuantLinearPCARCQ.forward (FQ/quant_backends.py:312-322) on host cores:
-    the four linears of ONE block at the benchmark's batch, repeated while the time budget lasts
-    (at least once); images/s = batch / (depth * time per block)."""
+def cpu_baseline(layers, inputs, batch, budget_s=12.0):
+    """Oracle restatement of QuantLinearPCARCQ.forward (FQ/quant_backends.py:312-322) on host cores: the four linears
+    of ONE block at the benchmark's batch, repeated while the time budget lasts (at least once); images/s = batch /
+    (depth * time per block).  Two figures: `value`, faithful to the reference (the weight is quantized and
+    reconstructed again on every call), and `value_weights_prebuilt` (the weight fake-quantized once beforehand)."""
     import torch
+    import torch.nn.functional as F
     from arcq_vit_amd import synth
     from oracle import arcq_ref
     block = layers[:4]
@@ -329,21 +378,90 @@ def cpu_baseline(layers, inputs, batch, budget_s=20.0):
     cb = synth.quantile_codebook(block[0].bits)
     thr = synth.midpoint_thresholds(cb)
     bs = [l.bias.cpu() for l in block]
-    with torch.no_grad():
-        arcq_ref.fake_quant_linear(xs[1][:256], block[1].w_fp32, bs[1], thr, cb, thr, cb, 64, 1e-6)  # warm up
+
+    def timed(fn, budget):
         reps, t0 = 0, time.perf_counter()
         while True:
+            fn()
+            reps += 1
+            if time.perf_counter() - t0 > budget or reps >= 8:
+                break
+        return (time.perf_counter() - t0) / reps, reps
+
+    with torch.no_grad():
+        arcq_ref.fake_quant_linear(xs[1][:256], block[1].w_fp32, bs[1], thr, cb, thr, cb, 64, 1e-6)  # warm up
+
+        def faithful():
             for l, x, b in zip(block, xs, bs):
                 arcq_ref.fake_quant_linear(x, l.w_fp32, b, thr, cb, thr, cb, 64, 1e-6)
-            reps += 1
-            if time.perf_counter() - t0 > budget_s or reps >= 8:
-                break
-        dt = (time.perf_counter() - t0) / reps
+        dt, reps = timed(faithful, budget_s)
+        wq = [arcq_ref.pcarcq_fake_quant(l.w_fp32, thr, cb, 64, 1e-6) for l in block]
+
+        def prebuilt():
+            for w, x, b in zip(wq, xs, bs):
+                F.linear(arcq_ref.pcarcq_fake_quant(x, thr, cb, 64, 1e-6), w, b)
+        dt2, reps2 = timed(prebuilt, budget_s)
     return {"value": batch / (depth * dt), "unit": "images/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"4 linears of one DeiT block at batch {batch} (M={xs[0].shape[0]}), {reps} repetitions, "
+            "sample": f"4 linears of one block at batch {batch} (M={xs[0].shape[0]}), {reps} repetitions (weights "
+                      f"re-quantized per call, as the reference does) and {reps2} (weights fake-quantized once), "
                       f"scaled by depth {depth}; torch fp32 on {torch.get_num_threads()} threads "
                       f"(os.cpu_count()={os.cpu_count()})",
-            "ms_per_block": dt * 1e3}
+            "ms_per_block": dt * 1e3, "value_weights_prebuilt": batch / (depth * dt2),
+            "ms_per_block_weights_prebuilt": dt2 * 1e3}
+
+
+def model_forward(model, bits, batches, steps, warmup, dev):
+    """Whole-model forward of the skeleton ViT (fp16 patch embedding, LayerNorm, softmax attention, GELU and head;
+    packed on-the-fly block linears with the shared scratch buffers), random-init weights, synthetic normalized
+    images: the protocol of scripts/benchmark_arcq_on_the_fly.py:202-243 (HIP graph at batch 1, eager otherwise; a
+    graph figure is given for the larger batch as well)."""
+    import torch
+    from arcq_vit_amd import synth
+    from arcq_vit_amd.vit import build_packed_vit
+    vit = build_packed_vit(model, bits, device="cuda", half_chain=True, shared_buffers=True,
+                           max_rows=max(batches) * synth.TOKENS)
+    out = {"model": model, "bits": bits, "trunk": "fp16 (patch embed, LayerNorm, attention, GELU, head)",
+           "blocks": len(vit.blocks)}
+    with torch.no_grad():
+        for b in batches:
+            x = synth.make_images(b, 1).to(dev).half()
+            n = max(steps // (4 if b > 1 else 1), 5)
+            res = {}
+            if b > 1:
+                t = time_loop(lambda: vit(x), n, max(warmup // 2, 2))
+                res["eager_images_per_s"] = b * n / t
+                res["eager_ms"] = t / n * 1e3
+            vit(x)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                vit(x)
+            t = time_loop(g.replay, n, max(warmup // 2, 2))
+            res["graph_images_per_s"] = b * n / t
+            res["graph_ms"] = t / n * 1e3
+            out[f"bs{b}"] = res
+            del g
+    return out
+
+
+def kernel_note(name):
+    if name in ("gemm_slab8_kernel<copy>", "gemm_pair_kernel"):
+        return ("fp16 MFMA GEMM + bias on weights that the stage-1 launch of the same layer reconstructed into an "
+                "fp16 workspace (copied global -> LDS); its own launch does no dequantization")
+    if name == "gemm_slab8_kernel":
+        return "packed weights reconstructed into LDS inside the kernel, fp16 MFMA GEMM + bias"
+    return "stages 2+3 fused (see arcq_linear_fused_kernel)"
+
+
+def layer_roofline(res, bits):
+    """Algorithmic flops of the step over the time of the whole step (stage 1, weight reconstruction, GEMM, gaps),
+    against the MFMA peak and against min(MFMA, HBM), the time either bound alone would allow."""
+    t = res["ms_per_step"] * 1e-3
+    flops, nbytes = res["flops_per_step"], res["gemm_bytes_per_step"]
+    t_mfma, t_hbm = flops / (PEAK_FP16_TFLOPS * 1e12), nbytes / (PEAK_HBM_GBS * 1e9)
+    return {"tflops": flops / t / 1e12, "frac_mfma": flops / t / 1e12 / PEAK_FP16_TFLOPS,
+            "gbs": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / PEAK_HBM_GBS,
+            "frac_min_mfma_hbm": max(t_mfma, t_hbm) / t, "ms_at_mfma_peak": t_mfma * 1e3, "ms_at_hbm_peak": t_hbm * 1e3}
 
 
 def main():
@@ -378,17 +496,25 @@ def main():
         "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"{args.model} {res['layers']} packed linears ({res['layers'] // 4} blocks x qkv/proj/fc1/fc2), W{args.bits}A{args.bits}, "
-                               f"g=64, batch {args.batch} (M={res['M']}), fp16 in/out, stage 1 + fused unpack+GEMM",
+                               f"g=64, batch {args.batch} (M={res['M']}), fp16 in/out; per layer: stage 1 (activation quantize + reconstruct, the fp16 weights "
+                               f"reconstructed in the same launch) then an fp16 MFMA GEMM + bias on them",
                    "model_shapes": args.model, "bits": args.bits, "batch": args.batch, "group_size": 64},
-        "roofline": {"bound": "mfma", "kernel": dom, "achieved": dk["tflops"],
+        "roofline": {"bound": "mfma", "kernel": dom, "kernel_does": kernel_note(dom), "achieved": dk["tflops"],
                      "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": dk["tflops"] / PEAK_FP16_TFLOPS,
-                     "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH.get((args.model, args.bits, args.batch), {}).get(dom),
+                     "traffic": profiled_traffic(args.model, args.bits, args.batch, dom),
                      "algorithmic_flops_per_launch": dk["flops_per_launch"],
                      "algorithmic_bytes_per_launch": dk["bytes_per_launch"],
                      "avg_launch_us": dk["us_per_launch"], "launches_per_step": dk["launches_per_step"],
                      "hbm_frac_of_same_kernel": dk["gbs"] / PEAK_HBM_GBS,
                      "all_fused_gemm_launches": {"tflops": res["gemm_tflops"], "avg_launch_us": res["gemm_us_per_launch"],
-                                                 "frac": res["gemm_tflops"] / PEAK_FP16_TFLOPS}},
+                                                 "frac": res["gemm_tflops"] / PEAK_FP16_TFLOPS},
+                     # the same GEMMs with the weights reconstructed inside the kernel (no workspace): the
+                     # "dequantization fused into the GEMM" variant, which the step does not run because it is slower
+                     "weights_rebuilt_inside_gemm": {"tflops": res["gemm_rebuild_inside_tflops"],
+                                                     "avg_launch_us": res["gemm_rebuild_inside_us_per_launch"],
+                                                     "frac": res["gemm_rebuild_inside_tflops"] / PEAK_FP16_TFLOPS},
+                     # whole layer = stage 1 (+ weight reconstruction) + GEMM, everything the step runs
+                     "layer": layer_roofline(res, args.bits)},
         "stage1": {"kernel": res["act_kernel"], "bound": "hbm", "achieved": res["act_gbs"], "peak": PEAK_HBM_GBS,
                    "unit": "GB/s", "frac": res["act_gbs"] / PEAK_HBM_GBS, "avg_launch_us": res["act_us_per_launch"]},
         "detail_bs%d" % args.batch: res,
@@ -400,6 +526,8 @@ def main():
                       "gemm_hbm_frac_warm": r1["gemm_gbs"] / PEAK_HBM_GBS, "act_us_per_launch": r1["act_us_per_launch"],
                       "hip_graph": True}
         out["bs1"]["cold_cache"] = cold_cache_bs1(args.model, args.bits, max(args.steps, 50), max(args.warmup, 10), dev)
+    if not args.no_model:
+        out["model_forward"] = model_forward(args.model, args.bits, sorted({1, args.batch}), args.steps, args.warmup, dev)
     out["launch_mode"] = "eager" if args.eager else "hip_graph_per_step"
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(layers, inputs, args.batch)
