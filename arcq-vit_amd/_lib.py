@@ -21,6 +21,23 @@ _c_int = ctypes.c_int
 _c_ptr = ctypes.c_void_p
 _c_f32 = ctypes.c_float
 
+class LinearExArgs(ctypes.Structure):
+    """``arcq_linear_ex_args`` of include/arcq_hip.h."""
+    _fields_ = [("struct_size", ctypes.c_uint32),
+                ("x_dtype", ctypes.c_int32), ("y_dtype", ctypes.c_int32), ("producer", ctypes.c_int32),
+                ("activation", ctypes.c_int32), ("bits", ctypes.c_int32), ("group_size", ctypes.c_int32),
+                ("ln_eps", ctypes.c_float),
+                ("M", ctypes.c_int64), ("N", ctypes.c_int64), ("K", ctypes.c_int64),
+                ("x", ctypes.c_void_p), ("ln_weight", ctypes.c_void_p), ("ln_bias", ctypes.c_void_p),
+                ("a_thresholds", ctypes.c_void_p), ("a_codebook", ctypes.c_void_p), ("packed_w", ctypes.c_void_p),
+                ("w_codebook", ctypes.c_void_p), ("w_center", ctypes.c_void_p), ("w_scale", ctypes.c_void_p),
+                ("w_code_sum", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("residual", ctypes.c_void_p),
+                ("x_hat_ws", ctypes.c_void_p), ("w_hat_ws", ctypes.c_void_p), ("y", ctypes.c_void_p)]
+
+
+ARCQ_PRODUCER_NONE, ARCQ_PRODUCER_LAYERNORM = 0, 1
+ARCQ_ACT_NONE, ARCQ_ACT_GELU = 0, 1
+
 # name -> argtypes, in the order of include/arcq_hip.h
 _SIGNATURES = {
     "arcq_pack_codes": [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_ptr],
@@ -40,6 +57,9 @@ _SIGNATURES = {
                            _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
     "arcq_linear_otf_static": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
+    "arcq_linear_otf_ex": [ctypes.POINTER(LinearExArgs), _c_ptr],
+    "arcq_act_quant_blocked_ln": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int,
+                                  _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr],
     "arcq_act_quant_blocked": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32, _c_ptr],
     "arcq_act_quant_blocked_with_weights": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32,
                                             _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr],

@@ -500,6 +500,155 @@ act_quant_blocked2_kernel(const TIN *__restrict__ x, const float *__restrict__ t
     }
 }
 
+// LayerNorm fused in front of the block-layout stage 1.  A workgroup owns one 32-row block and all G = K / 64 groups of
+// it, one wave per group (wave tile = 32 rows x one group, two lanes per group, as act_quant_blocked2_kernel), so the
+// row statistics LayerNorm needs are a sum over the workgroup: every lane folds its 32 values serially, the 2 G
+// partial sums of a row meet in LDS and every lane of the row adds them up in the same fixed order.
+//   mean = (sum of the partial sums, group by group, lower half first) / K
+//   var  = (the same sum over (x - mean)^2) / K
+//   y    = ((x - mean) * (1 / sqrt(var + ln_eps))) * gamma + beta        three roundings, no fma
+// y is rounded to the input's type (what a stand-alone LayerNorm kernel would have stored) and then quantized and
+// reconstructed exactly as act_quant_blocked2_kernel does.  MAXW = most waves (groups) per workgroup.
+template <typename TIN, int BITS, int MAXW>
+__global__ void __launch_bounds__(64 * MAXW)
+act_quant_rows_ln_kernel(const TIN *__restrict__ x, const float *__restrict__ gamma, const float *__restrict__ beta,
+                         float ln_eps, const float *__restrict__ thr, const float *__restrict__ cb,
+                         __half *__restrict__ x_hat, float eps, int G, int64_t rows, WeightJob wj)
+{
+    constexpr int L = 1 << BITS;
+    constexpr int kInPitch = Tile<TIN>::stride, kOutPitch = Tile<__half>::stride;     // dwords per tile row
+    constexpr int kPieces = 64 / Tile<TIN>::vec;           // 16-byte pieces per row of the tile (8 fp16 / 16 fp32)
+    constexpr int kRowsPerInstr = 64 / kPieces;            // 8 / 4
+    constexpr int kIters = 32 / kRowsPerInstr;             // 4 / 8
+    extern __shared__ __attribute__((aligned(16))) uint32_t rows_smem[];     // [G][32 * kInPitch] tiles, then [32][2 G + 1] partial sums
+    __shared__ float lut[L * 64];
+    __shared__ Bucket table[kMaxBuckets + 1];
+    __shared__ int slow_slots[MAXW];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;          // = this wave's group
+    if (blockIdx.x < wj.blocks) {       // workgroup-uniform: this workgroup rebuilds weights and is done
+        weight_dequant8_block_n<__half, BITS>(blockIdx.x, 64 * G, lut, wj.packed, wj.cb, wj.center, wj.scale, wj.code_sum,
+                                              wj.out, wj.N, wj.K, 64);
+        return;
+    }
+    const int64_t rb = blockIdx.x - wj.blocks;
+    const int64_t row_elems = static_cast<int64_t>(G) * 64;
+    uint32_t *tile = rows_smem + wave * (32 * kInPitch);
+    const int ppitch = 2 * G + 1;
+    float *part = reinterpret_cast<float *>(rows_smem + G * (32 * kInPitch));
+
+    uint4 raw[kIters];
+    {
+        const int64_t r0 = rb * 32 + lane / kPieces;
+        const TIN *p = x + r0 * row_elems + wave * 64 + (lane % kPieces) * Tile<TIN>::vec;
+#pragma unroll
+        for (int i = 0; i < kIters; ++i)         // rows past the tensor's end (a ragged last block) read as zeros
+            raw[i] = (r0 + i * kRowsPerInstr < rows) ? *reinterpret_cast<const uint4 *>(p + i * kRowsPerInstr * row_elems)
+                                                     : make_uint4(0, 0, 0, 0);
+    }
+    float th[L - 1], cbv[L];
+    load_quant_params<BITS>(thr, cb, th, cbv);
+    const BucketScale bq = pick_bucket_scale<BITS>(th);
+    build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * G);      // while the tile is on its way
+
+    const int row = lane >> 1, half = lane & 1;
+    {
+        uint32_t *dst = tile + (lane / kPieces) * kInPitch + (lane % kPieces) * 4;
+#pragma unroll
+        for (int i = 0; i < kIters; ++i) {
+            uint32_t *d = dst + i * kRowsPerInstr * kInPitch;
+            d[0] = raw[i].x; d[1] = raw[i].y; d[2] = raw[i].z; d[3] = raw[i].w;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();      // the tile is private to the wave and LDS operations execute in order
+    float xv[32];
+    {
+        const uint32_t *src = tile + row * kInPitch + half * (32 * static_cast<int>(sizeof(TIN)) / 4);
+        if constexpr (sizeof(TIN) == 4) {
+#pragma unroll
+            for (int j = 0; j < 32; ++j) xv[j] = __uint_as_float(src[j]);
+        } else {
+#pragma unroll
+            for (int p = 0; p < 16; ++p) {
+                const uint32_t w = src[p];
+                xv[2 * p] = __half2float(__ushort_as_half(static_cast<unsigned short>(w & 0xffffu)));
+                xv[2 * p + 1] = __half2float(__ushort_as_half(static_cast<unsigned short>(w >> 16)));
+            }
+        }
+    }
+    // ---- LayerNorm over the row ----
+    const float fk = static_cast<float>(row_elems);
+    auto row_total = [&](float mine) {          // sum over the row of every lane's `mine`, in the fixed order; two barriers
+        part[row * ppitch + 2 * wave + half] = mine;
+        __syncthreads();
+        float acc = 0.0f;
+        for (int i = 0; i < 2 * G; ++i) acc += part[row * ppitch + i];
+        __syncthreads();                        // (the buffer is written again right away)
+        return acc;
+    };
+    float a = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) a += xv[j];
+    const float mean = row_total(a) / fk;
+    float q = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+        xv[j] -= mean;
+        const float sq = xv[j] * xv[j];
+        q += sq;
+    }
+    const float var_row = row_total(q) / fk;
+    const float rstd = 1.0f / sqrtf(var_row + ln_eps);
+    {
+        const float4 *gp = reinterpret_cast<const float4 *>(gamma + wave * 64 + half * 32);
+        const float4 *bp = reinterpret_cast<const float4 *>(beta + wave * 64 + half * 32);
+#pragma unroll
+        for (int j4 = 0; j4 < 8; ++j4) {
+            const float4 gv = gp[j4], bv = bp[j4];
+            const float g4[4] = {gv.x, gv.y, gv.z, gv.w}, b4[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float t = xv[4 * j4 + e] * rstd;
+                const float u = t * g4[e];
+                float yv = u + b4[e];
+                if constexpr (sizeof(TIN) == 2) yv = __half2float(__float2half_rn(yv));     // what a LayerNorm kernel stores
+                xv[4 * j4 + e] = yv;
+            }
+        }
+    }
+    // ---- stage 1 on the normalized row (the tables were finished before the first barrier above) ----
+    bool table_ok = true;
+    for (int w = 0; w < G; ++w) table_ok = table_ok && (slow_slots[w] == 0);
+    float mu, var, s, sum_codes;
+    group_stats32x2(xv, eps, mu, var, s);
+    group_codes32x2<BITS>(xv, mu, var, s, th, bq, table, lut, table_ok, lane, sum_codes);
+    const float code_mean = sum_codes * 0.015625f;
+    {
+        uint32_t *dst = tile + row * kOutPitch + half * 16;
+#pragma unroll
+        for (int p = 0; p < 16; ++p) {
+            const __half2 h = __floats2half2_rn(fma_f32(s, xv[2 * p] - code_mean, mu), fma_f32(s, xv[2 * p + 1] - code_mean, mu));
+            dst[p] = *reinterpret_cast<const uint32_t *>(&h);
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    {
+        const int r = lane & 31;
+        const int nrows = static_cast<int>(rows - rb * 32 < 32 ? rows - rb * 32 : 32);     // < 32 in a ragged last block,
+        __half *base = x_hat + rb * (row_elems * 32) + (static_cast<int64_t>(wave) * 8 * nrows + r) * 8;   // stored compactly
+        if (r < nrows) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {  // instruction j: piece columns 2j and 2j + 1, nrows x 16 bytes each
+                const int kp = j * 2 + (lane >> 5);
+                const uint32_t *src = tile + r * kOutPitch + kp * 4;
+                store_writethrough16(base + kp * (nrows * 8), src[0], src[1], src[2], src[3]);
+            }
+        }
+    }
+}
+
 // Any group size: one thread per group, straight from global memory.  Slow
 // (strided reads) but has no layout assumptions; used when gs != 64 or the
 // pointers are not 16-byte aligned.
@@ -702,6 +851,69 @@ ARCQ_API int arcq_act_quant_blocked_with_weights(const void *x, int x_dtype, con
     WeightJob wj{packed_w, w_codebook, w_center, w_scale, w_code_sum, static_cast<__half *>(w_hat), N, cols,
                  static_cast<unsigned>((N * (cols / 8) + 255) / 256)};
     return act_quant_blocked_checked(x, x_dtype, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, stream, wj);
+}
+
+template <typename TIN>
+static int launch_rows_ln(const void *x, const float *gamma, const float *beta, float ln_eps, const float *thr, const float *cb,
+                          void *x_hat, int64_t rows, int64_t cols, int bits, float eps, hipStream_t stream, WeightJob wj)
+{
+    const int G = static_cast<int>(cols / 64);
+    const unsigned act_blocks = static_cast<unsigned>((rows + 31) / 32);
+    if (wj.blocks) wj.blocks = static_cast<unsigned>((wj.N * (wj.K / 8) + 64 * G - 1) / (64 * G));      // 64 G threads per block here
+    const size_t smem = (static_cast<size_t>(G) * 32 * Tile<TIN>::stride + 32 * (2 * G + 1)) * 4;
+#define ARCQ_LAUNCH_ROWS(B, W)                                                                                   \
+    do {                                                                                                         \
+        allow_dynamic_lds<act_quant_rows_ln_kernel<TIN, B, W>>(160 * 1024 - 16 * 1024);                          \
+        hipLaunchKernelGGL((act_quant_rows_ln_kernel<TIN, B, W>), dim3(act_blocks + wj.blocks), dim3(64 * G), smem, stream, \
+                           static_cast<const TIN *>(x), gamma, beta, ln_eps, thr, cb, static_cast<__half *>(x_hat), eps, G, \
+                           rows, wj);                                                                            \
+    } while (0)
+#define ARCQ_LAUNCH_ROWS_B(B) do { if (G <= 8) ARCQ_LAUNCH_ROWS(B, 8); else ARCQ_LAUNCH_ROWS(B, 16); } while (0)
+    if (bits == 4) ARCQ_LAUNCH_ROWS_B(4);
+    else if (bits == 3) ARCQ_LAUNCH_ROWS_B(3);
+    else ARCQ_LAUNCH_ROWS_B(2);
+#undef ARCQ_LAUNCH_ROWS_B
+#undef ARCQ_LAUNCH_ROWS
+    return launch_status("arcq_act_quant_blocked_ln");
+}
+
+// LayerNorm (weight ln_weight[cols], bias ln_bias[cols], fp32) followed by stage 1 into the block layout, in one
+// launch; optionally (packed_w != NULL) the same launch reconstructs w_hat[N, cols] as
+// arcq_act_quant_blocked_with_weights does.  cols / 64 must be between 1 and 16.
+ARCQ_API int arcq_act_quant_blocked_ln(const void *x, int x_dtype, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                       const float *thresholds, const float *codebook, void *x_hat_blocked,
+                                       int64_t rows, int64_t cols, int bits, float eps,
+                                       const uint8_t *packed_w, const float *w_codebook, const float *w_center,
+                                       const float *w_scale, const float *w_code_sum, void *w_hat, int64_t N, void *stream)
+{
+    if (!bits_ok(bits)) return fail(ARCQ_ERR_BITS, "arcq_act_quant_blocked_ln: bits must be 2, 3, or 4");
+    if (rows < 0 || cols < 0 || N < 0) return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked_ln: bad sizes");
+    if (cols % 64 != 0) return fail(ARCQ_ERR_GROUP, "arcq_act_quant_blocked_ln: in_features must be divisible by 64");
+    if (cols < 64 || cols > 1024)
+        return fail(ARCQ_ERR_UNSUPPORTED, "arcq_act_quant_blocked_ln: in_features must be between 64 and 1024 (got %lld)",
+                    static_cast<long long>(cols));
+    if (x_dtype != ARCQ_F32 && x_dtype != ARCQ_F16)
+        return fail(ARCQ_ERR_DTYPE, "arcq_act_quant_blocked_ln: x must be float32 or float16");
+    WeightJob wj{};
+    if (packed_w && N > 0) {
+        if (!w_codebook || !w_center || !w_scale || !w_code_sum || !w_hat)
+            return fail(ARCQ_ERR_NULL, "arcq_act_quant_blocked_ln: NULL weight tensor pointer");
+        if (!aligned(w_hat, 16) || !aligned(packed_w, 4))
+            return fail(ARCQ_ERR_ALIGN, "arcq_act_quant_blocked_ln: w_hat must be 16-byte, packed_w 4-byte aligned");
+        if (N * (cols / 8) >= (int64_t(1) << 38)) return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked_ln: weight tensor too large");
+        wj = WeightJob{packed_w, w_codebook, w_center, w_scale, w_code_sum, static_cast<__half *>(w_hat), N, cols, 1};
+    }
+    if (rows == 0 && wj.blocks == 0) return ARCQ_OK;
+    if (!x || !ln_weight || !ln_bias || !thresholds || !codebook || !x_hat_blocked)
+        return fail(ARCQ_ERR_NULL, "arcq_act_quant_blocked_ln: x, ln_weight, ln_bias, thresholds, codebook and x_hat_blocked must not be NULL");
+    if (x_hat_blocked == x) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_act_quant_blocked_ln: x_hat_blocked must not alias x");
+    if (rows * cols * 2 >= (int64_t(1) << 32)) return fail(ARCQ_ERR_SHAPE, "arcq_act_quant_blocked_ln: tensor too large");
+    if (!aligned(x, 16) || !aligned(x_hat_blocked, 16) || !aligned(ln_weight, 16) || !aligned(ln_bias, 16))
+        return fail(ARCQ_ERR_ALIGN, "arcq_act_quant_blocked_ln: x, x_hat_blocked, ln_weight and ln_bias must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (x_dtype == ARCQ_F32)
+        return launch_rows_ln<float>(x, ln_weight, ln_bias, ln_eps, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, st, wj);
+    return launch_rows_ln<__half>(x, ln_weight, ln_bias, ln_eps, thresholds, codebook, x_hat_blocked, rows, cols, bits, eps, st, wj);
 }
 
 ARCQ_API int arcq_act_quant(const void *x, int x_dtype, const float *thresholds, const float *codebook,

@@ -147,6 +147,54 @@ ARCQ_API int arcq_linear_otf_ws(const void *x, int x_dtype, const float *a_thres
                            x_hat_ws, w_hat_ws, true, y, y_dtype, M, N, K, bits, group_size, stream);
 }
 
+// The layer with LayerNorm in front and GELU / a residual behind fused in (see arcq_hip.h).
+ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
+{
+    if (!a) return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf_ex: args must not be NULL");
+    if (a->struct_size < sizeof(arcq_linear_ex_args))
+        return arcq::fail(ARCQ_ERR_SHAPE, "arcq_linear_otf_ex: struct_size %u is smaller than this library's %zu",
+                          a->struct_size, sizeof(arcq_linear_ex_args));
+    if (a->producer != ARCQ_PRODUCER_NONE && a->producer != ARCQ_PRODUCER_LAYERNORM)
+        return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: unknown producer %d", a->producer);
+    if (a->activation != ARCQ_ACT_NONE && a->activation != ARCQ_ACT_GELU)
+        return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: unknown activation %d", a->activation);
+    const bool options = a->producer != ARCQ_PRODUCER_NONE || a->activation != ARCQ_ACT_NONE || a->residual;
+    if (!options)
+        return linear_otf_impl(a->x, a->x_dtype, a->a_thresholds, a->a_codebook, a->packed_w, a->w_codebook, a->w_center,
+                               a->w_scale, a->w_code_sum, a->bias, a->x_hat_ws, a->w_hat_ws, true, a->y, a->y_dtype, a->M,
+                               a->N, a->K, a->bits, a->group_size, stream);
+    if (a->group_size != 64 || !arcq::bits_ok(a->bits) || !arcq::otf_blocked_pays(a->M, a->N, a->K))
+        return arcq::fail(ARCQ_ERR_UNSUPPORTED,
+                          "arcq_linear_otf_ex: the fused options need group_size 64, bits 2/3/4 and at least 512 rows "
+                          "(got M=%lld K=%lld group_size=%d)", static_cast<long long>(a->M), static_cast<long long>(a->K),
+                          a->group_size);
+    if (!a->x_hat_ws) return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf_ex: x_hat_ws must not be NULL");
+    if (a->x_hat_ws == a->x) return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: x_hat_ws must not alias x");
+    if (a->residual && !arcq::aligned(a->residual, 16))
+        return arcq::fail(ARCQ_ERR_ALIGN, "arcq_linear_otf_ex: residual must be 16-byte aligned");
+    const bool carry = a->w_hat_ws && arcq::blocked_uses_workspace(a->N, a->K) && a->packed_w && a->w_codebook && a->w_center &&
+                       a->w_scale && a->w_code_sum && arcq::aligned(a->w_hat_ws, 16) && arcq::aligned(a->packed_w, 16);
+    int rc;
+    if (a->producer == ARCQ_PRODUCER_LAYERNORM) {
+        if (a->K > 1024)
+            return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: the fused LayerNorm needs in_features <= 1024");
+        rc = arcq_act_quant_blocked_ln(a->x, a->x_dtype, a->ln_weight, a->ln_bias, a->ln_eps, a->a_thresholds, a->a_codebook,
+                                       a->x_hat_ws, a->M, a->K, a->bits, 1.0e-6f, carry ? a->packed_w : nullptr, a->w_codebook,
+                                       a->w_center, a->w_scale, a->w_code_sum, a->w_hat_ws, carry ? a->N : 0, stream);
+    } else if (carry) {
+        rc = arcq_act_quant_blocked_with_weights(a->x, a->x_dtype, a->a_thresholds, a->a_codebook, a->x_hat_ws, a->M, a->K,
+                                                 a->bits, 1.0e-6f, a->packed_w, a->w_codebook, a->w_center, a->w_scale,
+                                                 a->w_code_sum, a->w_hat_ws, a->N, stream);
+    } else {
+        rc = arcq_act_quant_blocked(a->x, a->x_dtype, a->a_thresholds, a->a_codebook, a->x_hat_ws, a->M, a->K, a->bits, 1.0e-6f,
+                                    stream);
+    }
+    if (rc != ARCQ_OK) return rc;
+    return arcq::linear_fused_blocked(a->x_hat_ws, a->packed_w, a->w_codebook, a->w_center, a->w_scale, a->w_code_sum, a->bias,
+                                      a->w_hat_ws, carry, a->y, a->y_dtype, a->M, a->N, a->K, a->bits, a->group_size, stream,
+                                      a->residual, a->activation == ARCQ_ACT_GELU);
+}
+
 // ---- the same layer for callers that cannot allocate --------------------------------------------------------
 // Both scratch buffers of arcq_linear_otf_ws live in a file-scope device array instead of caller memory.  Every GPU
 // the library runs on holds its own copy of the array (at its own address) until the process ends.

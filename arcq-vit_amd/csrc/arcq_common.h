@@ -114,4 +114,38 @@ template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ __half from_float<__half>(float v) { return __float2half_rn(v); }
 
+// Optional elementwise work on a GEMM's outputs after they have been rounded to the output type, each step rounding
+// to that type again -- the values separate elementwise kernels on the stored tensor would produce:
+//   gelu:     y = round(gelu(y)),  gelu(v) = (v * 0.5) * (1 + erf(v * sqrt(1/2)))    (the exact, erf-based GELU)
+//   residual: y = round(y + r)     r [M,N] of the output type (e.g. the transformer block's skip connection)
+// `v` holds 16 bytes of consecutive outputs of one row (8 fp16 or 4 fp32), `res` points at the residual values of the
+// same positions (or is nullptr), of which the first `valid` may be read.
+template <typename TOUT>
+__device__ __forceinline__ void post_ops16(u32x4_store_t &v, const TOUT *res, bool gelu, int valid)
+{
+    constexpr int n = 16 / static_cast<int>(sizeof(TOUT));
+    TOUT e[n];
+    __builtin_memcpy(e, &v, 16);
+    if (gelu) {
+#pragma unroll
+        for (int i = 0; i < n; ++i) {
+            const float x = to_float(e[i]);
+            e[i] = from_float<TOUT>((x * 0.5f) * (1.0f + erff(x * 0.70710678118654752440f)));
+        }
+    }
+    if (res) {
+        TOUT r[n];
+        if (valid >= n && (reinterpret_cast<uintptr_t>(res) & 15) == 0) {
+            const u32x4_store_t rv = *reinterpret_cast<const u32x4_store_t *>(res);
+            __builtin_memcpy(r, &rv, 16);
+        } else {
+#pragma unroll
+            for (int i = 0; i < n; ++i) r[i] = i < valid ? res[i] : from_float<TOUT>(0.0f);
+        }
+#pragma unroll
+        for (int i = 0; i < n; ++i) e[i] = from_float<TOUT>(to_float(e[i]) + to_float(r[i]));
+    }
+    __builtin_memcpy(&v, e, 16);
+}
+
 }  // namespace arcq

@@ -15,6 +15,10 @@ struct GemmArgs {
     void *y;                 // [M,N]
     bool y_f16;
     int M, N, K, bits;
+    // Post-operations on the rounded outputs (arcq_common.h, post_ops16); only the block-layout kernels
+    // (launch_gemm_slab8, launch_gemm_pair) apply them, the entry points keep them away from the others.
+    const void *residual = nullptr;   // [M,N] of y's type, or nullptr
+    bool gelu = false;
 };
 
 // Large-M kernel (256-column x up-to-256-row workgroup tiles); requires K >= 64.
@@ -41,7 +45,7 @@ bool blocked_uses_workspace(int64_t N, int64_t K);
 int linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_w, const float *w_codebook,
                          const float *w_center, const float *w_scale, const float *w_code_sum, const float *bias,
                          void *w_hat_ws, bool w_hat_ready, void *y, int y_dtype, int64_t M, int64_t N, int64_t K, int bits,
-                         int group_size, void *stream);
+                         int group_size, void *stream, const void *residual = nullptr, bool gelu = false);
 
 
 // Small-M kernel (64 x 64 tiles, K split across the waves of a workgroup); requires K >= 64.

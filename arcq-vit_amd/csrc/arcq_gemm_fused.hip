@@ -407,7 +407,7 @@ ARCQ_API int arcq_linear_fused_blocked(const void *x_hat_blocked,
 int arcq::linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_w, const float *w_codebook,
                                const float *w_center, const float *w_scale, const float *w_code_sum, const float *bias,
                                void *w_hat_ws, bool w_hat_ready, void *y, int y_dtype, int64_t M, int64_t N, int64_t K,
-                               int bits, int group_size, void *stream)
+                               int bits, int group_size, void *stream, const void *residual, bool gelu)
 {
     if (!bits_ok(bits)) return fail(ARCQ_ERR_BITS, "arcq_linear_fused_blocked: bits must be 2, 3, or 4");
     if (group_size != 64) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_fused_blocked: group_size must be 64 (got %d)", group_size);
@@ -432,6 +432,8 @@ int arcq::linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_
     }
     GemmArgs g{x_hat_blocked, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype == ARCQ_F16,
                static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), bits};
+    g.residual = residual;
+    g.gelu = gelu;
     launch_gemm_slab8(g, prebuilt ? w_hat_ws : nullptr, st);
     return launch_status("arcq_linear_fused_blocked");
 }

@@ -45,7 +45,8 @@ template <int WAVES, int SG> struct PairCfg {
 template <typename TOUT, int WAVES, int SG>
 __global__ void __launch_bounds__(64 * WAVES)
 gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K,
-                 int row_ranges, int blocks_per_range, const __half *__restrict__ w_hat)
+                 int row_ranges, int blocks_per_range, const __half *__restrict__ w_hat,
+                 const TOUT *__restrict__ residual, int gelu)
 {
     constexpr int kWaves = WAVES;
     constexpr int kSliceGroups = SG;
@@ -262,6 +263,13 @@ gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, 
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     v[i] = *reinterpret_cast<const u32x4_t *>(stage + (i * 8 + (lane >> 3)) * kStageRow + (lane & 7) * 16);
+                if (residual || gelu) {          // wave-uniform
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (row0 + i * 8 < M && col < N)
+                            post_ops16<TOUT>(v[i], residual ? residual + static_cast<int64_t>(row0 + i * 8) * N + col : nullptr,
+                                             gelu != 0, (N % kVec) == 0 ? kVec : N - col);
+                }
                 if (whole) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
@@ -408,7 +416,8 @@ void launch_pair_t(const GemmArgs &g, hipStream_t stream, const void *w_hat, int
     const int tiles = n_slabs * ranges;
     hipLaunchKernelGGL(kernel, dim3(8 * ((tiles + 7) / 8)), dim3(64 * WAVES), kSmem, stream,
                        static_cast<const __half *>(g.x_hat), g.bias, static_cast<TOUT *>(g.y), g.M, g.N, g.K, ranges,
-                       blocks_per_range, static_cast<const __half *>(w_hat));
+                       blocks_per_range, static_cast<const __half *>(w_hat), static_cast<const TOUT *>(g.residual),
+                       g.gelu ? 1 : 0);
 }
 
 }  // namespace

@@ -77,7 +77,8 @@ __global__ void __launch_bounds__(64 * WAVES)
 gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw, const float *__restrict__ cb,
                   const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
                   const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K,
-                  int row_ranges, int blocks_per_range, const __half *__restrict__ w_hat)
+                  int row_ranges, int blocks_per_range, const __half *__restrict__ w_hat,
+                  const TOUT *__restrict__ residual, int gelu)
 {
     constexpr int L = 1 << BITS;
     constexpr int kWaves = WAVES;
@@ -387,6 +388,13 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
 #pragma unroll
                     for (int i = 0; i < kStoreBatch; ++i)
                         v[i] = *reinterpret_cast<const u32x4_t *>(stage + ((ib + i) * 8 + (lane >> 3)) * kStageRow + (lane & 7) * 16);
+                    if (residual || gelu) {          // wave-uniform
+#pragma unroll
+                        for (int i = 0; i < kStoreBatch; ++i)
+                            if (row0 + (ib + i) * 8 < M && col < N)
+                                post_ops16<TOUT>(v[i], residual ? residual + static_cast<int64_t>(row0 + (ib + i) * 8) * N + col : nullptr,
+                                                 gelu != 0, (N % kVec) == 0 ? kVec : N - col);
+                    }
                     if (whole) {
 #pragma unroll
                         for (int i = 0; i < kStoreBatch; ++i)
@@ -442,7 +450,7 @@ void launch_slab8_w(const GemmArgs &g, hipStream_t stream, const void *w_hat)
     hipLaunchKernelGGL(kernel, dim3(8 * ((tiles + 7) / 8)), dim3(64 * WAVES), smem, stream,
                        static_cast<const __half *>(g.x_hat), g.pw, g.cb, g.wc, g.ws, g.wcs, g.bias,
                        static_cast<TOUT *>(g.y), g.M, g.N, g.K, ranges, blocks_per_range,
-                       static_cast<const __half *>(w_hat));
+                       static_cast<const __half *>(w_hat), static_cast<const TOUT *>(g.residual), g.gelu ? 1 : 0);
 }
 
 // Waves per workgroup.  While one wave of a SIMD writes its block out (2-2.5 us per pass: the stores queue behind

@@ -11,11 +11,12 @@ namespace arcq {
 // of the flattened tensor.  `lut` is an LDS array of
 // (1 << BITS) * 64 floats that this call fills with the codebook replicated per lane (conflict-free lookups); every
 // thread of the workgroup must call it (it contains a barrier).
-template <typename TOUT, int BITS, int THREADS = 256>
-__device__ __forceinline__ void weight_dequant8_block(int64_t block, float *lut, const uint8_t *__restrict__ packed,
-                                                      const float *__restrict__ cb, const float *__restrict__ center,
-                                                      const float *__restrict__ scale, const float *__restrict__ code_sum,
-                                                      TOUT *__restrict__ out, int64_t N, int64_t K, int gs)
+// `threads` = number of participating threads per workgroup (a template constant in the overload below).
+template <typename TOUT, int BITS>
+__device__ __forceinline__ void weight_dequant8_block_n(int64_t block, int threads, float *lut, const uint8_t *__restrict__ packed,
+                                                        const float *__restrict__ cb, const float *__restrict__ center,
+                                                        const float *__restrict__ scale, const float *__restrict__ code_sum,
+                                                        TOUT *__restrict__ out, int64_t N, int64_t K, int gs)
 {
     constexpr int L = 1 << BITS;
     const int lane = threadIdx.x & 63;
@@ -26,7 +27,7 @@ __device__ __forceinline__ void weight_dequant8_block(int64_t block, float *lut,
     __syncthreads();
 
     const int64_t chunks_per_row = K / 8;
-    const int64_t idx = block * THREADS + threadIdx.x;
+    const int64_t idx = block * threads + threadIdx.x;
     if (idx >= N * chunks_per_row) return;
     const int64_t n = idx / chunks_per_row;
     const int64_t k0 = (idx - n * chunks_per_row) * 8;
@@ -62,6 +63,15 @@ __device__ __forceinline__ void weight_dequant8_block(int64_t block, float *lut,
         reinterpret_cast<float4 *>(dst)[0] = make_float4(v[0], v[1], v[2], v[3]);
         reinterpret_cast<float4 *>(dst)[1] = make_float4(v[4], v[5], v[6], v[7]);
     }
+}
+
+template <typename TOUT, int BITS, int THREADS = 256>
+__device__ __forceinline__ void weight_dequant8_block(int64_t block, float *lut, const uint8_t *__restrict__ packed,
+                                                      const float *__restrict__ cb, const float *__restrict__ center,
+                                                      const float *__restrict__ scale, const float *__restrict__ code_sum,
+                                                      TOUT *__restrict__ out, int64_t N, int64_t K, int gs)
+{
+    weight_dequant8_block_n<TOUT, BITS>(block, THREADS, lut, packed, cb, center, scale, code_sum, out, N, K, gs);
 }
 
 }  // namespace arcq

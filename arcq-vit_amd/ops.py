@@ -12,6 +12,7 @@ kernels are enqueued on torch's current stream.  Nothing here synchronises.
 """
 from __future__ import annotations
 
+import ctypes
 from typing import List, Optional
 
 import torch
@@ -340,6 +341,85 @@ def quantize_activation_blocked(x: torch.Tensor, thresholds: torch.Tensor, codeb
                 _ptr(x), _dtype_code(x, "x"), _ptr(thr), _ptr(cbk), _ptr(out), m, k, bits, 1.0e-6,
                 _ptr(packed_w), *[_ptr(t) for t in meta], _ptr(w_hat), n, _stream()))
     return out
+
+
+def quantize_activation_blocked_ln(x: torch.Tensor, ln_weight: torch.Tensor, ln_bias: torch.Tensor, ln_eps: float,
+                                   thresholds: torch.Tensor, codebook: torch.Tensor, bits: int,
+                                   out: Optional[torch.Tensor] = None, weights=None,
+                                   w_hat: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``quantize_activation_blocked`` of ``LayerNorm(x)`` (over the last dimension, result rounded to ``x``'s
+    dtype) in one launch; ``64 <= K <= 1024``.  ``weights`` / ``w_hat`` as there."""
+    _check(x.is_cuda and x.dim() == 2, "x must be a CUDA tensor [M, K]")
+    _check_bits(bits)
+    x = x.contiguous()
+    m, k = x.shape
+    _check(k % 64 == 0 and 64 <= k <= 1024, "the fused LayerNorm needs K divisible by 64 and at most 1024")
+    if out is None:
+        shape = (m // 32, k // 8, 32, 8) if m % 32 == 0 else (m * k,)
+        out = torch.empty(shape, dtype=torch.float16, device=x.device)
+    else:
+        _check(out.is_cuda and out.dtype == torch.float16 and out.is_contiguous() and out.numel() >= m * k,
+               "out must be a contiguous float16 CUDA buffer of at least M*K elements")
+    thr, cbk, g, b = _f32c(thresholds), _f32c(codebook), _f32c(ln_weight), _f32c(ln_bias)
+    _check(g.numel() == k and b.numel() == k, "ln_weight and ln_bias must have K elements")
+    wp = [0, 0, 0, 0, 0, 0, 0]
+    keep = None
+    if weights is not None:
+        packed_w = weights[0].contiguous()
+        n = packed_w.shape[0]
+        _check(w_hat is not None, "weights need a w_hat buffer")
+        _check_w_ws(w_hat, n, k)
+        keep = [packed_w] + [_f32c(t) for t in weights[1:]]
+        wp = [_ptr(t) for t in keep] + [_ptr(w_hat), n]
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().arcq_act_quant_blocked_ln(
+            _ptr(x), _dtype_code(x, "x"), _ptr(g), _ptr(b), float(ln_eps), _ptr(thr), _ptr(cbk), _ptr(out), m, k, bits,
+            1.0e-6, *wp, _stream()))
+    return out
+
+
+def linear_otf_ex(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Tensor, packed_w: torch.Tensor,
+                  w_codebook: torch.Tensor, w_center: torch.Tensor, w_scale: torch.Tensor, w_code_sum: torch.Tensor,
+                  bias: Optional[torch.Tensor], bits: int, group_size: int, out_dtype: torch.dtype = torch.float16,
+                  layernorm=None, gelu: bool = False, residual: Optional[torch.Tensor] = None,
+                  x_hat_ws: Optional[torch.Tensor] = None, w_hat_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``residual + gelu(linear(stage1(LayerNorm(x))))`` with the optional parts fused into the layer's two launches
+    (``arcq_linear_otf_ex``): ``layernorm = (weight, bias, eps)`` or None, ``residual`` ``[M, N]`` of ``out_dtype`` or
+    None.  Raises ``RuntimeError`` where the library does not fuse (fewer than 512 rows, K > 1024 with LayerNorm)."""
+    _check(x.is_cuda and packed_w.is_cuda, "x and packed_w must be CUDA tensors")
+    _check(x.dim() == 2, "x must have shape [M, K]")
+    _check_bits(bits)
+    x = x.contiguous()
+    m, k = x.shape
+    n = packed_w.shape[0]
+    _check(packed_w.shape[1] == (k * bits + 7) // 8, "packed_w row length does not match K*bits/8")
+    if x_hat_ws is None:
+        x_hat_ws = torch.empty(m * k, dtype=torch.float16, device=x.device)
+    y = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    keep = [_f32c(a_thresholds), _f32c(a_codebook), packed_w.contiguous(), _f32c(w_codebook), _f32c(w_center),
+            _f32c(w_scale), _f32c(w_code_sum), None if bias is None or bias.numel() == 0 else _f32c(bias)]
+    a = _lib.LinearExArgs()
+    a.struct_size = ctypes.sizeof(_lib.LinearExArgs)
+    a.x_dtype, a.y_dtype = _dtype_code(x, "x"), _dtype_code(y, "y")
+    a.bits, a.group_size, a.M, a.N, a.K = bits, int(group_size), m, n, k
+    a.x = _ptr(x)
+    if layernorm is not None:
+        lw, lb, eps = layernorm
+        lw, lb = _f32c(lw), _f32c(lb)
+        keep += [lw, lb]
+        a.producer, a.ln_weight, a.ln_bias, a.ln_eps = _lib.ARCQ_PRODUCER_LAYERNORM, _ptr(lw), _ptr(lb), float(eps)
+    a.activation = _lib.ARCQ_ACT_GELU if gelu else _lib.ARCQ_ACT_NONE
+    (a.a_thresholds, a.a_codebook, a.packed_w, a.w_codebook, a.w_center, a.w_scale, a.w_code_sum,
+     a.bias) = [_ptr(t) or None for t in keep[:8]]
+    if residual is not None:
+        _check(residual.is_cuda and residual.dtype == out_dtype and residual.is_contiguous()
+               and tuple(residual.shape) == (m, n), "residual must be a contiguous [M, N] tensor of the output dtype")
+        a.residual = _ptr(residual)
+    _check_w_ws(w_hat_ws, n, k)
+    a.x_hat_ws, a.w_hat_ws, a.y = _ptr(x_hat_ws), _ptr(w_hat_ws) or None, _ptr(y)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().arcq_linear_otf_ex(ctypes.byref(a), _stream()))
+    return y
 
 
 def linear_fused_blocked(x_hat_blocked: torch.Tensor, m: int, k: int, packed_w: torch.Tensor, w_codebook: torch.Tensor,

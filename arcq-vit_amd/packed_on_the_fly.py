@@ -22,6 +22,7 @@ for these cases "same indices as the reference" is not pinned by any test):
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Dict, Optional, Tuple
 
 import torch
@@ -131,17 +132,38 @@ class ARCQPackedLinearOnTheFly(nn.Module):
                 self._buffers[name] = orig.to(device=new.device)
         return self
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, layernorm: Optional[nn.LayerNorm] = None, activation: Optional[str] = None,
+                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``residual + activation(linear(stage1(layernorm(x))))``.  The three optional parts (the LayerNorm in front
+        of the layer, ``activation="gelu"`` and the skip connection behind it, as they surround the block linears in
+        timm's ``Block``, FQ/timm_quant_models.py:63-121) are fused into the layer's two launches where the library
+        can (512 rows or more, group size 64, K <= 1024 for the LayerNorm) and run as separate torch operations
+        otherwise; without them this is the reference module's forward."""
         original_shape = x.shape
         if original_shape[-1] != self.in_features:
             raise ValueError(f"expected last dim {self.in_features}, got {original_shape[-1]}")
         if not x.is_cuda or not self.packed_weight_codes.is_cuda:
             raise RuntimeError("x and the layer's buffers must be CUDA tensors (there is no CPU forward)")
+        if activation not in (None, "gelu"):
+            raise ValueError(f"activation must be None or 'gelu', got {activation!r}")
         x2 = x.reshape(-1, self.in_features)
         if x2.dtype not in (torch.float16, torch.float32):
             x2 = x2.to(torch.float16)
         x2 = x2.contiguous()
         m = x2.shape[0]
+        extras = layernorm is not None or activation is not None or residual is not None
+        fuse = (extras and m >= 512 and self.group_size == 64 and self.in_features % 64 == 0
+                and (layernorm is None or (self.in_features <= 1024 and layernorm.elementwise_affine
+                                           and tuple(layernorm.normalized_shape) == (self.in_features,))))
+        if extras and not fuse:          # separate operations around the plain layer
+            if layernorm is not None:
+                x2 = layernorm(x2)
+            y = self.forward(x2)
+            if activation == "gelu":
+                y = torch.nn.functional.gelu(y)
+            if residual is not None:
+                y = y + residual.reshape(-1, self.out_features)
+            return y.reshape(*original_shape[:-1], self.out_features)
         prep = self._prep
         if prep is None or prep[2] != self.packed_weight_codes.data_ptr():
             prep = self._prepare()
@@ -157,13 +179,55 @@ class ARCQPackedLinearOnTheFly(nn.Module):
                              "out_features * in_features elements")
         y = torch.empty((m, self.out_features), dtype=self.out_dtype, device=x2.device)
         p = prep[1]
+        f16 = ARCQ_F16 if x2.dtype == torch.float16 else ARCQ_F32
+        y16 = ARCQ_F16 if self.out_dtype == torch.float16 else ARCQ_F32
+        stream = torch.cuda.current_stream().cuda_stream
         with torch.cuda.device(x2.device):
-            _lib.check(_lib.load().arcq_linear_otf_ws(
-                x2.data_ptr(), ARCQ_F16 if x2.dtype == torch.float16 else ARCQ_F32, p[0], p[1], p[2], p[3], p[4], p[5],
-                p[6], p[7], ws.data_ptr(), 0 if w_ws is None else w_ws.data_ptr(), y.data_ptr(),
-                ARCQ_F16 if self.out_dtype == torch.float16 else ARCQ_F32, m, self.out_features, self.in_features,
-                self.bits, self.group_size, torch.cuda.current_stream().cuda_stream))
+            if not extras:
+                _lib.check(_lib.load().arcq_linear_otf_ws(
+                    x2.data_ptr(), f16, p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7], ws.data_ptr(),
+                    0 if w_ws is None else w_ws.data_ptr(), y.data_ptr(), y16, m, self.out_features, self.in_features,
+                    self.bits, self.group_size, stream))
+            else:
+                a = _lib.LinearExArgs()
+                a.struct_size = ctypes.sizeof(_lib.LinearExArgs)
+                a.x_dtype, a.y_dtype, a.bits, a.group_size = f16, y16, self.bits, self.group_size
+                a.M, a.N, a.K = m, self.out_features, self.in_features
+                a.x = x2.data_ptr()
+                keep = []
+                if layernorm is not None:
+                    lw, lb = self._layernorm_params(layernorm)
+                    keep = [lw, lb]
+                    a.producer, a.ln_weight, a.ln_bias, a.ln_eps = (_lib.ARCQ_PRODUCER_LAYERNORM, lw.data_ptr(),
+                                                                   lb.data_ptr(), float(layernorm.eps))
+                a.activation = _lib.ARCQ_ACT_GELU if activation == "gelu" else _lib.ARCQ_ACT_NONE
+                (a.a_thresholds, a.a_codebook, a.packed_w, a.w_codebook, a.w_center, a.w_scale, a.w_code_sum,
+                 a.bias) = [v or None for v in p]
+                if residual is not None:
+                    r2 = residual.reshape(-1, self.out_features)
+                    if r2.dtype != self.out_dtype or tuple(r2.shape) != (m, self.out_features) or r2.device != x2.device:
+                        raise ValueError("residual must have the output's shape, dtype and device")
+                    r2 = r2.contiguous()
+                    keep.append(r2)
+                    a.residual = r2.data_ptr()
+                a.x_hat_ws, a.w_hat_ws, a.y = ws.data_ptr(), (None if w_ws is None else w_ws.data_ptr()), y.data_ptr()
+                _lib.check(_lib.load().arcq_linear_otf_ex(ctypes.byref(a), stream))
         return y.reshape(*original_shape[:-1], self.out_features)
+
+    def _layernorm_params(self, layernorm: nn.LayerNorm):
+        """fp32 copies of a LayerNorm's weight and bias, cached per LayerNorm module and parameter version."""
+        cache = self.__dict__.setdefault("_ln_cache", {})
+        key = id(layernorm)
+        ver = (layernorm.weight._version, layernorm.weight.data_ptr(),
+               None if layernorm.bias is None else layernorm.bias._version)
+        hit = cache.get(key)
+        if hit is None or hit[0] != ver:
+            w = layernorm.weight.detach().to(torch.float32).contiguous()
+            b = (torch.zeros_like(w) if layernorm.bias is None
+                 else layernorm.bias.detach().to(torch.float32).contiguous())
+            hit = (ver, w, b)
+            cache[key] = hit
+        return hit[1], hit[2]
 
     def estimated_persistent_mb(self) -> float:
         """MiB held by this layer's buffers (FQ/arcq_packed_on_the_fly.py:163-169)."""

@@ -37,12 +37,15 @@ class Attention(nn.Module):
         self.qkv = linear(dim, dim * 3, True)
         self.proj = linear(dim, dim, True)
 
+    def mix(self, qkv: torch.Tensor) -> torch.Tensor:
+        """Softmax attention on the output of ``qkv`` ``[B, tokens, 3 C]`` -> ``[B, tokens, C]`` (input of ``proj``)."""
+        b, n, c3 = qkv.shape
+        c = c3 // 3
+        q, k, v = qkv.reshape(b, n, 3, self.num_heads, c // self.num_heads).permute(2, 0, 3, 1, 4).unbind(0)
+        return F.scaled_dot_product_attention(q, k, v).transpose(1, 2).reshape(b, n, c)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        b, n, c = x.shape
-        qkv = self.qkv(x).reshape(b, n, 3, self.num_heads, c // self.num_heads).permute(2, 0, 3, 1, 4)
-        q, k, v = qkv.unbind(0)
-        y = F.scaled_dot_product_attention(q, k, v)
-        return self.proj(y.transpose(1, 2).reshape(b, n, c))
+        return self.proj(self.mix(self.qkv(x)))
 
 
 class Mlp(nn.Module):
@@ -63,8 +66,15 @@ class Block(nn.Module):
         self.attn = Attention(dim, heads, linear)
         self.norm2 = nn.LayerNorm(dim, eps=1e-6)
         self.mlp = Mlp(dim, hidden, linear)
+        # True (and the four linears on-the-fly packed layers): the LayerNorms, the GELU and the two skip connections
+        # run inside the packed layers' launches (ARCQPackedLinearOnTheFly.forward's optional arguments).
+        self.fuse_elementwise = False
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.fuse_elementwise and isinstance(self.mlp.act, nn.GELU) and self.mlp.act.approximate == "none":
+            a = self.attn
+            x = a.proj(a.mix(a.qkv(x, layernorm=self.norm1)), residual=x)
+            return self.mlp.fc2(self.mlp.fc1(x, layernorm=self.norm2, activation="gelu"), residual=x)
         x = x + self.attn(self.norm1(x))
         return x + self.mlp(self.norm2(x))
 
@@ -122,11 +132,12 @@ def build_fakequant_vit(model: str, bits: int, group_size: int = 64, seed: int =
 
 def build_packed_vit(model: str, bits: int, group_size: int = 64, seed: int = SEED, num_classes: int = 1000,
                      device: str = "cuda", half_chain: bool = True, depth: Optional[int] = None,
-                     shared_buffers: bool = False, max_rows: int = 0) -> VisionTransformer:
+                     shared_buffers: bool = False, max_rows: int = 0, fuse_elementwise: bool = False) -> VisionTransformer:
     """Fake-quant ViT -> packed (``convert_arcq_linear_to_packed``) -> on-the-fly layers -> device,
     the sequence of scripts/benchmark_arcq_on_the_fly.py:88-199.  ``half_chain`` casts the
     floating-point rest of the model to fp16 (packed metadata stays fp32).  ``shared_buffers`` gives all
-    layers one weight scratch buffer (:182-191 there) and, with ``max_rows`` tokens, one x_hat buffer."""
+    layers one weight scratch buffer (:182-191 there) and, with ``max_rows`` tokens, one x_hat buffer.
+    ``fuse_elementwise``: LayerNorm, GELU and the skip connections run inside the packed layers' launches."""
     vit = build_fakequant_vit(model, bits, group_size, seed, num_classes, depth)
     convert_arcq_linear_to_packed(vit, runtime_code_format="packed")
     to_on_the_fly(vit)
@@ -135,4 +146,6 @@ def build_packed_vit(model: str, bits: int, group_size: int = 64, seed: int = SE
         vit = vit.half()
     if shared_buffers:
         share_buffers(vit, max_rows)
+    for blk in vit.blocks:
+        blk.fuse_elementwise = bool(fuse_elementwise)
     return vit.eval()

@@ -414,33 +414,42 @@ def model_forward(model, bits, batches, steps, warmup, dev):
     """Whole-model forward of the skeleton ViT (fp16 patch embedding, LayerNorm, softmax attention, GELU and head;
     packed on-the-fly block linears with the shared scratch buffers), random-init weights, synthetic normalized
     images: the protocol of scripts/benchmark_arcq_on_the_fly.py:202-243 (HIP graph at batch 1, eager otherwise; a
-    graph figure is given for the larger batch as well)."""
+    graph figure is given for the larger batch as well).  Two models: the block's LayerNorms, GELU and skip connections
+    as separate torch kernels (`unfused`, the reference's structure) and inside the packed layers' launches
+    (`fused_elementwise`; below 512 rows the layers run them separately, so batch 1 shows no difference)."""
     import torch
     from arcq_vit_amd import synth
     from arcq_vit_amd.vit import build_packed_vit
-    vit = build_packed_vit(model, bits, device="cuda", half_chain=True, shared_buffers=True,
-                           max_rows=max(batches) * synth.TOKENS)
-    out = {"model": model, "bits": bits, "trunk": "fp16 (patch embed, LayerNorm, attention, GELU, head)",
-           "blocks": len(vit.blocks)}
-    with torch.no_grad():
-        for b in batches:
-            x = synth.make_images(b, 1).to(dev).half()
-            n = max(steps // (4 if b > 1 else 1), 5)
-            res = {}
-            if b > 1:
-                t = time_loop(lambda: vit(x), n, max(warmup // 2, 2))
-                res["eager_images_per_s"] = b * n / t
-                res["eager_ms"] = t / n * 1e3
-            vit(x)
-            torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
+    out = {"model": model, "bits": bits, "trunk": "fp16 (patch embed, LayerNorm, attention, GELU, head)"}
+    for name, fuse in (("unfused", False), ("fused_elementwise", True)):
+        vit = build_packed_vit(model, bits, device="cuda", half_chain=True, shared_buffers=True,
+                               max_rows=max(batches) * synth.TOKENS, fuse_elementwise=fuse)
+        out["blocks"] = len(vit.blocks)
+        part = {}
+        with torch.no_grad():
+            for b in batches:
+                if fuse and b * synth.TOKENS < 512:
+                    continue
+                x = synth.make_images(b, 1).to(dev).half()
+                n = max(steps // (4 if b > 1 else 1), 5)
+                res = {}
+                if b > 1:
+                    t = time_loop(lambda: vit(x), n, max(warmup // 2, 2))
+                    res["eager_images_per_s"] = b * n / t
+                    res["eager_ms"] = t / n * 1e3
                 vit(x)
-            t = time_loop(g.replay, n, max(warmup // 2, 2))
-            res["graph_images_per_s"] = b * n / t
-            res["graph_ms"] = t / n * 1e3
-            out[f"bs{b}"] = res
-            del g
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    vit(x)
+                t = time_loop(g.replay, n, max(warmup // 2, 2))
+                res["graph_images_per_s"] = b * n / t
+                res["graph_ms"] = t / n * 1e3
+                part[f"bs{b}"] = res
+                del g
+        out[name] = part
+        del vit
+        torch.cuda.empty_cache()
     return out
 
 

@@ -185,6 +185,54 @@ int arcq_linear_fused_blocked(const void *x_hat_blocked,
                               const float *bias, void *w_hat_ws, int w_hat_ready, void *y, int y_dtype,
                               int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
 
+/* ---- the layer with the elementwise work around it fused in ------------------------------------------------
+ * The transformer block the reference's models are built from (timm's Block via FQ/timm_quant_models.py:63-121) is
+ *     x = x + proj(attention(qkv(LayerNorm1(x))));   x = x + fc2(GELU(fc1(LayerNorm2(x))))
+ * with qkv / proj / fc1 / fc2 the packed linears.  This entry point runs one packed on-the-fly layer together with
+ * the work that sits directly in front of and behind it, so that the tensors in between never make a round trip
+ * through HBM in a launch of their own:
+ *     y = residual + activation(linear(stage1(producer(x))))
+ *   producer   ARCQ_PRODUCER_LAYERNORM: LayerNorm over the last dimension (ln_weight, ln_bias [K] fp32, ln_eps), its
+ *              result rounded to x's type, inside the stage-1 launch (arcq_act_quant_blocked_ln; K <= 1024)
+ *   activation ARCQ_ACT_GELU: the exact (erf) GELU of the rounded linear output, rounded again, in the GEMM's epilogue
+ *   residual   [M,N] of y's type, added to the rounded value, rounded again, in the GEMM's epilogue
+ * Every step rounds where a separate kernel would have stored its result, so y equals the unfused sequence bit for
+ * bit given the same LayerNorm output.  With no option set it is arcq_linear_otf_ws.  With an option set it needs
+ * group_size 64 and M >= 512 (the block-layout path) and returns ARCQ_ERR_UNSUPPORTED otherwise: compose the
+ * layer from the separate operations then.  Workspaces as arcq_linear_otf_ws (w_hat_ws may be NULL).
+ * struct_size = sizeof(arcq_linear_ex_args). */
+#define ARCQ_PRODUCER_NONE 0
+#define ARCQ_PRODUCER_LAYERNORM 1
+#define ARCQ_ACT_NONE 0
+#define ARCQ_ACT_GELU 1
+typedef struct arcq_linear_ex_args {
+    uint32_t struct_size;
+    int32_t x_dtype, y_dtype, producer, activation, bits, group_size;
+    float ln_eps;
+    int64_t M, N, K;
+    const void *x;
+    const float *ln_weight, *ln_bias;
+    const float *a_thresholds, *a_codebook;
+    const uint8_t *packed_w;
+    const float *w_codebook, *w_center, *w_scale, *w_code_sum, *bias;
+    const void *residual;
+    void *x_hat_ws, *w_hat_ws, *y;
+} arcq_linear_ex_args;
+int arcq_linear_otf_ex(const arcq_linear_ex_args *args, void *stream);
+
+/* LayerNorm + stage 1 into the block layout in one launch (the first half of arcq_linear_otf_ex with
+ * ARCQ_PRODUCER_LAYERNORM), exposed so that it can be called and tested on its own; no counterpart in the
+ * reference.  LayerNorm arithmetic, fp32: every lane's 32 values (half a group) are summed serially, a row's partial
+ * sums are added group by group, lower half first; mean = sum / cols; var = the same sum over (x - mean)^2, / cols;
+ * y = ((x - mean) * (1 / sqrt(var + ln_eps))) * ln_weight + ln_bias with one rounding per operation, then rounded to
+ * x's type.  64 <= cols <= 1024.  packed_w != NULL: the launch also reconstructs w_hat[N, cols] (fp16), as
+ * arcq_act_quant_blocked_with_weights does. */
+int arcq_act_quant_blocked_ln(const void *x, int x_dtype, const float *ln_weight, const float *ln_bias, float ln_eps,
+                              const float *thresholds, const float *codebook, void *x_hat_blocked,
+                              int64_t rows, int64_t cols, int bits, float eps,
+                              const uint8_t *packed_w, const float *w_codebook, const float *w_center,
+                              const float *w_scale, const float *w_code_sum, void *w_hat, int64_t N, void *stream);
+
 /* arcq_linear_otf_ws for callers that cannot allocate device memory or lend workspaces (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The two
  * scratch buffers come from a static device array of ARCQ_STATIC_SCRATCH_BYTES inside the library, of which every GPU

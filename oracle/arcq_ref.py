@@ -370,3 +370,54 @@ def fake_quant_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
     x_q = pcarcq_fake_quant(x, a_thr, a_cb, group_size, eps)
     w_q = pcarcq_fake_quant(weight, w_thr, w_cb, group_size, eps)
     return F.linear(x_q, w_q, bias)
+
+
+# --------------------------------------------------------------------------
+# LayerNorm in front of stage 1 (the fused producer of arcq_act_quant_blocked_ln) and the GELU of the
+# fused epilogue.  The reference runs both as timm / torch modules around the packed linears
+# (FQ/timm_quant_models.py:63-121: timm Block = LayerNorm -> Attention / Mlp with nn.GELU); timm is not
+# available offline, so these restate torch.nn.LayerNorm / nn.GELU() semantics, in the summation order the
+# HIP kernel documents, and are pinned against torch's own float64 layer_norm / erf in the tests.
+# --------------------------------------------------------------------------
+def layernorm_rows_np(x, weight, bias, eps: float, out_f16: bool) -> np.ndarray:
+    """LayerNorm over the last dimension (a multiple of 64) in the kernel's fp32 order: serial sums over
+    each run of 32 values, a row's partial sums added in order; mean = sum / K; var = the same over
+    (x - mean)^2; y = ((x - mean) * (1 / sqrt(var + eps))) * weight + bias, one rounding per operation;
+    optionally rounded to fp16 (what a stand-alone fp16 LayerNorm would store).  Returns fp32."""
+    x = np.ascontiguousarray(_f32(x))
+    rows, k = x.shape
+    assert k % 64 == 0
+    parts = k // 32
+    x3 = x.reshape(rows, parts, 32)
+    f32 = np.float32
+
+    def serial(v):
+        a = np.zeros(v.shape[:2], dtype=f32)
+        for j in range(32):
+            a = (a + v[:, :, j]).astype(f32)
+        return a
+
+    def total(p):
+        acc = np.zeros(rows, dtype=f32)
+        for i in range(parts):
+            acc = (acc + p[:, i]).astype(f32)
+        return acc
+
+    mean = (total(serial(x3)) / f32(k)).astype(f32)
+    d = (x3 - mean[:, None, None]).astype(f32)
+    var = (total(serial((d * d).astype(f32))) / f32(k)).astype(f32)
+    rstd = (f32(1.0) / np.sqrt((var + f32(eps)).astype(f32)).astype(f32)).astype(f32)
+    t = (d * rstd[:, None, None]).astype(f32)
+    u = (t * _f32(weight).reshape(1, parts, 32)).astype(f32)
+    y = (u + _f32(bias).reshape(1, parts, 32)).astype(f32).reshape(rows, k)
+    if out_f16:
+        y = y.astype(np.float16).astype(f32)
+    return y
+
+
+def gelu_f64_np(x) -> np.ndarray:
+    """Exact GELU ``0.5 x (1 + erf(x / sqrt 2))`` in float64 (nn.GELU(), approximate='none')."""
+    import math
+    x = np.asarray(x, dtype=np.float64)
+    erf = np.vectorize(math.erf, otypes=[np.float64])
+    return 0.5 * x * (1.0 + erf(x / math.sqrt(2.0)))

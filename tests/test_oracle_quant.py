@@ -328,3 +328,31 @@ def test_fma_division_sequence_is_ieee_division(oracle):
     guard range that is the correctly rounded quotient.  20 million random pairs incl. mantissa extremes."""
     for seed in (1, 2, 3, 4):
         assert oracle.check_div_sequence(5_000_000, seed) == 0
+
+
+def test_layernorm_restatement_is_layernorm(oracle):
+    """The fp32 LayerNorm restatement used in front of stage 1 against torch's own layer_norm in float64: a biased
+    variance, eps inside the square root and the affine step are what the comparison fixes (an unbiased variance
+    moves the result by 1 / (2 K), eps outside the root by ~eps / sigma on the small-variance rows)."""
+    g = torch.Generator().manual_seed(11)
+    k = 384
+    x = torch.randn(64, k, generator=g) * 2.0 + 0.5
+    x[32:] *= 1e-3                                  # variance ~ 4e-6: the same size as eps below
+    w = torch.randn(k, generator=g) * 0.5 + 1.0
+    b = torch.randn(k, generator=g) * 0.1
+    for eps in (1e-6, 1e-5):
+        got = oracle.layernorm_rows_np(x.numpy(), w.numpy(), b.numpy(), eps, out_f16=False)
+        want = torch.nn.functional.layer_norm(x.double(), (k,), w.double(), b.double(), eps).numpy()
+        assert np.max(np.abs(got - want) / (np.abs(want) + 1.0)) < 2e-6
+        wrong_var = torch.nn.functional.layer_norm(x.double(), (k,), w.double(), b.double(), eps).numpy() * np.sqrt((k - 1) / k)
+        assert np.max(np.abs(got - wrong_var)) > 1e-4
+    got16 = oracle.layernorm_rows_np(x.half().numpy(), w.numpy(), b.numpy(), 1e-6, out_f16=True)
+    want16 = torch.nn.functional.layer_norm(x.half().double(), (k,), w.double(), b.double(), 1e-6).half().float().numpy()
+    ulp = np.abs(got16 - want16) / np.maximum(np.abs(np.spacing(want16.astype(np.float16)).astype(np.float32)), 1e-8)
+    assert ulp.max() <= 1.0 and (ulp > 0).mean() < 2e-3      # same fp16 value but for rare round-off at a rounding boundary
+
+
+def test_gelu_reference_matches_torch(oracle):
+    x = torch.linspace(-8, 8, 4001, dtype=torch.float64)
+    want = torch.nn.functional.gelu(x).numpy()
+    assert np.max(np.abs(oracle.gelu_f64_np(x.numpy()) - want)) < 1e-14
