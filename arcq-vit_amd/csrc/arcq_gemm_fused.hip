@@ -372,7 +372,7 @@ ARCQ_API const char *arcq_linear_otf_ws_kernel(int64_t M, int64_t N, int64_t K, 
         GemmArgs g{};
         g.M = static_cast<int>(M), g.N = static_cast<int>(N), g.K = static_cast<int>(K);
         const char *e = tuning().pair;
-        return (e ? e[0] == '1' : gemm_pair_pays(g)) ? "gemm_pair_kernel" : "gemm_slab8_kernel<copy>";
+        return (e ? e[0] != '0' : gemm_pair_pays(g)) ? "gemm_pair_kernel" : "gemm_slab8_kernel<copy>";
     }
     return arcq_linear_fused_ws_kernel(M, N, K, have_workspace);
 }

@@ -312,6 +312,7 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
                 if (gl + 1 < ng) unit(r1, r0, gl + 1);
                 if (gl + 2 < ng) unit(r2, r1, gl + 2);
             }
+
             const int rot = ng % 3;
             if (rot == 1) {             // r0 consumed (r2 refilled): next unit is in r1, the one after in r2
 #pragma unroll
@@ -483,7 +484,7 @@ void launch_gemm_slab8(const GemmArgs &g, const void *w_hat, hipStream_t stream)
 {
     if (w_hat) {
         const char *e = tuning().pair;           // tuning aid: 0 / 1 pin the choice
-        if (e ? e[0] == '1' : gemm_pair_pays(g)) {
+        if (e ? e[0] != '0' : gemm_pair_pays(g)) {
             launch_gemm_pair(g, w_hat, stream);
             return;
         }

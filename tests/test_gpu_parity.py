@@ -516,10 +516,11 @@ def test_fused_gemm_pair_kernel(cuda, oracle, monkeypatch, bits, out_dtype, m, n
     xb = ops.quantize_activation_blocked(x.to(cuda), thr.to(cuda), cb.to(cuda), bits, weights=w, w_hat=ws)
     monkeypatch.setenv("ARCQ_PAIR", "0")
     ref = ops.linear_fused_blocked(xb, m, k, *w, bias, bits, out_dtype=out_dtype, w_hat_ws=ws, w_hat_ready=True)
-    monkeypatch.setenv("ARCQ_PAIR", "1")
-    y = ops.linear_fused_blocked(xb, m, k, *w, bias, bits, out_dtype=out_dtype, w_hat_ws=ws, w_hat_ready=True)
+    for variant in ("1", "2"):          # one slab buffer of six groups / two of three with the copy under the multiplication
+        monkeypatch.setenv("ARCQ_PAIR", variant)
+        y = ops.linear_fused_blocked(xb, m, k, *w, bias, bits, out_dtype=out_dtype, w_hat_ws=ws, w_hat_ready=True)
+        assert torch.equal(y, ref), variant
     monkeypatch.delenv("ARCQ_PAIR")
-    assert torch.equal(y, ref)
     rows = torch.randint(0, m, (40,), generator=torch.Generator().manual_seed(2))
     rows[0], rows[1] = 0, m - 1
     a = oracle.act_quant_c(x[rows].float().numpy(), thr, cb, bits, 64)["x_hat"].astype(np.float16)
