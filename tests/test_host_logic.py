@@ -94,6 +94,9 @@ def test_abi_argument_errors_need_no_gpu():
     assert b"group_size 64" in lib.arcq_last_error()
     assert lib.arcq_linear_fused(8, 16, 8, 8, 8, 8, 0, 16, 1, 4, 4, 128, 4, 64, 0) == -7  # misaligned x_hat
     assert lib.arcq_linear_forward_packed(*([8] * 11), 4, 4, 128, 4, 64, 8, 0) == -4      # 8 levels < 2^4
+    assert lib.arcq_linear_forward_packed(*([8] * 11), 4, 4, 128, 4, 64, 200, 0) == -4    # a 200 x 200 table does not fit LDS
+    assert b"levels <= 128" in lib.arcq_last_error()
+    assert lib.arcq_linear_forward_u8(*([8] * 11), 4, 4, 128, 64, 129, 0) == -4
     assert lib.arcq_linear_otf(8, 0, 8, 8, 8, 8, 8, 8, 8, 0, 8, 16, 1, 4, 4, 128, 4, 64, 0) == -5  # fp32 x aliasing ws
     with pytest.raises(RuntimeError, match="aliasing|alias"):
         A._lib.check(-5)
