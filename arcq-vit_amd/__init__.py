@@ -16,7 +16,9 @@ from .ops import (  # noqa: F401
     unpack_weight_hip,
 )
 from .pack_py import pack_codes_py, unpack_codes_py  # noqa: F401
+from .packed_conv import ARCQPackedPatchConv  # noqa: F401
 from .packed_convert import (  # noqa: F401
+    convert_arcq_conv_to_packed,
     convert_arcq_linear_to_packed,
     count_packed_linear,
     load_packed_state_dict,
@@ -26,7 +28,13 @@ from .packed_convert import (  # noqa: F401
 from .packed_fast_linear import ARCQPackedLinearFast  # noqa: F401
 from .packed_linear import ARCQPackedLinear, _quantize_weight_reference, infer_packed_hparams  # noqa: F401
 from .packed_on_the_fly import ARCQPackedLinearOnTheFly, clear_workspaces  # noqa: F401
-from .quant_source import FrozenARCQQuantizer, QuantLinearPCARCQ  # noqa: F401
+from .quant_source import (  # noqa: F401
+    FrozenARCQQuantizer,
+    LSQQuantizer,
+    QuantConv2dPCARCQ,
+    QuantLinearLSQ,
+    QuantLinearPCARCQ,
+)
 
 __all__ = [
     "pack_codes", "unpack_codes", "unpack_codes_u8", "quantize_activation", "quantize_activation_dequant",
@@ -35,4 +43,5 @@ __all__ = [
     "ARCQPackedLinear", "ARCQPackedLinearOnTheFly", "ARCQPackedLinearFast", "QuantLinearPCARCQ",
     "FrozenARCQQuantizer", "convert_arcq_linear_to_packed", "count_packed_linear", "to_on_the_fly",
     "load_packed_state_dict", "infer_packed_hparams", "share_buffers", "clear_workspaces",
+    "ARCQPackedPatchConv", "convert_arcq_conv_to_packed", "QuantConv2dPCARCQ", "QuantLinearLSQ", "LSQQuantizer",
 ]

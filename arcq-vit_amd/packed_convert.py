@@ -13,8 +13,10 @@ from typing import Dict, List
 import torch
 import torch.nn as nn
 
+from .packed_conv import ARCQPackedPatchConv
 from .packed_linear import ARCQPackedLinear
 from .packed_on_the_fly import ARCQPackedLinearOnTheFly
+from .quant_source import QuantConv2dPCARCQ, QuantLinearLSQ
 
 
 def _is_pcarcq_linear(module: nn.Module) -> bool:
@@ -31,6 +33,28 @@ def convert_arcq_linear_to_packed(model: nn.Module, runtime_code_format: str = "
         else:
             convert_arcq_linear_to_packed(child, runtime_code_format=runtime_code_format)
     return model
+
+
+def _is_pcarcq_conv(module: nn.Module) -> bool:
+    return (module.__class__.__name__ == "QuantConv2dPCARCQ" and hasattr(module, "conv")
+            and hasattr(module, "act_quant") and hasattr(module, "weight_quant"))
+
+
+def convert_arcq_conv_to_packed(model: nn.Module) -> int:
+    """Replace (in place) every ``QuantConv2dPCARCQ`` that is a patch convolution by an ``ARCQPackedPatchConv``;
+    other geometries stay as they are.  Returns the number replaced.  The reference has no counterpart: its
+    converter leaves convolutions as fake quantization (FQ/arcq_packed_convert.py:8-14)."""
+    done = 0
+    for name, child in list(model.named_children()):
+        if _is_pcarcq_conv(child):
+            c = child.conv
+            if (tuple(c.stride) == tuple(c.kernel_size) and tuple(int(p) for p in c.padding) == (0, 0)
+                    and tuple(c.dilation) == (1, 1) and c.groups == 1):
+                setattr(model, name, ARCQPackedPatchConv(child))
+                done += 1
+        else:
+            done += convert_arcq_conv_to_packed(child)
+    return done
 
 
 def count_packed_linear(model: nn.Module) -> int:
@@ -84,7 +108,10 @@ def load_packed_state_dict(model: nn.Module, state_dict: Dict[str, torch.Tensor]
     """
     state_dict = {k.replace("module.", "", 1) if k.startswith("module.") else k: v for k, v in state_dict.items()}
     consumed = set()
-    for prefix in packed_layer_prefixes(state_dict):
+    installed = []
+
+    def install(prefix: str, layer: nn.Module) -> None:
+        installed.append(prefix)
         path = prefix[:-1].split(".") if prefix else []
         if not path:
             raise KeyError("a packed layer cannot be the model root")
@@ -95,14 +122,47 @@ def load_packed_state_dict(model: nn.Module, state_dict: Dict[str, torch.Tensor]
             parent = getattr(parent, part)
         if not hasattr(parent, path[-1]):
             raise KeyError(f"packed checkpoint names '{prefix[:-1]}', which the model does not have")
-        layer = ARCQPackedLinear.from_packed_state(state_dict, prefix, runtime_code_format)
-        setattr(parent, path[-1], ARCQPackedLinearOnTheFly.from_packed(layer) if on_the_fly else layer)
+        setattr(parent, path[-1], layer)
+
+    for prefix in packed_layer_prefixes(state_dict):
+        if prefix + "conv_geometry" in state_dict:
+            install(prefix, ARCQPackedPatchConv.from_packed_state(state_dict, prefix))
+        else:
+            layer = ARCQPackedLinear.from_packed_state(state_dict, prefix, runtime_code_format)
+            install(prefix, ARCQPackedLinearOnTheFly.from_packed(layer) if on_the_fly else layer)
+        consumed.update(k for k in state_dict if k.startswith(prefix))
+    # Layers the reference's converter leaves as fake quantization: the patch-embedding convolution
+    # (keys conv.weight + ARCQ quantizer buffers) and the LSQ classifier head (linear.weight + step parameters).
+    for key in list(state_dict):
+        if key.endswith("conv.weight") and key[: -len("conv.weight")] + "act_quant._pc_cb" in state_dict:
+            prefix = key[: -len("conv.weight")]
+            w = state_dict[key]
+            bits = int(state_dict[prefix + "weight_quant._pc_cb"].numel()).bit_length() - 1
+            a_bits = int(state_dict[prefix + "act_quant._pc_cb"].numel()).bit_length() - 1
+            layer = QuantConv2dPCARCQ(w.shape[1], w.shape[0], tuple(w.shape[2:]), tuple(w.shape[2:]), 0,
+                                      prefix + "conv.bias" in state_dict, bits, a_bits)
+            for q in (layer.act_quant, layer.weight_quant):
+                q._pc_ready = True
+        elif key.endswith("linear.weight") and key[: -len("linear.weight")] + "act_quant.step" in state_dict:
+            prefix = key[: -len("linear.weight")]
+            w = state_dict[key]
+            layer = QuantLinearLSQ(w.shape[1], w.shape[0], prefix + "linear.bias" in state_dict)
+        else:
+            continue
+        for name, _ in list(layer.named_buffers()) + list(layer.named_parameters()):
+            stored = state_dict.get(prefix + name)
+            if stored is not None:      # buffers registered empty / step sizes of another shape take the stored shape
+                owner = layer.get_submodule(name.rsplit(".", 1)[0]) if "." in name else layer
+                attr = name.rsplit(".", 1)[-1]
+                if attr in owner._buffers:
+                    owner._buffers[attr] = stored.detach().clone()
+                else:
+                    owner._parameters[attr] = nn.Parameter(stored.detach().clone(), requires_grad=False)
+        install(prefix, layer.eval())
         consumed.update(k for k in state_dict if k.startswith(prefix))
     rest = {k: v for k, v in state_dict.items() if k not in consumed}
     missing, unexpected = model.load_state_dict(rest, strict=False)
-    packed_keys = {k for k, _ in model.state_dict().items()
-                   if any(k.startswith(p) for p in packed_layer_prefixes(state_dict))}
-    missing = [k for k in missing if k not in packed_keys]
+    missing = [k for k in missing if not any(k.startswith(p) for p in installed)]
     if missing or unexpected:
         raise KeyError(f"packed checkpoint mismatch: missing={missing[:8]} unexpected={list(unexpected)[:8]}")
     return model

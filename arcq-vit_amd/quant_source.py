@@ -76,3 +76,80 @@ class QuantLinearPCARCQ(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return F.linear(self.act_quant(x), self.weight_quant(self.linear.weight), self.linear.bias)
+
+
+class QuantConv2dPCARCQ(nn.Module):
+    """``conv`` + ``act_quant`` + ``weight_quant`` (FQ/quant_backends.py:329-384 without the DC conditioner, which the
+    ``pcarcq_nodc`` backend leaves off): the activation is quantized in NHWC order, so a group is
+    ``min(group_size, in_ch)`` channels of one pixel (three for RGB input), the weight as the 2-D matrix
+    ``[out_ch, in_ch * kh * kw]`` in groups of ``group_size``; then ``F.conv2d``."""
+
+    def __init__(self, in_ch: int, out_ch: int, k, s, p, bias: bool, w_bits: int, a_bits: int, group_size: int = 64):
+        super().__init__()
+        self.conv = nn.Conv2d(in_ch, out_ch, k, stride=s, padding=p, bias=bias)
+        act_gs = min(group_size, in_ch) if in_ch > 0 else group_size
+        self.act_quant = FrozenARCQQuantizer(bits=a_bits, group_size=act_gs)
+        self.weight_quant = FrozenARCQQuantizer(bits=w_bits, group_size=group_size)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        w = self.conv.weight
+        x_q = self.act_quant(x.permute(0, 2, 3, 1).contiguous()).permute(0, 3, 1, 2).contiguous()
+        w_q = self.weight_quant(w.reshape(w.shape[0], -1)).reshape_as(w)
+        c = self.conv
+        return F.conv2d(x_q, w_q, c.bias, c.stride, c.padding, c.dilation, c.groups)
+
+
+class LSQQuantizer(nn.Module):
+    """Uniform quantizer with a learned step size, eval behaviour only.
+
+    The reference constructs ``quant.lsq.LSQQuantizer(bits, signed, per_channel, ch_axis)``
+    (FQ/quant_backends.py:125-136) but does not ship ``quant/lsq.py``; its checkpoint loader shows that the step
+    size is a parameter named ``step`` whose shape may differ from the registered one
+    (scripts/benchmark_arcq_packed_inference.py:93-95).  What is here is the published LSQ forward (Esser et al.,
+    ICLR 2020): ``round(clamp(x / step, Qn, Qp)) * step`` with ``Qn = -2^(bits-1)``, ``Qp = 2^(bits-1) - 1`` for
+    signed and ``0 .. 2^bits - 1`` for unsigned tensors; a per-channel step broadcasts along ``ch_axis``.  With no
+    reference source to compare against, parity of this class is unpinned."""
+
+    def __init__(self, bits: int = 8, signed: bool = True, per_channel: bool = False, ch_axis: int = 0):
+        super().__init__()
+        self.bits = int(bits)
+        self.signed = bool(signed)
+        self.per_channel = bool(per_channel)
+        self.ch_axis = int(ch_axis)
+        self.qn = -(1 << (self.bits - 1)) if self.signed else 0
+        self.qp = (1 << (self.bits - 1)) - 1 if self.signed else (1 << self.bits) - 1
+        self.step = nn.Parameter(torch.ones(1))
+
+    def init_from(self, x: torch.Tensor) -> None:
+        """Step size from data, the LSQ paper's initialisation ``2 mean|x| / sqrt(Qp)`` (per channel if so built)."""
+        with torch.no_grad():
+            if self.per_channel:
+                dims = [d for d in range(x.dim()) if d != self.ch_axis % x.dim()]
+                mean_abs = x.detach().abs().mean(dim=dims)
+            else:
+                mean_abs = x.detach().abs().mean().reshape(1)
+            self.step = nn.Parameter((2.0 * mean_abs / (self.qp ** 0.5)).clamp_min(1e-8).float())
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.bits >= 32:
+            return x
+        step = self.step.to(x.dtype)
+        if step.numel() > 1:
+            shape = [1] * x.dim()
+            shape[self.ch_axis % x.dim()] = step.numel()
+            step = step.reshape(shape)
+        return torch.clamp(x / step, self.qn, self.qp).round() * step
+
+
+class QuantLinearLSQ(nn.Module):
+    """``linear`` + per-tensor activation LSQ + per-output-channel weight LSQ (FQ/quant_backends.py:125-136); the
+    ``pcarcq_nodc`` backend uses it at 8/8 bits for the classifier head (:420-421)."""
+
+    def __init__(self, in_f: int, out_f: int, bias: bool, w_bits: int = 8, a_bits: int = 8):
+        super().__init__()
+        self.linear = nn.Linear(in_f, out_f, bias=bias)
+        self.act_quant = LSQQuantizer(bits=a_bits, signed=True, per_channel=False)
+        self.weight_quant = LSQQuantizer(bits=w_bits, signed=True, per_channel=True, ch_axis=0)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(self.act_quant(x), self.weight_quant(self.linear.weight), self.linear.bias)

@@ -3,8 +3,10 @@
 mlp.{fc1,fc2}}``, ``norm``, ``head``), so packed-checkpoint keys produced from a timm model
 (FQ/timm_quant_models.py:155-182) line up.  timm itself is not available offline.
 
-Only the four block linears are quantized (the packed path's scope); patch embedding, LayerNorm,
-softmax attention, GELU and the head stay in floating point, as the reference's README states.
+By default only the four block linears are quantized (the packed path's scope); patch embedding, LayerNorm,
+softmax attention, GELU and the head stay in floating point, as the reference's README states.  The builders can
+also give the model the reference's full quantization scope (FQ/timm_quant_models.py:63-121): the ARCQ wrapper on the
+patch-embedding convolution and the W8A8 LSQ wrapper on the head.
 """
 from __future__ import annotations
 
@@ -14,8 +16,9 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .packed_convert import convert_arcq_linear_to_packed, share_buffers, to_on_the_fly
-from .quant_source import QuantLinearPCARCQ
+from .packed_convert import (convert_arcq_conv_to_packed, convert_arcq_linear_to_packed, share_buffers,
+                             to_on_the_fly)
+from .quant_source import QuantConv2dPCARCQ, QuantLinearLSQ, QuantLinearPCARCQ
 from .synth import MODEL_DIMS, SEED, quantile_codebook
 
 LinearFactory = Callable[[int, int, bool], nn.Module]
@@ -103,10 +106,13 @@ class VisionTransformer(nn.Module):
 
 
 def build_fakequant_vit(model: str, bits: int, group_size: int = 64, seed: int = SEED,
-                        num_classes: int = 1000, depth: Optional[int] = None) -> VisionTransformer:
+                        num_classes: int = 1000, depth: Optional[int] = None, quantize_patch_embed: bool = False,
+                        head_quant: str = "fp32") -> VisionTransformer:
     """Random-init ViT whose block linears are ``QuantLinearPCARCQ`` with quantile codebooks
     (weights N(0, 0.02^2), as timm's trunc_normal_(std=.02) init; biases N(0, 0.01^2)).
-    ``depth`` overrides the model's number of blocks (a shallower model of the same widths)."""
+    ``depth`` overrides the model's number of blocks (a shallower model of the same widths).
+    ``quantize_patch_embed`` wraps ``patch_embed.proj`` in ``QuantConv2dPCARCQ`` (same codebook), ``head_quant="w8a8"``
+    the head in ``QuantLinearLSQ`` with step sizes initialised from the weights and from unit-variance input."""
     cfg = dict(MODEL_DIMS[model])
     if depth is not None:
         cfg["depth"] = int(depth)
@@ -127,19 +133,36 @@ def build_fakequant_vit(model: str, bits: int, group_size: int = 64, seed: int =
             elif name.endswith("bias"):
                 p.copy_(torch.randn(p.shape, generator=g) * 0.01)
             # LayerNorm weights keep their default of one
+        if quantize_patch_embed:
+            conv = vit.patch_embed.proj
+            q = QuantConv2dPCARCQ(conv.in_channels, conv.out_channels, conv.kernel_size, conv.stride, conv.padding,
+                                  True, bits, bits, group_size)
+            q.conv.load_state_dict(conv.state_dict())
+            q.act_quant.set_codebook(cb)
+            q.weight_quant.set_codebook(cb)
+            vit.patch_embed.proj = q
+        if head_quant != "fp32":
+            head = QuantLinearLSQ(vit.head.in_features, vit.head.out_features, True, 8, 8)
+            head.linear.load_state_dict(vit.head.state_dict())
+            head.weight_quant.init_from(head.linear.weight)
+            head.act_quant.init_from(torch.randn(4096, generator=g))
+            vit.head = head
     return vit.eval()
 
 
 def build_packed_vit(model: str, bits: int, group_size: int = 64, seed: int = SEED, num_classes: int = 1000,
                      device: str = "cuda", half_chain: bool = True, depth: Optional[int] = None,
-                     shared_buffers: bool = False, max_rows: int = 0, fuse_elementwise: bool = False) -> VisionTransformer:
+                     shared_buffers: bool = False, max_rows: int = 0, fuse_elementwise: bool = False,
+                     quantize_patch_embed: bool = False, head_quant: str = "fp32") -> VisionTransformer:
     """Fake-quant ViT -> packed (``convert_arcq_linear_to_packed``) -> on-the-fly layers -> device,
     the sequence of scripts/benchmark_arcq_on_the_fly.py:88-199.  ``half_chain`` casts the
     floating-point rest of the model to fp16 (packed metadata stays fp32).  ``shared_buffers`` gives all
     layers one weight scratch buffer (:182-191 there) and, with ``max_rows`` tokens, one x_hat buffer.
-    ``fuse_elementwise``: LayerNorm, GELU and the skip connections run inside the packed layers' launches."""
-    vit = build_fakequant_vit(model, bits, group_size, seed, num_classes, depth)
+    ``fuse_elementwise``: LayerNorm, GELU and the skip connections run inside the packed layers' launches.
+    ``quantize_patch_embed``: the patch embedding is an ``ARCQPackedPatchConv``; ``head_quant="w8a8"``: LSQ head."""
+    vit = build_fakequant_vit(model, bits, group_size, seed, num_classes, depth, quantize_patch_embed, head_quant)
     convert_arcq_linear_to_packed(vit, runtime_code_format="packed")
+    convert_arcq_conv_to_packed(vit)
     to_on_the_fly(vit)
     vit = vit.to(device)
     if half_chain:
