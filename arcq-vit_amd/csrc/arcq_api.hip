@@ -32,7 +32,7 @@ int launch_status(const char *what)
 
 namespace {
 struct TuningStore {
-    char gemm_kernel[32], otf_fused[8], pair[8];
+    char gemm_kernel[32], otf_fused[8], pair[8], rows[8];
     Tuning view;
 };
 TuningStore g_tuning;
@@ -52,6 +52,7 @@ void read_tuning()
     g_tuning.view.gemm_kernel = grab("ARCQ_GEMM_KERNEL", g_tuning.gemm_kernel, sizeof(g_tuning.gemm_kernel));
     g_tuning.view.otf_fused = grab("ARCQ_OTF_FUSED", g_tuning.otf_fused, sizeof(g_tuning.otf_fused));
     g_tuning.view.pair = grab("ARCQ_PAIR", g_tuning.pair, sizeof(g_tuning.pair));
+    g_tuning.view.rows = grab("ARCQ_ROWS", g_tuning.rows, sizeof(g_tuning.rows));
 }
 }  // namespace
 
@@ -103,6 +104,17 @@ static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds
             arcq::launch_otf_small(a, static_cast<hipStream_t>(stream));
             return arcq::launch_status("arcq_linear_otf");
         }
+    }
+    // Short rows, many of them, fp16 input, both workspaces scratch: the whole layer in one launch (x_hat stays in
+    // LDS, the weight workspace takes w_hat in the 32-column block layout); same results bit for bit.
+    if (scratch_only && w_hat_ws && x_dtype == ARCQ_F16 && group_size == 64 && arcq::bits_ok(bits) &&
+        arcq::otf_rows_pays(M, N, K) && x && a_thresholds && a_codebook && packed_w && w_codebook && w_center && w_scale &&
+        w_code_sum && y && (y_dtype == ARCQ_F16 || y_dtype == ARCQ_F32) && arcq::aligned(x, 16) && arcq::aligned(y, 16) &&
+        arcq::aligned(w_hat_ws, 16) && arcq::aligned(packed_w, 4)) {
+        arcq::OtfRowsArgs a{x, a_thresholds, a_codebook, nullptr, nullptr, 0.0f, packed_w, w_codebook, w_center, w_scale,
+                            w_code_sum, bias, w_hat_ws, y, y_dtype == ARCQ_F16, nullptr, false, static_cast<int>(M),
+                            static_cast<int>(N), static_cast<int>(K), bits, 1.0e-6f};
+        return arcq::launch_otf_rows(a, static_cast<hipStream_t>(stream));
     }
     // Scratch-only workspaces and 512 rows or more: x_hat in the block layout, eight-wave weight-stationary GEMM
     // (bit-identical results; invalid arguments fall through to the entry points below, which report them).
@@ -172,6 +184,19 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
     if (a->x_hat_ws == a->x) return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: x_hat_ws must not alias x");
     if (a->residual && !arcq::aligned(a->residual, 16))
         return arcq::fail(ARCQ_ERR_ALIGN, "arcq_linear_otf_ex: residual must be 16-byte aligned");
+    if (a->w_hat_ws && a->x_dtype == ARCQ_F16 && arcq::otf_rows_pays(a->M, a->N, a->K) && a->x && a->a_thresholds &&
+        a->a_codebook && a->packed_w && a->w_codebook && a->w_center && a->w_scale && a->w_code_sum && a->y &&
+        (a->y_dtype == ARCQ_F16 || a->y_dtype == ARCQ_F32) && arcq::aligned(a->x, 16) && arcq::aligned(a->y, 16) &&
+        arcq::aligned(a->w_hat_ws, 16) && arcq::aligned(a->packed_w, 4) &&
+        (a->producer != ARCQ_PRODUCER_LAYERNORM || (a->ln_weight && a->ln_bias && arcq::aligned(a->ln_weight, 16) &&
+                                                    arcq::aligned(a->ln_bias, 16)))) {
+        const bool ln = a->producer == ARCQ_PRODUCER_LAYERNORM;
+        arcq::OtfRowsArgs r{a->x, a->a_thresholds, a->a_codebook, ln ? a->ln_weight : nullptr, ln ? a->ln_bias : nullptr,
+                            a->ln_eps, a->packed_w, a->w_codebook, a->w_center, a->w_scale, a->w_code_sum, a->bias,
+                            a->w_hat_ws, a->y, a->y_dtype == ARCQ_F16, a->residual, a->activation == ARCQ_ACT_GELU,
+                            static_cast<int>(a->M), static_cast<int>(a->N), static_cast<int>(a->K), a->bits, 1.0e-6f};
+        return arcq::launch_otf_rows(r, static_cast<hipStream_t>(stream));
+    }
     const bool carry = a->w_hat_ws && arcq::blocked_uses_workspace(a->N, a->K) && a->packed_w && a->w_codebook && a->w_center &&
                        a->w_scale && a->w_code_sum && arcq::aligned(a->w_hat_ws, 16) && arcq::aligned(a->packed_w, 16);
     int rc;

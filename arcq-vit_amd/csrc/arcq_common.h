@@ -19,12 +19,13 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 // Turns hipGetLastError() after a launch into the ABI's return value.
 int launch_status(const char *what);
 
-// Tuning switches from the environment (ARCQ_GEMM_KERNEL, ARCQ_OTF_FUSED, ARCQ_PAIR), read once per process;
+// Tuning switches from the environment (ARCQ_GEMM_KERNEL, ARCQ_OTF_FUSED, ARCQ_PAIR, ARCQ_ROWS), read once per process;
 // arcq_reload_tuning() reads them again.  nullptr = not set.
 struct Tuning {
     const char *gemm_kernel;   // "stream" | "slab" | "small" | "splitk" | "slab8" | "prebuilt"
     const char *otf_fused;     // "0" | "2"
     const char *pair;          // "0" | "1"
+    const char *rows;          // "0" | "1": the one-launch row-stationary layer kernel off / wherever it can run
 };
 const Tuning &tuning();
 

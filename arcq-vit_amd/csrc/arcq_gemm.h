@@ -67,4 +67,27 @@ struct OtfSmallArgs {
 bool otf_small_supported(int64_t M, int64_t N, int64_t K, bool any_supported);
 void launch_otf_small(const OtfSmallArgs &a, hipStream_t stream);
 
+// Whole layer in one launch for short rows: stage 1 (optionally LayerNorm first) into LDS, product with weights that
+// the same launch reconstructs into the weight workspace in its 32-column block layout ([N/32][K/8][32][8] fp16).
+struct OtfRowsArgs {
+    const void *x;           // [M,K] fp16
+    const float *a_thr, *a_cb;
+    const float *ln_weight, *ln_bias;    // fp32 [K], or nullptr: no LayerNorm
+    float ln_eps;
+    const uint8_t *pw;
+    const float *w_cb, *wc, *ws, *wcs, *bias;
+    void *w_hat_ws;          // at least N*K fp16, 16-byte aligned
+    void *y;
+    bool y_f16;
+    const void *residual;    // [M,N] of y's type, or nullptr
+    bool gelu;
+    int M, N, K, bits;
+    float eps;
+};
+// Shapes the kernel can run (M >= 512, K a multiple of 64 up to 512, N a multiple of 32, everything within LDS).
+bool otf_rows_supported(int64_t M, int64_t N, int64_t K);
+// Whether the whole-layer entry points take it for this shape (fp16 input, both workspaces given).
+bool otf_rows_pays(int64_t M, int64_t N, int64_t K);
+int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream);
+
 }  // namespace arcq

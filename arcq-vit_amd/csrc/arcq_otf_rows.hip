@@ -1,0 +1,507 @@
+// Whole on-the-fly layer in ONE launch for short rows (K <= 512) and many of them: a workgroup owns 64 rows of x,
+// quantizes them into LDS (stage 1, optionally with the LayerNorm in front of it) and multiplies them with every
+// column of w_hat, which streams through the registers from a 32-column block layout in the weight workspace.
+//
+//   y[M,N] = post( stage1( [LayerNorm] x )[M,K] * w_hat[N,K]^T + bias )
+//
+// Why a second design beside the weight-stationary kernels: with K = 384 a launch of those does 4-20 us of work per
+// CU, and the fixed costs of two launches (launch ramp, first loads, the x_hat round trip through L2, the drain)
+// are a third of the layer.  Here x_hat never leaves the CU (64 rows x K fp16 = 48 KB of LDS at K = 384), stage 1
+// runs on all twelve waves at once (wave = 32 rows x one group, two lanes per group), and the product starts the
+// moment the workgroup's own rows are done.  The price is that every workgroup reads all of w_hat from L2
+// (N*K*2 bytes, 0.9 MB for DeiT-S qkv) -- affordable only while K is short.
+//
+// Weights: w_hat is rebuilt from the packed codes inside the same launch, cooperatively: every workgroup
+// reconstructs 1/gridDim of it into the workspace (16-byte pieces, written through to memory), adds to a counter,
+// does its stage 1, and then waits for the counter to show that all shares have been written.  The wait is bounded:
+// a workgroup that has not seen the others finish within a few milliseconds (they may not be resident) rebuilds
+// the whole matrix itself -- same values, so a share written twice is harmless -- and goes on.  No workgroup ever
+// waits before it has contributed its share, so the counter always completes.
+//
+// Layout of the weight workspace: [N/32][K/8][32 columns][8 values] fp16 -- the MFMA fragment of a 32-column block
+// and k-step (lane = column, 8 consecutive k) is one 16-byte load per lane, 512 contiguous bytes per half wave.
+// Accumulation order per output (groups ascending, four k-steps of 16 per group, fp32) is that of the
+// weight-stationary kernels, so y is bit-identical to theirs.
+#include "arcq_common.h"
+#include "arcq_gemm.h"
+#include "arcq_act_quant_core.h"
+
+#include <mutex>
+
+namespace arcq {
+namespace {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kInPitch = 33;                 // dwords per row of a wave's stage-1 input tile (64 fp16 + 1 pad)
+constexpr int kWaveLds = 4608;               // bytes of LDS per wave: input tile (4224), later the output staging tile
+constexpr unsigned long long kEpoch = 1ull << 20;     // what one launch adds to its counter, whatever its grid
+constexpr long long kSpinTicks = 500000;     // bounded wait for the other workgroups' shares: 5 ms of the 100 MHz clock
+
+constexpr int gcd_of(int a, int b) { return b == 0 ? a : gcd_of(b, a % b); }
+
+struct RowsParams {
+    const __half *x;                 // [M,K] fp16
+    const float *thr, *cb_a;         // activation thresholds / codebook
+    float eps;
+    const float *gamma, *beta;       // LayerNorm weight / bias (fp32), gamma == nullptr: no LayerNorm
+    float ln_eps;
+    const uint8_t *pw;               // packed weight codes [N, K*bits/8]
+    const float *cb_w, *wc, *ws, *wcs;
+    __half *w_blk;                   // weight workspace, block layout
+    unsigned long long *counter;     // nullptr: w_blk is complete already
+    const float *bias;               // [N] or nullptr
+    void *y;
+    const void *residual;
+    int gelu;
+    int M, N, G;
+};
+
+// Piece idx of the block-layout w_hat, idx = ((n / 32) * (K / 8) + k / 8) * 32 + n % 32, holds w_hat[n][k .. k + 8):
+// value (cb[code] - code_sum/64) * scale + center with one fma (FQ/arcq_packed_triton.py:59-74), stored at
+// out + 8 idx, written through to memory.  In two steps so that the loads of the first can travel under other work.
+struct Piece {
+    uint32_t w;
+    float c, s, m;
+};
+template <int BITS>
+__device__ __forceinline__ void fetch_piece(const RowsParams &p, int64_t idx, Piece &pc)
+{
+    const int K = 64 * p.G, P = K / 8;
+    const int64_t pcols = static_cast<int64_t>(K) * BITS / 8;
+    const int r = static_cast<int>(idx & 31);
+    const int64_t t = idx >> 5;
+    const int pp = static_cast<int>(t % P);
+    const int64_t n = (t / P) * 32 + r;
+    pc.w = load_codes8<BITS>(p.pw + n * pcols + pp * BITS);
+    const int64_t mi = n * p.G + (pp >> 3);
+    pc.c = p.wc[mi];
+    pc.s = p.ws[mi];
+    pc.m = p.wcs[mi] * 0.015625f;      // code_sum / 64, exact
+}
+template <int BITS>
+__device__ __forceinline__ void finish_piece(const RowsParams &p, int64_t idx, const Piece &pc)
+{
+    constexpr int L = 1 << BITS;
+    float cbv[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) cbv[q] = p.cb_w[(pc.w >> (BITS * q)) & (L - 1)];      // 64 bytes, cached
+    uint32_t out[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const __half2 h = __floats2half2_rn(fma_f32(cbv[2 * q] - pc.m, pc.s, pc.c), fma_f32(cbv[2 * q + 1] - pc.m, pc.s, pc.c));
+        out[q] = *reinterpret_cast<const uint32_t *>(&h);
+    }
+    store_writethrough16(p.w_blk + idx * 8, out[0], out[1], out[2], out[3]);
+}
+
+// G = K / 64 groups per row (the workgroup has 2 G waves); RING = groups of w_hat fragments a wave holds (the one
+// being multiplied and RING - 1 on their way from L2); AHEAD = k-steps by which the LDS reads of the x_hat fragments
+// run ahead of the MFMAs that use them.
+template <int BITS, typename TOUT, int G, int RING, int AHEAD>
+__global__ void __launch_bounds__(128 * G)
+otf_rows_kernel(const RowsParams p)
+{
+    constexpr int L = 1 << BITS;
+    constexpr int MAXW = 2 * G;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ float lut[L * 64];
+    __shared__ Bucket table[kMaxBuckets + 1];
+    __shared__ int slow_slots[MAXW];
+    __shared__ int s_flag;
+
+    constexpr int K = 64 * G, W = 2 * G;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int nthreads = 64 * W;
+    constexpr int pitch = K * 2 + 16;                               // bytes per x_hat row in LDS (conflict-free 16-byte reads)
+    unsigned char *xs = smem;                                   // [64][pitch]
+    unsigned char *wave_lds = smem + 64 * pitch + wave * kWaveLds;
+    float *part = reinterpret_cast<float *>(smem + 64 * pitch + W * kWaveLds);      // [64][2 G + 1]
+    float *s_bias = part + 64 * (2 * G + 1);                    // [N]
+    const int64_t row_base = static_cast<int64_t>(blockIdx.x) * 64;
+    const int64_t pieces = static_cast<int64_t>(p.N) * (K / 8);
+
+    // The wave's stage-1 tile (wave = (row block rb2, group g): 32 rows x 64 values) is requested first, so that it
+    // travels while the weights are rebuilt.
+    const int rb2 = wave / G, g = wave - rb2 * G;
+    uint4 raw[4];
+    {
+        const int64_t r0 = row_base + rb2 * 32 + lane / 8;
+        const __half *src = p.x + r0 * K + g * 64 + (lane % 8) * 8;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)          // rows past the tensor's end read as zeros
+            raw[i] = (r0 + i * 8 < p.M) ? *reinterpret_cast<const uint4 *>(src + static_cast<int64_t>(i) * 8 * K)
+                                        : make_uint4(0, 0, 0, 0);
+    }
+
+    // ---- this workgroup's share of w_hat: the inputs of this thread's first piece are requested here, the piece is
+    // finished under stage 1's set-up ----
+    int64_t share_lo = 0, share_hi = 0;
+    Piece pc{};
+    unsigned long long target = 0;
+    if (p.counter) {
+        int64_t per = (pieces + gridDim.x - 1) / gridDim.x;
+        per = (per + 7) & ~int64_t(7);                          // whole 128-byte lines per workgroup
+        share_lo = blockIdx.x * per;
+        share_hi = share_lo + per < pieces ? share_lo + per : pieces;
+        if (share_lo + tid < share_hi) fetch_piece<BITS>(p, share_lo + tid, pc);
+    }
+
+    // ---- stage 1: wave = (row block rb2, group g), two lanes per (row, group) ----
+    for (int i = tid; i < p.N; i += nthreads) s_bias[i] = p.bias ? p.bias[i] : 0.0f;
+    {
+        uint32_t *tile = reinterpret_cast<uint32_t *>(wave_lds);
+        float th[L - 1], cbv[L];
+        load_quant_params<BITS>(p.thr, p.cb_a, th, cbv);
+        const BucketScale bq = pick_bucket_scale<BITS>(th);
+        build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, nthreads);     // while the tile is on its way
+        if (p.counter) {
+            if (share_lo + tid < share_hi) finish_piece<BITS>(p, share_lo + tid, pc);
+            for (int64_t idx = share_lo + nthreads + tid; idx < share_hi; idx += nthreads) {     // (large N*K only)
+                fetch_piece<BITS>(p, idx, pc);
+                finish_piece<BITS>(p, idx, pc);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the written-through pieces have reached memory
+        }
+        const int row = lane >> 1, half = lane & 1;
+        {
+            uint32_t *dst = tile + (lane / 8) * kInPitch + (lane % 8) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                uint32_t *d = dst + i * 8 * kInPitch;
+                d[0] = raw[i].x; d[1] = raw[i].y; d[2] = raw[i].z; d[3] = raw[i].w;
+            }
+        }
+        __syncthreads();                          // the tables are complete, and so is the workgroup's share of w_hat
+        if (p.counter && tid == 0) {
+            const unsigned long long inc = blockIdx.x == 0 ? kEpoch - (gridDim.x - 1) : 1ull;
+            const unsigned long long old = __hip_atomic_fetch_add(p.counter, inc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            target = (old & ~(kEpoch - 1)) + kEpoch;            // every launch adds kEpoch in total
+        }
+        float xv[32];
+        {
+            const uint32_t *src = tile + row * kInPitch + half * 16;
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                const uint32_t w = src[q];
+                xv[2 * q] = __half2float(__ushort_as_half(static_cast<unsigned short>(w & 0xffffu)));
+                xv[2 * q + 1] = __half2float(__ushort_as_half(static_cast<unsigned short>(w >> 16)));
+            }
+        }
+        if (p.gamma) {
+            // LayerNorm over the row, arithmetic and summation order of act_quant_rows_ln_kernel: every lane folds its
+            // 32 values serially, the 2 G partial sums of a row meet in LDS and are added group by group, lower half
+            // first; y = ((x - mean) * rstd) * gamma + beta, rounded to fp16 as a LayerNorm kernel would store it.
+            const float fk = static_cast<float>(K);
+            const int ppitch = 2 * G + 1;
+            float *prow = part + (rb2 * 32 + row) * ppitch;
+            auto row_total = [&](float mine) {
+                prow[2 * g + half] = mine;
+                __syncthreads();
+                float acc = 0.0f;
+                for (int i = 0; i < 2 * G; ++i) acc += prow[i];
+                __syncthreads();
+                return acc;
+            };
+            float a = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 32; ++j) a += xv[j];
+            const float mean = row_total(a) / fk;
+            float q = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 32; ++j) {
+                xv[j] -= mean;
+                const float sq = xv[j] * xv[j];
+                q += sq;
+            }
+            const float var_row = row_total(q) / fk;
+            const float rstd = 1.0f / sqrtf(var_row + p.ln_eps);
+            const float4 *gp = reinterpret_cast<const float4 *>(p.gamma + g * 64 + half * 32);
+            const float4 *bp = reinterpret_cast<const float4 *>(p.beta + g * 64 + half * 32);
+#pragma unroll
+            for (int j4 = 0; j4 < 8; ++j4) {
+                const float4 gv = gp[j4], bv = bp[j4];
+                const float g4[4] = {gv.x, gv.y, gv.z, gv.w}, b4[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float t = xv[4 * j4 + e] * rstd;
+                    const float u = t * g4[e];
+                    xv[4 * j4 + e] = __half2float(__float2half_rn(u + b4[e]));
+                }
+            }
+        }
+        bool table_ok = true;
+        for (int w = 0; w < W; ++w) table_ok = table_ok && (slow_slots[w] == 0);
+        float mu, var, s, sum_codes;
+        group_stats32x2(xv, p.eps, mu, var, s);
+        group_codes32x2<BITS>(xv, mu, var, s, th, bq, table, lut, table_ok, lane, sum_codes);
+        const float code_mean = sum_codes * 0.015625f;
+        unsigned char *dst = xs + (rb2 * 32 + row) * pitch + g * 128 + half * 64;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            u32x4_t o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int j = 8 * q4 + 2 * e;
+                const __half2 h = __floats2half2_rn(fma_f32(s, xv[j] - code_mean, mu), fma_f32(s, xv[j + 1] - code_mean, mu));
+                o[e] = *reinterpret_cast<const uint32_t *>(&h);
+            }
+            *reinterpret_cast<u32x4_t *>(dst + q4 * 16) = o;
+        }
+    }
+
+    // ---- every share of w_hat written? ----
+    if (p.counter && tid == 0) {
+        int ok = 1;
+        const long long t0 = wall_clock64();
+        while (__hip_atomic_load(p.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+            if (wall_clock64() - t0 > kSpinTicks) {
+                ok = 0;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(4);
+        }
+        s_flag = ok;
+    }
+    // One wave drops whatever this CU's L1 and this XCD's L2 may hold of the workspace (nothing, unless a line was
+    // fetched before its writer was done), before anyone reads it.
+    if (p.counter && wave == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    __syncthreads();                              // x_hat is complete in LDS; s_flag is set
+    if (p.counter) {
+        if (!s_flag) {                            // workgroup-uniform
+            for (int64_t idx = tid; idx < pieces; idx += nthreads) {
+                fetch_piece<BITS>(p, idx, pc);
+                finish_piece<BITS>(p, idx, pc);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+    }
+
+    // ---- the product: wave tile = 64 rows x one 32-column block; blocks wave, wave + W, ... ----
+    const int lr = lane & 31, lh = lane >> 5;
+    const int ncb = p.N / 32;
+    const unsigned char *xs_lane = xs + lr * pitch + lh * 64;
+    const char *w_lane = reinterpret_cast<const char *>(p.w_blk) + lh * 2048 + lr * 16;
+    const int64_t cb_bytes = static_cast<int64_t>(K) * 64;     // bytes per 32-column block
+    int ld_cb = wave, ld_g = 0;
+    auto load_unit = [&](u32x4_t (&r)[4]) {      // the four fragments of one group; past the wave's last block it re-reads a valid one
+        const int c = ld_cb < ncb ? ld_cb : ncb - 1;
+        const char *q = w_lane + c * cb_bytes + ld_g * 4096;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) r[kk] = *reinterpret_cast<const u32x4_t *>(q + kk * 512);
+        if (++ld_g == G) {
+            ld_g = 0;
+            ld_cb += W;
+        }
+    };
+    // Ring of RING groups, walked with compile-time slot numbers: group number s (counted over the wave's column
+    // blocks) sits in slot s % RING and, once multiplied, its slot takes group s + RING - 1.  kUnroll column blocks
+    // bring the ring back to where it started.
+    constexpr int kUnroll = RING / gcd_of(G, RING);
+    static_assert((kUnroll * G) % RING == 0, "ring does not close");
+    u32x4_t ring[RING][4];
+#pragma unroll
+    for (int i = 0; i < RING - 1; ++i) load_unit(ring[i]);
+
+    constexpr int kSlots = 2 * AHEAD;
+    constexpr int kStageRow = 32 * static_cast<int>(sizeof(TOUT)) + 16;      // bytes per staged output row
+    constexpr int kVec = 16 / static_cast<int>(sizeof(TOUT));
+    constexpr int kPiecesPerRow = 32 / kVec;                                  // 4 (fp16) / 8 (fp32)
+    constexpr int kRowsPerInstr = 64 / kPiecesPerRow;                         // 16 / 8
+    TOUT *y = static_cast<TOUT *>(p.y);
+    const TOUT *residual = static_cast<const TOUT *>(p.residual);
+
+    for (int cb0 = wave; cb0 < ncb; cb0 += kUnroll * W) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int cbk = cb0 + u * W;
+        if (cbk >= ncb) break;
+        float16_t acc[2];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[rb][v] = 0.0f;
+        half8_t xf[kSlots][2];
+#pragma unroll
+        for (int a = 0; a < AHEAD; ++a)
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb)
+                xf[a][rb] = *reinterpret_cast<const half8_t *>(xs_lane + rb * 32 * pitch + a * 16);
+#pragma unroll
+        for (int gl = 0; gl < G; ++gl) {
+            const u32x4_t (&cur_set)[4] = ring[(u * G + gl) % RING];
+            u32x4_t (&load_set)[4] = ring[(u * G + gl + RING - 1) % RING];
+            const unsigned char *xsrc = xs_lane + gl * 128;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const int t = kk + AHEAD;           // the k-step whose x_hat fragments are read now; t >= 4: of the next group
+                const int off = t < 4 ? t * 16 : 128 + (t - 4) * 16;      // (past the row on the last group: unused)
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb)
+                    xf[t % kSlots][rb] = *reinterpret_cast<const half8_t *>(xsrc + rb * 32 * pitch + off);
+                if (kk == 1) load_unit(load_set);
+                half8_t wf;
+                __builtin_memcpy(&wf, &cur_set[kk], 16);
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb)
+                    acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf, xf[kk % kSlots][rb], acc[rb], 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // 1 MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 // 1 LDS read
+                    if (kk == 1) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);    // 2 global loads
+                }
+            }
+        }
+
+        // ---- epilogue: bias, rounding, optional GELU / residual; 32 x 32 outputs at a time through the wave's
+        // staging tile so that every lane stores 16 contiguous bytes ----
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+            float4 bv[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) bv[q] = *reinterpret_cast<const float4 *>(s_bias + cbk * 32 + 8 * q + 4 * lh);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int cl = 8 * q + 4 * lh;
+                const float o0 = acc[rb][4 * q] + bv[q].x, o1 = acc[rb][4 * q + 1] + bv[q].y;
+                const float o2 = acc[rb][4 * q + 2] + bv[q].z, o3 = acc[rb][4 * q + 3] + bv[q].w;
+                unsigned char *dst = wave_lds + lr * kStageRow + cl * static_cast<int>(sizeof(TOUT));
+                if constexpr (sizeof(TOUT) == 2) {
+                    const __half2 lo = __floats2half2_rn(o0, o1), hi = __floats2half2_rn(o2, o3);
+                    u32x2_t pk;
+                    pk[0] = *reinterpret_cast<const uint32_t *>(&lo);
+                    pk[1] = *reinterpret_cast<const uint32_t *>(&hi);
+                    *reinterpret_cast<u32x2_t *>(dst) = pk;
+                } else {
+                    u32x4_t pk;
+                    pk[0] = __float_as_uint(o0); pk[1] = __float_as_uint(o1);
+                    pk[2] = __float_as_uint(o2); pk[3] = __float_as_uint(o3);
+                    *reinterpret_cast<u32x4_t *>(dst) = pk;
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+            const int col = cbk * 32 + (lane % kPiecesPerRow) * kVec;
+#pragma unroll
+            for (int i = 0; i < 32 / kRowsPerInstr; ++i) {
+                const int r = i * kRowsPerInstr + lane / kPiecesPerRow;
+                u32x4_store_t v = *reinterpret_cast<const u32x4_store_t *>(wave_lds + r * kStageRow + (lane % kPiecesPerRow) * 16);
+                const int64_t grow = row_base + rb * 32 + r;
+                if (grow < p.M) {
+                    if (residual || p.gelu)
+                        post_ops16<TOUT>(v, residual ? residual + grow * p.N + col : nullptr, p.gelu != 0, kVec);
+                    store_streaming16(y + grow * p.N + col, v[0], v[1], v[2], v[3]);
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+      }
+    }
+}
+
+// One counter per stream (calls on one stream run one after another; calls on different streams may overlap and must
+// not count into the same word).  The counters live in device memory that is zero when the code object is loaded.
+constexpr int kCounterSlots = 256;
+__device__ unsigned long long g_rows_counters[kCounterSlots];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_rows_mutex;
+unsigned long long *g_counters_ptr[kMaxDevices];
+void *g_slot_stream[kMaxDevices][kCounterSlots];
+int g_slots_used[kMaxDevices];
+
+// Device address of the counter of `stream` on the current device; nullptr if it cannot be had.
+unsigned long long *counter_for(hipStream_t stream)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_rows_mutex);
+    if (!g_counters_ptr[dev]) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_rows_counters)) != hipSuccess || !ptr) return nullptr;
+        g_counters_ptr[dev] = static_cast<unsigned long long *>(ptr);
+    }
+    int slot = -1;
+    for (int i = 0; i < g_slots_used[dev]; ++i)
+        if (g_slot_stream[dev][i] == static_cast<void *>(stream)) slot = i;
+    if (slot < 0) {
+        if (g_slots_used[dev] == kCounterSlots) return nullptr;      // more streams than counters: the caller falls back
+        slot = g_slots_used[dev]++;
+        g_slot_stream[dev][slot] = static_cast<void *>(stream);
+    }
+    return g_counters_ptr[dev] + slot;
+}
+
+size_t rows_lds_bytes(int N, int K)
+{
+    const int G = K / 64;
+    return static_cast<size_t>(64) * (K * 2 + 16) + static_cast<size_t>(2 * G) * kWaveLds + 64 * (2 * G + 1) * sizeof(float) +
+           static_cast<size_t>(N) * sizeof(float);
+}
+
+template <int BITS, typename TOUT, int G, int RING, int AHEAD>
+void launch_rows_g(const RowsParams &p, size_t smem, hipStream_t stream)
+{
+    allow_dynamic_lds<otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>>(160 * 1024 - 10 * 1024);
+    hipLaunchKernelGGL((otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>), dim3((p.M + 63) / 64), dim3(128 * G), smem, stream, p);
+}
+
+// Three fragment groups per wave (a fourth in flight changed nothing: the stream from L2 is bound by throughput, not
+// latency, and the registers are better left to the compiler).
+template <int BITS, typename TOUT>
+void launch_rows(const RowsParams &p, size_t smem, hipStream_t stream)
+{
+    constexpr int kRing = 3;
+    if (p.G == 3) launch_rows_g<BITS, TOUT, 3, kRing, 2>(p, smem, stream);
+    else if (p.G == 4) launch_rows_g<BITS, TOUT, 4, kRing, 2>(p, smem, stream);
+    else launch_rows_g<BITS, TOUT, 6, kRing, 2>(p, smem, stream);
+}
+
+}  // namespace
+
+bool otf_rows_supported(int64_t M, int64_t N, int64_t K)
+{
+    if (M < 512 || M >= (int64_t(1) << 31) - 64 || (K != 192 && K != 256 && K != 384) || N < 32 || N % 32 != 0 ||
+        N > 16384)
+        return false;
+    return rows_lds_bytes(static_cast<int>(N), static_cast<int>(K)) <= 160 * 1024 - 10 * 1024;
+}
+
+bool otf_rows_pays(int64_t M, int64_t N, int64_t K)
+{
+    if (!otf_rows_supported(M, N, K) || tuning().gemm_kernel) return false;
+    const char *e = tuning().rows;
+    if (e) return e[0] != '0';
+    return true;
+}
+
+int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream)
+{
+    RowsParams p{};
+    p.x = static_cast<const __half *>(a.x);
+    p.thr = a.a_thr, p.cb_a = a.a_cb, p.eps = a.eps;
+    p.gamma = a.ln_weight, p.beta = a.ln_bias, p.ln_eps = a.ln_eps;
+    p.pw = a.pw, p.cb_w = a.w_cb, p.wc = a.wc, p.ws = a.ws, p.wcs = a.wcs;
+    p.w_blk = static_cast<__half *>(a.w_hat_ws);
+    p.counter = counter_for(stream);
+    if (!p.counter) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf: no counter left for this stream");
+    p.bias = a.bias, p.y = a.y, p.residual = a.residual, p.gelu = a.gelu ? 1 : 0;
+    p.M = a.M, p.N = a.N, p.G = a.K / 64;
+    const size_t smem = rows_lds_bytes(a.N, a.K);
+    if (a.y_f16) {
+        if (a.bits == 4) launch_rows<4, __half>(p, smem, stream);
+        else if (a.bits == 3) launch_rows<3, __half>(p, smem, stream);
+        else launch_rows<2, __half>(p, smem, stream);
+    } else {
+        if (a.bits == 4) launch_rows<4, float>(p, smem, stream);
+        else if (a.bits == 3) launch_rows<3, float>(p, smem, stream);
+        else launch_rows<2, float>(p, smem, stream);
+    }
+    return launch_status("arcq_linear_otf");
+}
+
+}  // namespace arcq

@@ -79,9 +79,10 @@ def test_model_forward_layerwise_fullbatch(cuda, oracle, model, bits, batch, dep
 @pytest.mark.parametrize("bits", [4, 3])
 def test_benchmarked_layer_call_fullsize(cuda, oracle, name, k, n, bits):
     """ops.linear_otf(..., w_hat_ws=ws) -- arcq_linear_otf_ws, the call bench.py times -- at M = 12 608 for the four
-    DeiT-S shapes: the activation workspace holds the oracle's x_hat bit for bit (in the library's 32-row block
-    layout, which this path uses from 512 rows on), the weight workspace the oracle's w_hat, and sampled rows of y
-    match the fp64 oracle within the fp32-accumulation bound plus one fp16 rounding."""
+    DeiT-S shapes: where the layer runs as two launches the activation workspace holds the oracle's x_hat bit for bit
+    (in the library's 32-row block layout), the weight workspace the oracle's w_hat (row-major, or in 32-column
+    blocks after the one-launch kernel), and sampled rows of y match the fp64 oracle within the fp32-accumulation
+    bound plus one fp16 rounding."""
     m = 64 * synth.TOKENS
     cb = synth.quantile_codebook(bits)
     thr = synth.midpoint_thresholds(cb)
@@ -103,6 +104,9 @@ def test_benchmarked_layer_call_fullsize(cuda, oracle, name, k, n, bits):
         assert np.array_equal(_np(x_ws).view(np.uint16), _np(_to_blocked(torch.from_numpy(a))).view(np.uint16)), path
     if path.endswith("<copy>") or "pair" in path:       # the stage-1 launch rebuilt the weights
         assert np.array_equal(_np(w_ws).view(np.uint16), w16.reshape(-1).view(np.uint16)), path
+    if path == "otf_rows_kernel":                       # one launch: x_hat stays in LDS, w_hat in 32-column blocks
+        blocked = np.ascontiguousarray(w16.reshape(n // 32, 32, k // 8, 8).transpose(0, 2, 1, 3)).reshape(-1)
+        assert np.array_equal(_np(w_ws).view(np.uint16), blocked.view(np.uint16)), path
     rows = torch.randint(0, m, (64,), generator=torch.Generator().manual_seed(3))
     rows[0], rows[1] = 0, m - 1
     y64, mag = oracle.linear_f64_c(a[rows.numpy()], w16, bias.numpy())

@@ -364,7 +364,15 @@ def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
     # The whole-layer entry point with scratch workspaces: whole 32-row blocks from 512 rows on take the block layout.
     monkeypatch.delenv("ARCQ_GEMM_KERNEL")
     both8 = b"gemm_slab8_kernel<copy>"
+    rows = b"otf_rows_kernel"         # short rows (K = 192 / 256 / 384) and both workspaces: the whole layer in one launch
+    assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 1) == rows
+    assert lib.arcq_linear_otf_ws_kernel(12608, 576, 192, 1) == rows
+    assert lib.arcq_linear_otf_ws_kernel(1000, 1024, 256, 1) == rows                        # any number of rows from 512 on
+    assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 320, 1) == both8                     # (no instance for five groups)
+    assert lib.arcq_linear_otf_ws_kernel(12608, 1000, 384, 1) == both8                     # (N must be whole 32-column blocks)
+    monkeypatch.setenv("ARCQ_ROWS", "0")
     assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 1) == both8                     # the rebuild rides in stage 1
+    monkeypatch.delenv("ARCQ_ROWS")
     assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 0) == b"gemm_slab8_kernel"
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 1) == both8
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 0) == b"gemm_slab8_kernel"
