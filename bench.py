@@ -119,15 +119,20 @@ class Layer:
 
     # The two halves of arcq_linear_otf_ws on their own.  Block-layout shapes: arcq_act_quant_blocked_with_weights
     # (stage 1 plus the weight reconstruction carried in the same launch) and arcq_linear_fused_blocked on weights
-    # that are ready; other shapes: arcq_act_quant and arcq_linear_fused_ws.
+    # that are ready; other shapes: arcq_act_quant and arcq_linear_fused_ws.  A layer that runs as ONE launch
+    # ("rows": otf_rows_kernel, stage 1 + weight reconstruction + GEMM) has no halves: call_act does nothing and
+    # call_gemm is the whole layer.
     def mode(self, lib, m):
         name = lib.arcq_linear_otf_ws_kernel(m, self.n, self.k, 1)
-        return ("copy" if name in (b"gemm_slab8_kernel<copy>", b"gemm_pair_kernel") else
+        return ("rows" if name == b"otf_rows_kernel" else
+                "copy" if name in (b"gemm_slab8_kernel<copy>", b"gemm_pair_kernel") else
                 "blocked" if b"slab8" in name else "rowmajor")
 
     def call_act(self, lib, x, ws, stream):
         from arcq_vit_amd._lib import ARCQ_F16
         mode = self.mode(lib, x.shape[0])
+        if mode == "rows":
+            return 0
         if mode == "copy":
             return lib.arcq_act_quant_blocked_with_weights(
                 x.data_ptr(), ARCQ_F16, self.thr.data_ptr(), self.cb.data_ptr(), ws.data_ptr(), x.shape[0], self.k,
@@ -138,9 +143,11 @@ class Layer:
                                               ws.data_ptr(), x.shape[0], self.k, self.bits, 1.0e-6, stream)
         return lib.arcq_act_quant(*self.act_args(x, ws, stream))
 
-    def call_gemm(self, lib, ws, y, m, stream):
+    def call_gemm(self, lib, ws, y, m, stream, x=None):
         from arcq_vit_amd._lib import ARCQ_F16
         mode = self.mode(lib, m)
+        if mode == "rows":
+            return lib.arcq_linear_otf_ws(*self.otf_args(x, ws, y, stream))
         if mode == "rowmajor":
             return lib.arcq_linear_fused_ws(*self.gemm_args(ws, y, m, stream))
         # "copy": W_WS holds some layer's reconstructed weights of at least this size (timing does not depend on which)
@@ -149,9 +156,12 @@ class Layer:
             self.code_sum.data_ptr(), self.bias.data_ptr(), Layer.W_WS.data_ptr() if mode == "copy" else 0,
             1 if mode == "copy" else 0, y.data_ptr(), ARCQ_F16, m, self.n, self.k, self.bits, 64, stream)
 
-    def call_gemm_rebuild_inside(self, lib, ws, y, m, stream):
-        """The fused GEMM with the weights reconstructed inside the kernel (no weight workspace at all)."""
+    def call_gemm_rebuild_inside(self, lib, ws, y, m, stream, x=None):
+        """The fused GEMM with the weights reconstructed inside the kernel (no weight workspace at all); a one-launch
+        layer as it is (its weights are rebuilt inside its launch anyway)."""
         from arcq_vit_amd._lib import ARCQ_F16
+        if self.mode(lib, m) == "rows":
+            return lib.arcq_linear_otf_ws(*self.otf_args(x, ws, y, stream))
         if self.mode(lib, m) == "rowmajor":
             return lib.arcq_linear_fused(ws.data_ptr(), self.packed.data_ptr(), self.cb.data_ptr(), self.center.data_ptr(),
                                          self.scale.data_ptr(), self.code_sum.data_ptr(), self.bias.data_ptr(),
@@ -234,13 +244,13 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
 
     def step_gemm():
         for l in layers:
-            rc = l.call_gemm(lib, ws, y, m, stream)
+            rc = l.call_gemm(lib, ws, y, m, stream, inputs[short(l)])
             if rc:
                 _lib.check(rc)
 
     def step_gemm_inside():
         for l in layers:
-            rc = l.call_gemm_rebuild_inside(lib, ws, y, m, stream)
+            rc = l.call_gemm_rebuild_inside(lib, ws, y, m, stream, inputs[short(l)])
             if rc:
                 _lib.check(rc)
 
@@ -259,9 +269,9 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
                     elif kind == "act":
                         rc = l.call_act(lib, x, ws, sp)
                     elif kind == "inside":
-                        rc = l.call_gemm_rebuild_inside(lib, ws, y, m, sp)
+                        rc = l.call_gemm_rebuild_inside(lib, ws, y, m, sp, x)
                     else:
-                        rc = l.call_gemm(lib, ws, y, m, sp)
+                        rc = l.call_gemm(lib, ws, y, m, sp, x)
                     if rc:
                         _lib.check(rc)
             return g.replay
@@ -289,7 +299,7 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
         else:
             def fn(sub=sub):
                 for l in sub:
-                    l.call_gemm(lib, ws, y, m, stream)
+                    l.call_gemm(lib, ws, y, m, stream, inputs[short(l)])
         t = time_loop(fn, steps, warmup)
         kf = sum(synth.algorithmic_flops(m, l.n, l.k) for l in sub)
         kb = sum(synth.algorithmic_bytes(m, l.n, l.k, bits) for l in sub)
@@ -299,9 +309,11 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
                             "bytes_per_launch": kb / len(sub),
                             "shapes_nk": sorted({(l.n, l.k) for l in sub})}
 
+    act_layers = [l for l in layers if l.mode(lib, m) != "rows"]          # layers with a stage-1 launch of their own
+    n_act = max(len(act_layers), 1)
     flops = sum(synth.algorithmic_flops(m, l.n, l.k) for l in layers)
     gemm_bytes = sum(synth.algorithmic_bytes(m, l.n, l.k, bits) for l in layers)
-    act_bytes = sum(2 * 2 * m * l.k for l in layers)          # fp16 in, fp16 out
+    act_bytes = sum(2 * 2 * m * l.k for l in act_layers)          # fp16 in, fp16 out
     res = {
         "batch": batch, "M": m, "layers": len(layers),
         "ms_per_step": t_full / steps * 1e3,
@@ -313,13 +325,14 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
         "gemm_rebuild_inside_us_per_launch": t_inside / steps / len(layers) * 1e6,
         "gemm_rebuild_inside_tflops": flops * steps / t_inside / 1e12,
         "act_ms_per_step": t_act / steps * 1e3,
-        "act_us_per_launch": t_act / steps / len(layers) * 1e6,
+        "act_us_per_launch": t_act / steps / n_act * 1e6, "act_launches_per_step": len(act_layers),
         "act_gbs": act_bytes * steps / t_act / 1e9,
         "flops_per_step": flops, "gemm_bytes_per_step": gemm_bytes, "gemm_kernels": per_kernel,
         # stage-1 kernel of the first layer's shape (the large-M layers all take the same one)
         "act_kernel": {"copy": "act_quant_blocked2_kernel (block layout, weight reconstruction carried along)",
                        "blocked": "act_quant_blocked2_kernel (block layout)",
-                       "rowmajor": "act_quant_g64_kernel / act_quant_small_kernel (row-major)"}[layers[0].mode(lib, m)],
+                       "rowmajor": "act_quant_g64_kernel / act_quant_small_kernel (row-major)"}[
+                           (act_layers or layers)[0].mode(lib, m) if act_layers else "copy"],
     }
     return res, layers, inputs
 
@@ -454,6 +467,9 @@ def model_forward(model, bits, batches, steps, warmup, dev):
 
 
 def kernel_note(name):
+    if name == "otf_rows_kernel":
+        return ("the WHOLE layer in one launch: stage 1 of 64 rows into LDS, the fp16 weights reconstructed cooperatively "
+                "into the workspace, fp16 MFMA GEMM + bias; its duration includes stage 1 and the reconstruction")
     if name in ("gemm_slab8_kernel<copy>", "gemm_pair_kernel"):
         return ("fp16 MFMA GEMM + bias on weights that the stage-1 launch of the same layer reconstructed into an "
                 "fp16 workspace (copied global -> LDS); its own launch does no dequantization")
@@ -505,8 +521,8 @@ def main():
         "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"{args.model} {res['layers']} packed linears ({res['layers'] // 4} blocks x qkv/proj/fc1/fc2), W{args.bits}A{args.bits}, "
-                               f"g=64, batch {args.batch} (M={res['M']}), fp16 in/out; per layer: stage 1 (activation quantize + reconstruct, the fp16 weights "
-                               f"reconstructed in the same launch) then an fp16 MFMA GEMM + bias on them",
+                               f"g=64, batch {args.batch} (M={res['M']}), fp16 in/out; per layer: stage 1 (activation quantize + reconstruct), the fp16 weights "
+                               f"reconstructed from the packed codes, an fp16 MFMA GEMM + bias -- one launch for K <= 384, two launches otherwise",
                    "model_shapes": args.model, "bits": args.bits, "batch": args.batch, "group_size": 64},
         "roofline": {"bound": "mfma", "kernel": dom, "kernel_does": kernel_note(dom), "achieved": dk["tflops"],
                      "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": dk["tflops"] / PEAK_FP16_TFLOPS,
@@ -522,6 +538,7 @@ def main():
                      "weights_rebuilt_inside_gemm": {"tflops": res["gemm_rebuild_inside_tflops"],
                                                      "avg_launch_us": res["gemm_rebuild_inside_us_per_launch"],
                                                      "frac": res["gemm_rebuild_inside_tflops"] / PEAK_FP16_TFLOPS},
+                     # all_fused_gemm_launches counts a one-launch layer whole (stage 1 included)
                      # whole layer = stage 1 (+ weight reconstruction) + GEMM, everything the step runs
                      "layer": layer_roofline(res, args.bits)},
         "stage1": {"kernel": res["act_kernel"], "bound": "hbm", "achieved": res["act_gbs"], "peak": PEAK_HBM_GBS,

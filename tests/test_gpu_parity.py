@@ -215,6 +215,47 @@ def test_stage1_two_lane_fallback_paths(cuda, oracle):
     check(const, thr)
 
 
+@pytest.mark.parametrize("bits", [4, 3, 2])
+def test_stage1_threshold_neighbourhoods(cuda, oracle, bits):
+    """Hard cases for the code decision t > thr with t = RN(d/s): thresholds that ARE occurring t values (exact ties:
+    false), their neighbours one ulp below (true) and above, thresholds on round values and on / next to the
+    boundaries of the kernels' lookup buckets (whole and shifted grids of 1/4 and 1/8), and a large launch for
+    coverage; x_hat must equal the oracle's bit for bit in the small kernel, the block layout and fp16."""
+    cb = synth.quantile_codebook(bits)
+    n_thr = (1 << bits) - 1
+    x = synth.make_activation(640, 384, 17)
+    d = lambda t: t.to(cuda)
+
+    def check(xx, tt):
+        want = oracle.act_quant_c(xx.numpy(), tt, cb, bits, 64)["x_hat"]
+        got = ops.dequant_activation_hip(d(xx), d(tt), d(cb), 64)
+        assert np.array_equal(_np(got).view(np.uint32), want.view(np.uint32))
+        blk = ops.quantize_activation_blocked(d(xx), d(tt), d(cb), bits).reshape(-1)
+        assert np.array_equal(_np(blk).view(np.uint16),
+                              _np(_to_blocked(torch.from_numpy(want.astype(np.float16)))).view(np.uint16))
+        h = xx.to(torch.float16)
+        want16 = oracle.act_quant_c(h.float().numpy(), tt, cb, bits, 64)["x_hat"].astype(np.float16)
+        assert np.array_equal(_np(ops.dequant_activation_hip(d(h), d(tt), d(cb), 64)).view(np.uint16), want16.view(np.uint16))
+
+    ref0 = oracle.act_quant_c(x.numpy(), synth.midpoint_thresholds(cb), cb, bits, 64)
+    t = ((x.numpy().reshape(640, 6, 64) - ref0["center"][..., None]) / ref0["scale"][..., None]).astype(np.float32)
+    u = np.sort(np.unique(t[np.abs(t) < 2.0]))
+    ties = u[np.linspace(50, u.size - 51, n_thr).astype(np.int64)].copy()
+    for thr in (ties, np.nextafter(ties, np.float32(-np.inf)), np.nextafter(ties, np.float32(np.inf))):
+        thr = torch.from_numpy(thr.astype(np.float32))
+        assert bool((thr[1:] - thr[:-1] > 0.13).all())          # wide apart: the coarse bucket table is in use
+        check(x, thr)
+    grid = torch.linspace(-1.75, 1.75, n_thr).mul(8).round().div(8)          # round values: 0, 1/4, 1/2 ...
+    check(x, grid)
+    for scale in (4.0, 8.0):                   # a grid shifted by a fraction of a bucket
+        edge = (grid * scale - 0.381966) / scale
+        check(x, edge)
+        check(x, torch.from_numpy(np.nextafter(edge.numpy(), np.float32(np.inf))))
+        check(x, edge + 3.0e-6)
+    big = synth.make_activation(12608, 384, 18)
+    check(big, synth.midpoint_thresholds(cb))
+
+
 def test_stage1_empty(cuda):
     cb, thr = _cb(4)
     out = ops.quantize_activation(torch.zeros((0, 128), device=cuda), thr.to(cuda), cb.to(cuda), 4, 64)
