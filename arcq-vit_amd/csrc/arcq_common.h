@@ -108,6 +108,46 @@ inline void allow_dynamic_lds(int bytes)
     done.fetch_or(bit, std::memory_order_release);
 }
 
+// Order of the (row range, slab) tiles of a weight-stationary GEMM whose slabs are copied from a reconstructed
+// weight matrix.  Workgroups are dealt to the 8 XCDs round-robin and every XCD takes a contiguous run of tile numbers;
+// with the slab fastest a run covers all N / 128 slabs of one or two row ranges, so that the slabs sharing a range read
+// x_hat through one L2 -- but once K spans several slab slices every pass over the rows copies the slab again, and
+// N * K * 2 bytes of weights per XCD (6 MB for ViT-L qkv) do not stay in its 4 MB L2: measured at the L2, the launch
+// then fetched 3.5 times the x_hat it needs.  Slabs are therefore dealt in groups whose weights fit half the L2
+// (`group` slabs: 2 MB / (128 * K * 2), groups of equal size): a run then covers one group x several ranges, the
+// re-copies hit L2, and x_hat is fetched once per group instead of once.  That trade is taken only where it saves
+// traffic by this estimate: x_hat (M * K * 2 bytes) once more per additional group, against the weights
+// (N * K * 2 bytes) once more per XCD and per pass after the first (`blocks_per_pass` = row blocks a workgroup
+// multiplies per pass over K).  DeiT-B qkv / fc1: 58.8 -> 53.5 and 77.3 -> 68.5 us; ViT-L qkv / fc1: 1 % faster;
+// ViT-L fc2 (K = 4096: x_hat is 413 MB) keeps the plain order, which is 2.4 % faster there.
+__host__ __device__ inline int slab_group_size(int n_slabs, int K, int M, int blocks_per_range, int blocks_per_pass)
+{
+    const int64_t slab_bytes = int64_t(128) * K * 2;
+    const int fit = static_cast<int>((int64_t(2) << 20) / slab_bytes);
+    if (fit >= n_slabs) return n_slabs;
+    const int passes = (blocks_per_range + blocks_per_pass - 1) / blocks_per_pass;
+    if (fit < 1 || passes <= 1) return n_slabs;
+    const int groups = (n_slabs + fit - 1) / fit;
+    const int64_t extra_x = int64_t(M) * K * 2 * (groups - 1);
+    const int64_t rereads_w = 8 * n_slabs * slab_bytes * (passes - 1);
+    return extra_x < rereads_w ? (n_slabs + groups - 1) / groups : n_slabs;
+}
+__device__ __forceinline__ void tile_range_slab(int tile, int n_slabs, int row_ranges, int group, int &range, int &slab)
+{
+    if (group >= n_slabs) {
+        range = tile / n_slabs;
+        slab = tile - range * n_slabs;
+        return;
+    }
+    const int per_group = group * row_ranges;       // tiles of a full group
+    const int sg = tile / per_group;
+    const int first = sg * group;
+    const int size = min(group, n_slabs - first);
+    const int rem = tile - sg * per_group;
+    range = rem / size;
+    slab = first + (rem - range * size);
+}
+
 __device__ __forceinline__ float to_float(float v) { return v; }
 __device__ __forceinline__ float to_float(__half v) { return __half2float(v); }
 

@@ -75,16 +75,18 @@ gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, 
     const int lh = lane >> 5;
     const int G = K / 64;
 
-    // Tile = (row range, slab), slab fastest; each XCD (workgroups are dealt to the 8 XCDs round-robin) takes a
-    // contiguous run of tiles so that the slabs sharing a row range read x_hat through one L2.
+    // Tile = (row range, slab); each XCD (workgroups are dealt to the 8 XCDs round-robin) takes a contiguous run of
+    // tiles, ordered as tile_range_slab describes.
     const int n_slabs = (N + kSlabN - 1) / kSlabN;
     const int tiles = n_slabs * row_ranges;
     const int per_xcd = (tiles + 7) / 8;
     const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (tile >= tiles) return;
-    const int n_base = (tile % n_slabs) * kSlabN;
+    int tile_range, tile_slab;
+    tile_range_slab(tile, n_slabs, row_ranges, slab_group_size(n_slabs, K, M, blocks_per_range, 2 * kWaves), tile_range, tile_slab);
+    const int n_base = tile_slab * kSlabN;
     const int total_blocks = (M + 31) / 32;
-    const int blk0 = (tile / n_slabs) * blocks_per_range;
+    const int blk0 = tile_range * blocks_per_range;
     const int blk1 = min(total_blocks, blk0 + blocks_per_range);
     const int nblk = blk1 - blk0;
     const int full_passes = nblk / (2 * kWaves);       // every wave multiplies a pair of blocks

@@ -107,9 +107,12 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     const int per_xcd = (tiles + 7) / 8;
     const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (tile >= tiles) return;
-    const int n_base = (tile % n_slabs) * kSlabN;
+    // (weights copied from the workspace: slabs in groups that fit L2, see tile_range_slab)
+    int tile_range, tile_slab;
+    tile_range_slab(tile, n_slabs, row_ranges, PRE ? slab_group_size(n_slabs, K, M, blocks_per_range, kWaves) : n_slabs, tile_range, tile_slab);
+    const int n_base = tile_slab * kSlabN;
     const int total_blocks = (M + 31) / 32;
-    const int blk0 = (tile / n_slabs) * blocks_per_range;
+    const int blk0 = tile_range * blocks_per_range;
     const int blk1 = min(total_blocks, blk0 + blocks_per_range);
     // Row blocks of this wave: blk0 + wave, + 8, + 16, ... (one per pass).  Dealing them round-robin instead of in
     // contiguous runs keeps the four SIMDs (waves w, w + 4, w + 8 share one) within one block of each other.
