@@ -140,8 +140,14 @@ int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const
  * output columns, large models) the weights are rebuilt once into w_hat_ws (arcq_weight_dequant) and the GEMM copies
  * them; for all other shapes, or with w_hat_ws == NULL, these behave exactly like arcq_linear_fused / arcq_linear_otf.
  * y is bit-identical in every case; the contents of w_hat_ws after the call are unspecified.  arcq_linear_otf_ws treats
- * x_hat_ws as scratch too (unspecified contents afterwards: it may hold x_hat in the block layout described below);
- * call arcq_linear_otf to get x_hat row-major in x_hat_ws. */
+ * x_hat_ws as scratch too (unspecified contents afterwards: it may hold x_hat in the block layout described below, or
+ * be left untouched); call arcq_linear_otf to get x_hat row-major in x_hat_ws.
+ * With fp16 x, M >= 512, K = 192 / 256 / 384, N a multiple of 32 and w_hat_ws given, arcq_linear_otf_ws runs the whole
+ * layer as ONE launch (x_hat stays on chip; w_hat_ws is filled cooperatively, in 32-column blocks
+ * [N/32][K/8][32][8]).  That launch counts in a word of the library's static device memory chosen by `stream`: calls
+ * on one stream run one after another as always; a HIP graph captured from a stream must not be replayed
+ * concurrently with other calls made on that same stream; a process can use 256 different streams for such calls
+ * per device (ARCQ_ERR_UNSUPPORTED beyond).  ARCQ_ROWS=0 in the environment keeps the two-launch path. */
 int arcq_linear_fused_ws(const void *x_hat,
                          const uint8_t *packed_w, const float *w_codebook,
                          const float *w_center, const float *w_scale, const float *w_code_sum,
@@ -198,7 +204,8 @@ int arcq_linear_fused_blocked(const void *x_hat_blocked,
  *   residual   [M,N] of y's type, added to the rounded value, rounded again, in the GEMM's epilogue
  * Every step rounds where a separate kernel would have stored its result, so y equals the unfused sequence bit for
  * bit given the same LayerNorm output.  With no option set it is arcq_linear_otf_ws.  With an option set it needs
- * group_size 64 and M >= 512 (the block-layout path) and returns ARCQ_ERR_UNSUPPORTED otherwise: compose the
+ * group_size 64 and M >= 512 (the block-layout path or the one-launch kernel described at arcq_linear_otf_ws, which
+ * then also runs the LayerNorm, GELU and residual) and returns ARCQ_ERR_UNSUPPORTED otherwise: compose the
  * layer from the separate operations then.  Workspaces as arcq_linear_otf_ws (w_hat_ws may be NULL).
  * struct_size = sizeof(arcq_linear_ex_args). */
 #define ARCQ_PRODUCER_NONE 0
