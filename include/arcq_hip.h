@@ -139,6 +139,10 @@ int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const
  * unpack_weight_triton).  For shapes where many workgroups would each repeat the weight reconstruction (long K with few
  * output columns, large models) the weights are rebuilt once into w_hat_ws (arcq_weight_dequant) and the GEMM copies
  * them; for all other shapes, or with w_hat_ws == NULL, these behave exactly like arcq_linear_fused / arcq_linear_otf.
+ * arcq_linear_otf_ws with a workspace and 512 rows or more always takes the workspace route: the fp16 weights are
+ * reconstructed into w_hat_ws inside the layer's first (or only) launch and the GEMM reads them from there, i.e. the
+ * dense weight does pass through memory (L2-resident: at most a few MB) -- the reference's unpack-then-GEMM order,
+ * without a launch of its own.  Without a workspace the weights are reconstructed inside the GEMM kernel.
  * y is bit-identical in every case; the contents of w_hat_ws after the call are unspecified.  arcq_linear_otf_ws treats
  * x_hat_ws as scratch too (unspecified contents afterwards: it may hold x_hat in the block layout described below, or
  * be left untouched); call arcq_linear_otf to get x_hat row-major in x_hat_ws.
