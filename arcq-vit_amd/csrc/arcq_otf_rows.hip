@@ -157,7 +157,11 @@ otf_rows_kernel(const RowsParams p)
         float th[L - 1], cbv[L];
         load_quant_params<BITS>(p.thr, p.cb_a, th, cbv);
         const BucketScale bq = pick_bucket_scale<BITS>(th);
-        build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, nthreads);     // while the tile is on its way
+        // The lookup tables are built by one wave per SIMD while the tiles are on their way (every participating
+        // thread pays ~250 instructions of set-up whether or not it owns a table entry, and stage 1 is
+        // instruction-bound: all 2 G waves building cost 17 % of the phase).
+        constexpr int kBuilders = W < 4 ? W : 4;
+        if (wave < kBuilders) build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * kBuilders);
         if (p.counter) {
             if (share_lo + tid < share_hi) finish_piece<BITS>(p, share_lo + tid, pc);
             for (int64_t idx = share_lo + nthreads + tid; idx < share_hi; idx += nthreads) {     // (large N*K only)
@@ -234,7 +238,7 @@ otf_rows_kernel(const RowsParams p)
             }
         }
         bool table_ok = true;
-        for (int w = 0; w < W; ++w) table_ok = table_ok && (slow_slots[w] == 0);
+        for (int w = 0; w < kBuilders; ++w) table_ok = table_ok && (slow_slots[w] == 0);
         float mu, var, s, sum_codes;
         group_stats32x2(xv, p.eps, mu, var, s);
         group_codes32x2<BITS>(xv, mu, var, s, th, bq, table, lut, table_ok, lane, sum_codes);
