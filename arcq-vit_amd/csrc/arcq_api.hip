@@ -110,11 +110,12 @@ static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds
     if (scratch_only && w_hat_ws && x_dtype == ARCQ_F16 && group_size == 64 && arcq::bits_ok(bits) &&
         arcq::otf_rows_pays(M, N, K) && x && a_thresholds && a_codebook && packed_w && w_codebook && w_center && w_scale &&
         w_code_sum && y && (y_dtype == ARCQ_F16 || y_dtype == ARCQ_F32) && arcq::aligned(x, 16) && arcq::aligned(y, 16) &&
-        arcq::aligned(w_hat_ws, 16) && arcq::aligned(packed_w, 4)) {
+        arcq::aligned(w_hat_ws, 128) && arcq::aligned(packed_w, 4)) {
         arcq::OtfRowsArgs a{x, a_thresholds, a_codebook, nullptr, nullptr, 0.0f, packed_w, w_codebook, w_center, w_scale,
                             w_code_sum, bias, w_hat_ws, y, y_dtype == ARCQ_F16, nullptr, false, static_cast<int>(M),
                             static_cast<int>(N), static_cast<int>(K), bits, 1.0e-6f};
-        return arcq::launch_otf_rows(a, static_cast<hipStream_t>(stream));
+        const int rc = arcq::launch_otf_rows(a, static_cast<hipStream_t>(stream));
+        if (rc != arcq::kNoCounter) return rc;
     }
     // Scratch-only workspaces and 512 rows or more: x_hat in the block layout, eight-wave weight-stationary GEMM
     // (bit-identical results; invalid arguments fall through to the entry points below, which report them).
@@ -187,7 +188,7 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
     if (a->w_hat_ws && a->x_dtype == ARCQ_F16 && arcq::otf_rows_pays(a->M, a->N, a->K) && a->x && a->a_thresholds &&
         a->a_codebook && a->packed_w && a->w_codebook && a->w_center && a->w_scale && a->w_code_sum && a->y &&
         (a->y_dtype == ARCQ_F16 || a->y_dtype == ARCQ_F32) && arcq::aligned(a->x, 16) && arcq::aligned(a->y, 16) &&
-        arcq::aligned(a->w_hat_ws, 16) && arcq::aligned(a->packed_w, 4) &&
+        arcq::aligned(a->w_hat_ws, 128) && arcq::aligned(a->packed_w, 4) &&
         (a->producer != ARCQ_PRODUCER_LAYERNORM || (a->ln_weight && a->ln_bias && arcq::aligned(a->ln_weight, 16) &&
                                                     arcq::aligned(a->ln_bias, 16)))) {
         const bool ln = a->producer == ARCQ_PRODUCER_LAYERNORM;
@@ -195,7 +196,8 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
                             a->ln_eps, a->packed_w, a->w_codebook, a->w_center, a->w_scale, a->w_code_sum, a->bias,
                             a->w_hat_ws, a->y, a->y_dtype == ARCQ_F16, a->residual, a->activation == ARCQ_ACT_GELU,
                             static_cast<int>(a->M), static_cast<int>(a->N), static_cast<int>(a->K), a->bits, 1.0e-6f};
-        return arcq::launch_otf_rows(r, static_cast<hipStream_t>(stream));
+        const int rc = arcq::launch_otf_rows(r, static_cast<hipStream_t>(stream));
+        if (rc != arcq::kNoCounter) return rc;
     }
     const bool carry = a->w_hat_ws && arcq::blocked_uses_workspace(a->N, a->K) && a->packed_w && a->w_codebook && a->w_center &&
                        a->w_scale && a->w_code_sum && arcq::aligned(a->w_hat_ws, 16) && arcq::aligned(a->packed_w, 16);

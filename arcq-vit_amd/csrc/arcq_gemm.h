@@ -88,6 +88,8 @@ struct OtfRowsArgs {
 bool otf_rows_supported(int64_t M, int64_t N, int64_t K);
 // Whether the whole-layer entry points take it for this shape (fp16 input, both workspaces given).
 bool otf_rows_pays(int64_t M, int64_t N, int64_t K);
+// Returns kNoCounter (and launches nothing, records no error) when the stream cannot be given a counter.
+constexpr int kNoCounter = -1000;
 int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream);
 
 }  // namespace arcq

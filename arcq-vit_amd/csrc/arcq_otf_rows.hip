@@ -470,7 +470,8 @@ void launch_rows(const RowsParams &p, size_t smem, hipStream_t stream)
 
 bool otf_rows_supported(int64_t M, int64_t N, int64_t K)
 {
-    if (M < 512 || M >= (int64_t(1) << 31) - 64 || (K != 192 && K != 256 && K != 384) || N < 32 || N % 32 != 0 ||
+    // (at most 2^19 workgroups: what one launch adds to its counter must stay below the counter's epoch)
+    if (M < 512 || M > (int64_t(64) << 19) || (K != 192 && K != 256 && K != 384) || N < 32 || N % 32 != 0 ||
         N > 16384)
         return false;
     return rows_lds_bytes(static_cast<int>(N), static_cast<int>(K)) <= 160 * 1024 - 10 * 1024;
@@ -493,7 +494,7 @@ int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream)
     p.pw = a.pw, p.cb_w = a.w_cb, p.wc = a.wc, p.ws = a.ws, p.wcs = a.wcs;
     p.w_blk = static_cast<__half *>(a.w_hat_ws);
     p.counter = counter_for(stream);
-    if (!p.counter) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf: no counter left for this stream");
+    if (!p.counter) return kNoCounter;       // more streams than counters: the caller takes the two-launch path
     p.bias = a.bias, p.y = a.y, p.residual = a.residual, p.gelu = a.gelu ? 1 : 0;
     p.M = a.M, p.N = a.N, p.G = a.K / 64;
     const size_t smem = rows_lds_bytes(a.N, a.K);

@@ -146,12 +146,14 @@ int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const
  * y is bit-identical in every case; the contents of w_hat_ws after the call are unspecified.  arcq_linear_otf_ws treats
  * x_hat_ws as scratch too (unspecified contents afterwards: it may hold x_hat in the block layout described below, or
  * be left untouched); call arcq_linear_otf to get x_hat row-major in x_hat_ws.
- * With fp16 x, M >= 512, K = 192 / 256 / 384, N a multiple of 32 and w_hat_ws given, arcq_linear_otf_ws runs the whole
+ * With fp16 x, M >= 512, K = 192 / 256 / 384, N a multiple of 32 and w_hat_ws given (128-byte aligned),
+ * arcq_linear_otf_ws runs the whole
  * layer as ONE launch (x_hat stays on chip; w_hat_ws is filled cooperatively, in 32-column blocks
  * [N/32][K/8][32][8]).  That launch counts in a word of the library's static device memory chosen by `stream`: calls
  * on one stream run one after another as always; a HIP graph captured from a stream must not be replayed
- * concurrently with other calls made on that same stream; a process can use 256 different streams for such calls
- * per device (ARCQ_ERR_UNSUPPORTED beyond).  ARCQ_ROWS=0 in the environment keeps the two-launch path. */
+ * concurrently with other calls made on that same stream; the first 256 streams a process uses for such calls on a
+ * device get a word each, calls on further streams take the two-launch path.  ARCQ_ROWS=0 in the environment keeps
+ * the two-launch path everywhere. */
 int arcq_linear_fused_ws(const void *x_hat,
                          const uint8_t *packed_w, const float *w_codebook,
                          const float *w_center, const float *w_scale, const float *w_code_sum,

@@ -54,6 +54,10 @@ def test_rows_kernel_against_oracle_and_two_launch_path(cuda, oracle, monkeypatc
     tol = (k + 2) * 2.0 ** -24 * mag + np.abs(y64) * ulp + 2.0 ** -25
     err = np.abs(_np(y[rows.to(cuda)]).astype(np.float64) - y64)
     assert np.all(err <= tol), float((err / tol).max())
+    # a weight workspace that is not 128-byte aligned (a view 16 bytes into a buffer) takes the two-launch path
+    off = torch.zeros(n * k + 8, dtype=torch.float16, device=cuda)[8:]
+    y1 = ops.linear_otf(d(x), *args, out_dtype=out, w_hat_ws=off)
+    assert torch.equal(y, y1) and np.array_equal(_np(off).view(np.uint16), w16.reshape(-1).view(np.uint16))
     monkeypatch.setenv("ARCQ_ROWS", "0")
     assert _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1) != b"otf_rows_kernel"
     y2 = ops.linear_otf(d(x), *args, out_dtype=out, w_hat_ws=torch.zeros_like(w_ws))
