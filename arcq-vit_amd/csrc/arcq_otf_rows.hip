@@ -67,17 +67,18 @@ struct Piece {
     uint32_t w;
     float c, s, m;
 };
-template <int BITS>
+template <int BITS, int G>
 __device__ __forceinline__ void fetch_piece(const RowsParams &p, int64_t idx, Piece &pc)
 {
-    const int K = 64 * p.G, P = K / 8;
-    const int64_t pcols = static_cast<int64_t>(K) * BITS / 8;
-    const int r = static_cast<int>(idx & 31);
-    const int64_t t = idx >> 5;
-    const int pp = static_cast<int>(t % P);
-    const int64_t n = (t / P) * 32 + r;
+    constexpr int K = 64 * G, P = K / 8, pcols = K * BITS / 8;     // compile-time: the divisions below are multiplications
+    const uint32_t i = static_cast<uint32_t>(idx);                 // N * K / 8 < 2^31 (N <= 16384, K <= 384)
+    const uint32_t r = i & 31u;
+    const uint32_t t = i >> 5;
+    const uint32_t nb = t / P;
+    const uint32_t pp = t - nb * P;
+    const uint32_t n = nb * 32u + r;
     pc.w = load_codes8<BITS>(p.pw + n * pcols + pp * BITS);
-    const int64_t mi = n * p.G + (pp >> 3);
+    const uint32_t mi = n * G + (pp >> 3);
     pc.c = p.wc[mi];
     pc.s = p.ws[mi];
     pc.m = p.wcs[mi] * 0.015625f;      // code_sum / 64, exact
@@ -139,6 +140,14 @@ otf_rows_kernel(const RowsParams p)
 
     // ---- this workgroup's share of w_hat: the inputs of this thread's first piece are requested here, the piece is
     // finished under stage 1's set-up ----
+    // Division of the extra work over the waves (stage 1 is instruction-bound and waves w, w + 4, w + 8 share a SIMD):
+    // waves 1-3 build the activation lookup tables, the others reconstruct the weight pieces -- wave 0 and waves 4..
+    // are piece threads 0..63, 64.. -- so that no SIMD carries more than one builder and one piece wave beside
+    // its plain ones (two piece waves on SIMD 0).
+    constexpr int kBuilders = W < 4 ? 1 : 3;
+    constexpr int kBuilder0 = W < 4 ? 0 : 1;
+    constexpr int kPieceThreads = W < 4 ? 64 * W : 64 * (W - 3);
+    const int ptid = W < 4 ? tid : (wave == 0 ? lane : (wave >= 4 ? (wave - 3) * 64 + lane : -1));
     int64_t share_lo = 0, share_hi = 0;
     Piece pc{};
     unsigned long long target = 0;
@@ -147,7 +156,7 @@ otf_rows_kernel(const RowsParams p)
         per = (per + 7) & ~int64_t(7);                          // whole 128-byte lines per workgroup
         share_lo = blockIdx.x * per;
         share_hi = share_lo + per < pieces ? share_lo + per : pieces;
-        if (share_lo + tid < share_hi) fetch_piece<BITS>(p, share_lo + tid, pc);
+        if (ptid >= 0 && share_lo + ptid < share_hi) fetch_piece<BITS, G>(p, share_lo + ptid, pc);
     }
 
     // ---- stage 1: wave = (row block rb2, group g), two lanes per (row, group) ----
@@ -157,15 +166,15 @@ otf_rows_kernel(const RowsParams p)
         float th[L - 1], cbv[L];
         load_quant_params<BITS>(p.thr, p.cb_a, th, cbv);
         const BucketScale bq = pick_bucket_scale<BITS>(th);
-        // The lookup tables are built by one wave per SIMD while the tiles are on their way (every participating
-        // thread pays ~250 instructions of set-up whether or not it owns a table entry, and stage 1 is
-        // instruction-bound: all 2 G waves building cost 17 % of the phase).
-        constexpr int kBuilders = W < 4 ? W : 4;
-        if (wave < kBuilders) build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid, 64 * kBuilders);
+        // The lookup tables are built by three waves while the tiles are on their way (every participating thread
+        // pays ~250 instructions of set-up whether or not it owns a table entry: all 2 G waves building cost 17 % of
+        // the phase).
+        if (wave >= kBuilder0 && wave < kBuilder0 + kBuilders)
+            build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid - 64 * kBuilder0, 64 * kBuilders);
         if (p.counter) {
-            if (share_lo + tid < share_hi) finish_piece<BITS>(p, share_lo + tid, pc);
-            for (int64_t idx = share_lo + nthreads + tid; idx < share_hi; idx += nthreads) {     // (large N*K only)
-                fetch_piece<BITS>(p, idx, pc);
+            if (ptid >= 0 && share_lo + ptid < share_hi) finish_piece<BITS>(p, share_lo + ptid, pc);
+            for (int64_t idx = share_lo + kPieceThreads + ptid; ptid >= 0 && idx < share_hi; idx += kPieceThreads) {     // (large N*K only)
+                fetch_piece<BITS, G>(p, idx, pc);
                 finish_piece<BITS>(p, idx, pc);
             }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the written-through pieces have reached memory
@@ -277,7 +286,7 @@ otf_rows_kernel(const RowsParams p)
     if (p.counter) {
         if (!s_flag) {                            // workgroup-uniform
             for (int64_t idx = tid; idx < pieces; idx += nthreads) {
-                fetch_piece<BITS>(p, idx, pc);
+                fetch_piece<BITS, G>(p, idx, pc);
                 finish_piece<BITS>(p, idx, pc);
             }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
