@@ -104,3 +104,29 @@ def test_full_scope_model_forward(cuda):
     cos16 = torch.nn.functional.cosine_similarity(got16.flatten(), ref.flatten(), dim=0)
     assert bool(torch.isfinite(got16).all()) and float(cos16) >= 0.9, float(cos16)
     print(f"logit cosine vs fp32 fake quantization: fp32 chain {float(cos):.4f}, half chain {float(cos16):.4f}")
+
+
+def test_packed_checkpoint_round_trip_on_gpu(cuda, tmp_path):
+    """Training checkpoint -> converter command line (patch convolution packed too) -> packed file -> plain skeleton
+    via load_packed_state_dict -> GPU forward: the logits equal those of the model converted in memory, bit for bit
+    (same buffers, same kernels)."""
+    import yaml
+    from arcq_vit_amd import convert
+    from arcq_vit_amd.vit import VisionTransformer
+    kw = dict(num_classes=10, quantize_patch_embed=True, head_quant="w8a8")
+    src = build_fakequant_vit("deit_tiny", 4, **kw)
+    ckpt = tmp_path / "best.pt"
+    torch.save({"model": {"module." + k: v for k, v in src.state_dict().items()}, "epoch": 1}, ckpt)
+    cfg = tmp_path / "cfg.yaml"
+    cfg.write_text(yaml.safe_dump({"model_name": "deit_tiny_patch16_224", "num_classes": 10, "w_bits": 4, "a_bits": 4,
+                                   "head_quant": "w8a8"}))
+    convert.main(["--config", str(cfg), "--checkpoint", str(ckpt), "--output-dir", str(tmp_path), "--pack-patch-embed"])
+    state = torch.load(tmp_path / "deit_tiny_w4a4_packed_packed.pt", map_location="cpu", weights_only=True)
+    d = synth.MODEL_DIMS["deit_tiny"]
+    loaded = A.load_packed_state_dict(VisionTransformer(d["dim"], d["depth"], d["heads"], d["mlp"], 10), state).to(cuda).eval()
+    direct = build_packed_vit("deit_tiny", 4, device="cuda", half_chain=False, **kw)
+    assert isinstance(loaded.patch_embed.proj, A.ARCQPackedPatchConv)
+    assert sum(isinstance(m, A.ARCQPackedLinearOnTheFly) for m in loaded.modules()) == 48
+    x = synth.make_images(4, 9).to(cuda)
+    with torch.no_grad():
+        assert torch.equal(loaded(x), direct(x))
