@@ -105,11 +105,13 @@ linear_index_u8_kernel(const uint8_t *__restrict__ xcodes, const float *__restri
 // the order in which one output's terms are added; that is the reference's, per output: serial over j in fp64 for
 // the packed format; for the byte format the 32 strided partial sums folded by the shuffle-down tree, which is
 // evaluated here depth first (the same additions, associated the same way) so that only five values per output are live.
-constexpr int kTileRows = 16, kTileOuts = 64, kOutsPerThread = 4;
+constexpr int kTileRows = 16, kTileOuts = 64;
 
 // BITS = 2 / 3 / 4: packed codes, fp64 accumulation.  BITS = 0: byte codes, fp32, tree order.
-template <int BITS>
-__global__ void __launch_bounds__(256)
+// OPT = outputs per thread: four (256 threads per workgroup) for launches that fill the chip; one (1024 threads) for
+// small ones, whose duration is the length of one thread's chain of additions (197 x 768 x 192: 156 tiles).
+template <int BITS, int OPT>
+__global__ void __launch_bounds__(1024 / OPT)
 linear_index_tile_kernel(const uint8_t *__restrict__ xq, const float *__restrict__ xc, const float *__restrict__ xs,
                          const float *__restrict__ xcs, const uint8_t *__restrict__ wq,
                          const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
@@ -120,10 +122,13 @@ linear_index_tile_kernel(const uint8_t *__restrict__ xq, const float *__restrict
     extern __shared__ float s_table[];
     __shared__ __attribute__((aligned(16))) uint8_t s_x[kTileRows][64];
     __shared__ __attribute__((aligned(16))) uint8_t s_w[64][kTileOuts];          // [j][output]
+    constexpr int kOutsPerThread = OPT;
+    constexpr int kThreads = 1024 / OPT;
+    constexpr int kThreadsPerRow = kTileOuts / OPT;
     const int tid = threadIdx.x;
-    for (int i = tid; i < levels * levels; i += 256) s_table[i] = table[i];
-    const int tr = tid >> 4;                       // row of the tile
-    const int to = (tid & 15) * kOutsPerThread;    // first of this thread's outputs in the tile
+    for (int i = tid; i < levels * levels; i += kThreads) s_table[i] = table[i];
+    const int tr = tid / kThreadsPerRow;                       // row of the tile
+    const int to = (tid % kThreadsPerRow) * kOutsPerThread;    // first of this thread's outputs in the tile
     const int64_t r = static_cast<int64_t>(blockIdx.y) * kTileRows + tr;
     const int64_t o0 = static_cast<int64_t>(blockIdx.x) * kTileOuts + to;
     const int64_t groups = in_f / 64;
@@ -156,9 +161,7 @@ linear_index_tile_kernel(const uint8_t *__restrict__ xq, const float *__restrict
                 }
                 *reinterpret_cast<uint2 *>(&s_x[row][ch * 8]) = make_uint2(lo, hi);
             }
-#pragma unroll
-            for (int rep = 0; rep < 2; ++rep) {                      // w: 64 outputs x 8 chunks, two per thread
-                const int job = rep * 256 + tid;
+            for (int job = tid; job < kTileOuts * 8; job += kThreads) {      // w: 64 outputs x 8 chunks of eight codes
                 const int out = job >> 3, ch = job & 7;
                 const int64_t oo = static_cast<int64_t>(blockIdx.x) * kTileOuts + out;
                 const uint32_t w8 = load_codes8<BITS>(wq + (oo < out_f ? oo : out_f - 1) * pcols + g * kRowBytes + ch * BITS);
@@ -166,13 +169,13 @@ linear_index_tile_kernel(const uint8_t *__restrict__ xq, const float *__restrict
                 for (int q = 0; q < 8; ++q) s_w[ch * 8 + q][out] = static_cast<uint8_t>((w8 >> (BITS * q)) & ((1u << BITS) - 1u));
             }
         } else {
-            {                                                        // x: 16 rows x 64 bytes, one dword per thread
+            if (tid < 256) {                                         // x: 16 rows x 64 bytes, one dword per thread
                 const int row = tid >> 4, c4 = (tid & 15) * 4;
                 const int64_t rr = static_cast<int64_t>(blockIdx.y) * kTileRows + row;
                 *reinterpret_cast<uint32_t *>(&s_x[row][c4]) =
                     *reinterpret_cast<const uint32_t *>(xq + (rr < rows ? rr : rows - 1) * pcols + g * 64 + c4);
             }
-            {                                                        // w: 64 outputs x 64 bytes, sixteen bytes per thread
+            if (tid < 256) {                                         // w: 64 outputs x 64 bytes, sixteen bytes per thread
                 const int out = tid >> 2, c16 = (tid & 3) * 16;
                 const int64_t oo = static_cast<int64_t>(blockIdx.x) * kTileOuts + out;
                 const uint4 v = *reinterpret_cast<const uint4 *>(wq + (oo < out_f ? oo : out_f - 1) * pcols + g * 64 + c16);
@@ -185,9 +188,13 @@ linear_index_tile_kernel(const uint8_t *__restrict__ xq, const float *__restrict
         // one j for this thread's row and its four outputs: the table entries P[x code][w code]
         auto entries = [&](int j, float (&e)[kOutsPerThread]) __attribute__((always_inline)) {
             const int a = static_cast<int>(s_x[tr][j]) * levels;
-            const uint32_t wb = *reinterpret_cast<const uint32_t *>(&s_w[j][to]);
+            if constexpr (OPT == 4) {
+                const uint32_t wb = *reinterpret_cast<const uint32_t *>(&s_w[j][to]);
 #pragma unroll
-            for (int i = 0; i < kOutsPerThread; ++i) e[i] = s_table[a + static_cast<int>((wb >> (8 * i)) & 255u)];
+                for (int i = 0; i < kOutsPerThread; ++i) e[i] = s_table[a + static_cast<int>((wb >> (8 * i)) & 255u)];
+            } else {
+                e[0] = s_table[a + static_cast<int>(s_w[j][to])];
+            }
         };
         acc_t cross[kOutsPerThread];
         if constexpr (BITS != 0) {
@@ -275,6 +282,10 @@ linear_index_tile_kernel(const uint8_t *__restrict__ xq, const float *__restrict
     }
 }
 
+// Launches of at most this many 16 x 64 tiles give every thread one output instead of four.
+constexpr int kSmallTiles = 512;
+static size_t tile_table_bytes(int levels) { return static_cast<size_t>(levels) * levels * sizeof(float); }
+
 static int check_common(const char *fn, int64_t rows, int64_t out_f, int64_t in_f, int gs, int levels)
 {
     if (rows < 0 || out_f < 0 || in_f < 0 || gs <= 0) return fail(ARCQ_ERR_SHAPE, "%s: bad sizes", fn);
@@ -312,16 +323,17 @@ ARCQ_API int arcq_linear_forward_packed(const uint8_t *packed_x, const float *x_
         aligned(packed_w, 4)) {
         dim3 tgrid(static_cast<unsigned>((out_features + kTileOuts - 1) / kTileOuts),
                    static_cast<unsigned>((rows + kTileRows - 1) / kTileRows));
-#define ARCQ_LAUNCH_TILE(B)                                                                                              \
+        const bool small = static_cast<int64_t>(tgrid.x) * tgrid.y <= kSmallTiles;
+#define ARCQ_LAUNCH_TILE(B, O)                                                                                           \
     do {                                                                                                                  \
-        allow_dynamic_lds<linear_index_tile_kernel<B>>(64 * 1024);                                                        \
-        hipLaunchKernelGGL((linear_index_tile_kernel<B>), tgrid, dim3(256), levels * levels * sizeof(float),              \
+        allow_dynamic_lds<linear_index_tile_kernel<B, O>>(64 * 1024);                                                     \
+        hipLaunchKernelGGL((linear_index_tile_kernel<B, O>), tgrid, dim3(1024 / O), tile_table_bytes(levels),              \
                            static_cast<hipStream_t>(stream), packed_x, x_center, x_scale, x_code_sum, packed_w, w_center, \
                            w_scale, w_code_sum, product_table, bias, y, rows, out_features, in_features, levels);         \
     } while (0)
-        if (bits == 4) ARCQ_LAUNCH_TILE(4);
-        else if (bits == 3) ARCQ_LAUNCH_TILE(3);
-        else ARCQ_LAUNCH_TILE(2);
+        if (bits == 4) { if (small) ARCQ_LAUNCH_TILE(4, 1); else ARCQ_LAUNCH_TILE(4, 4); }
+        else if (bits == 3) { if (small) ARCQ_LAUNCH_TILE(3, 1); else ARCQ_LAUNCH_TILE(3, 4); }
+        else { if (small) ARCQ_LAUNCH_TILE(2, 1); else ARCQ_LAUNCH_TILE(2, 4); }
 #undef ARCQ_LAUNCH_TILE
         return launch_status("arcq_linear_forward_packed");
     }
@@ -354,10 +366,17 @@ ARCQ_API int arcq_linear_forward_u8(const uint8_t *x_codes, const float *x_cente
         aligned(w_codes, 16)) {
         dim3 tgrid(static_cast<unsigned>((out_features + kTileOuts - 1) / kTileOuts),
                    static_cast<unsigned>((rows + kTileRows - 1) / kTileRows));
-        allow_dynamic_lds<linear_index_tile_kernel<0>>(64 * 1024);
-        hipLaunchKernelGGL((linear_index_tile_kernel<0>), tgrid, dim3(256), levels * levels * sizeof(float),
-                           static_cast<hipStream_t>(stream), x_codes, x_center, x_scale, x_code_sum, w_codes, w_center,
-                           w_scale, w_code_sum, product_table, bias, y, rows, out_features, in_features, levels);
+        if (static_cast<int64_t>(tgrid.x) * tgrid.y <= kSmallTiles) {
+            allow_dynamic_lds<linear_index_tile_kernel<0, 1>>(64 * 1024);
+            hipLaunchKernelGGL((linear_index_tile_kernel<0, 1>), tgrid, dim3(1024), tile_table_bytes(levels),
+                               static_cast<hipStream_t>(stream), x_codes, x_center, x_scale, x_code_sum, w_codes, w_center,
+                               w_scale, w_code_sum, product_table, bias, y, rows, out_features, in_features, levels);
+        } else {
+            allow_dynamic_lds<linear_index_tile_kernel<0, 4>>(64 * 1024);
+            hipLaunchKernelGGL((linear_index_tile_kernel<0, 4>), tgrid, dim3(256), tile_table_bytes(levels),
+                               static_cast<hipStream_t>(stream), x_codes, x_center, x_scale, x_code_sum, w_codes, w_center,
+                               w_scale, w_code_sum, product_table, bias, y, rows, out_features, in_features, levels);
+        }
         return launch_status("arcq_linear_forward_u8");
     }
     dim3 grid(static_cast<unsigned>((out_features + kIdxTile - 1) / kIdxTile),
