@@ -70,24 +70,24 @@ def unwrap_checkpoint(checkpoint) -> Dict[str, torch.Tensor]:
 
 def restore_dynamic_state_tensors(model: nn.Module, state: Dict[str, torch.Tensor]) -> int:
     """Put stored tensors in place of buffers (any shape) and of parameters named ``step``, which
-    ``load_state_dict`` cannot do when the registered shape differs
-    (scripts/benchmark_arcq_packed_inference.py:82-98)."""
-    modules = dict(model.named_modules())
-    restored = 0
-    for key, value in state.items():
-        if "." not in key or not isinstance(value, torch.Tensor):
+    ``load_state_dict`` cannot do when the registered shape differs (what
+    scripts/benchmark_arcq_packed_inference.py:82-98 does after its ordinary load).  Returns how many were placed."""
+    owners = dict(model.named_modules())
+    placed = 0
+    for key, tensor in state.items():
+        owner_name, dot, leaf = key.rpartition(".")
+        owner = owners.get(owner_name) if dot else None
+        if owner is None or not isinstance(tensor, torch.Tensor):
             continue
-        module_name, attr = key.rsplit(".", 1)
-        module = modules.get(module_name)
-        if module is None:
+        fresh = tensor.detach().clone()
+        if leaf in owner._buffers:
+            owner._buffers[leaf] = fresh
+        elif leaf == "step" and leaf in owner._parameters:
+            owner._parameters[leaf] = nn.Parameter(fresh)
+        else:
             continue
-        if attr in module._buffers:
-            module._buffers[attr] = value.detach().clone()
-            restored += 1
-        elif attr in module._parameters and attr == "step":
-            module._parameters[attr] = nn.Parameter(value.detach().clone())
-            restored += 1
-    return restored
+        placed += 1
+    return placed
 
 
 def load_training_checkpoint(model: nn.Module, source: Union[str, Path, Dict]) -> LoadReport:
@@ -107,26 +107,29 @@ def load_training_checkpoint(model: nn.Module, source: Union[str, Path, Dict]) -
     return LoadReport(len(missing), len(unexpected), skipped_shape, restored)
 
 
+def _filled(value) -> bool:
+    return isinstance(value, torch.Tensor) and value.numel() > 0
+
+
 def mark_arcq_codebooks_ready(model: nn.Module) -> Tuple[int, int]:
     """Flag every quantizer that holds a non-empty codebook and thresholds as compiled and stop recompilation
     (scripts/benchmark_arcq_packed_inference.py:116-140).  Returns ``(ready, missing)``."""
-    ready = missing = 0
+    counts = {True: 0, False: 0}
     for module in model.modules():
         if hasattr(module, "_pc_cb") and hasattr(module, "_pc_thresholds"):
-            cb, thr = module._pc_cb, module._pc_thresholds
-            if isinstance(cb, torch.Tensor) and cb.numel() > 0 and isinstance(thr, torch.Tensor) and thr.numel() > 0:
+            ok = _filled(module._pc_cb) and _filled(module._pc_thresholds)
+            if ok:
                 module._pc_ready = True
-                ready += 1
-            else:
-                missing += 1
+            counts[ok] += 1
+        # quantizers of the training code base recompile at scheduled steps: none are left
         if hasattr(module, "phase_compile"):
             module.phase_compile = True
         if hasattr(module, "compile_steps"):
             try:
                 module.compile_steps = set()
-            except Exception:
+            except (AttributeError, TypeError):
                 pass
-    return ready, missing
+    return counts[True], counts[False]
 
 
 def model_key_of(config: Dict, fallback: Optional[str] = None) -> str:
