@@ -9,10 +9,14 @@ namespace arcq {
 
 constexpr int kMaxBuckets = 512;   // table entries 0 .. nb (nb <= 512); entry nb is reached by t == 8 only
 
-// Bucket geometry: t in [-8, 8] maps to floor(t * scale + 8 * scale); nb = 16 * scale buckets can hold a threshold.
-// The scale is the smallest of 4, 8, 16, 32 buckets per unit of t that separates every pair of thresholds
-// (scale * smallest gap > 1), so the usual codebooks need a 65- or 129-entry table instead of 513.
-struct BucketScale { float scale, offset; int nb; };
+// Bucket geometry: t in [-8, 8] maps to floor(f), f = t * scale + 8 * scale rounded to a multiple of 1/8; nb = 16 * scale
+// buckets can hold a threshold.  The scale is the smallest of 4, 8, 16, 32 buckets per unit of t that separates every
+// pair of thresholds (scale * smallest gap > 1), so the usual codebooks need a 65- or 129-entry table instead of 513.
+// f is formed as 2^20 + f in one fma: in that binade a float's unit in the last place is 1/8, so the low mantissa bits
+// of the result ARE 8 * f -- the byte offset of an 8-byte table entry once the three fraction bits are masked off.
+// The map t -> bucket is monotone (fma and the mask are), which is all the code search needs.
+constexpr float kBucketBias = 1048576.0f;      // 2^20
+struct BucketScale { float scale, offset; int nb; };      // offset = 8 * scale + 2^20 (exact)
 
 template <int BITS>
 __device__ __forceinline__ BucketScale pick_bucket_scale(const float (&th)[(1 << BITS) - 1])
@@ -27,7 +31,7 @@ __device__ __forceinline__ BucketScale pick_bucket_scale(const float (&th)[(1 <<
     if (gap * 4.0f > 1.0f) scale = 4.0f;
     BucketScale q;
     q.scale = scale;
-    q.offset = 8.0f * scale;
+    q.offset = 8.0f * scale + kBucketBias;
     q.nb = static_cast<int>(16.0f * scale);
     return q;
 }
@@ -36,19 +40,20 @@ __device__ __forceinline__ BucketScale pick_bucket_scale(const float (&th)[(1 <<
 __device__ __forceinline__ int bucket_of_threshold(float t, const BucketScale &q)
 {
     const float f = __fmaf_rn(t, q.scale, q.offset);
-    if (!(f >= 0.0f)) return -1;                // below the table, or NaN
-    if (f >= static_cast<float>(q.nb)) return q.nb;
-    return __float2int_rz(f);
+    if (!(f >= kBucketBias)) return -1;         // below the table, or NaN
+    if (f >= kBucketBias + static_cast<float>(q.nb)) return q.nb;
+    return __float2int_rz(f - kBucketBias);     // exact difference
 }
 
-// Bucket of t = d/s on the fast path: |t| <= 8, so f lies in [0, nb] and one saturating conversion
-// (negative zero and tiny negatives give 0) is the whole index computation.
-__device__ __forceinline__ uint32_t bucket_of(float t, const BucketScale &q)
+// Byte offset into the table of the bucket of t = d/s on the fast path: |t| <= 8, so f lies in [0, nb] <= 512 and the
+// offset is bits 3..12 of the biased sum.
+__device__ __forceinline__ uint32_t bucket_offset_of(float t, const BucketScale &q)
 {
-    return static_cast<uint32_t>(__fmaf_rn(t, q.scale, q.offset));
+    return __float_as_uint(__fmaf_rn(t, q.scale, q.offset)) & 0x1ff8u;
 }
 
 struct Bucket { float thr; int base; };     // the threshold inside the bucket (+inf if none); thresholds in lower buckets
+static_assert(sizeof(Bucket) == 8, "bucket_offset_of assumes 8-byte table entries");
 
 template <int BITS>
 __device__ __forceinline__ void load_quant_params(const float *__restrict__ thr, const float *__restrict__ cb,
@@ -142,7 +147,7 @@ __device__ __forceinline__ void group_codes64(float (&xv)[64], float mu, float v
     if (fast) {
         const float y = 1.0f / s;
         const float ns = -s;
-        const uint32_t lane4 = static_cast<uint32_t>(lane) * 4u;
+        const char *lut_lane = reinterpret_cast<const char *>(lut) + lane * 4;      // + 256 c: one shift-add per lookup
 #pragma unroll
         for (int j = 0; j < 64; ++j) {
             const float d = xv[j];
@@ -151,10 +156,10 @@ __device__ __forceinline__ void group_codes64(float (&xv)[64], float mu, float v
             q = __fmaf_rn(e, y, q);
             e = __fmaf_rn(ns, q, d);
             q = __fmaf_rn(e, y, q);        // == RN(d / s)
-            const Bucket bk = table[bucket_of(q, bq)];
+            const Bucket bk = *reinterpret_cast<const Bucket *>(reinterpret_cast<const char *>(table) + bucket_offset_of(q, bq));
             const uint32_t c = static_cast<uint32_t>(bk.base) + ((q > bk.thr) ? 1u : 0u);
             if constexpr (CODES) code[j] = c;
-            const float v = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(lut) + ((c << 8) | lane4));
+            const float v = *reinterpret_cast<const float *>(lut_lane + (c << 8));
             xv[j] = v;
             sum_codes += v;
         }
@@ -235,7 +240,7 @@ __device__ __forceinline__ void group_codes32x2(float (&xv)[32], float mu, float
     if (fast) {
         const float y = 1.0f / s;
         const float ns = -s;
-        const uint32_t lane4 = static_cast<uint32_t>(lane) * 4u;
+        const char *lut_lane = reinterpret_cast<const char *>(lut) + lane * 4;      // + 256 c: one shift-add per lookup
 #pragma unroll
         for (int j = 0; j < 32; ++j) {
             const float d = xv[j];
@@ -244,9 +249,9 @@ __device__ __forceinline__ void group_codes32x2(float (&xv)[32], float mu, float
             q = __fmaf_rn(e, y, q);
             e = __fmaf_rn(ns, q, d);
             q = __fmaf_rn(e, y, q);        // == RN(d / s)
-            const Bucket bk = table[bucket_of(q, bq)];
+            const Bucket bk = *reinterpret_cast<const Bucket *>(reinterpret_cast<const char *>(table) + bucket_offset_of(q, bq));
             const uint32_t c = static_cast<uint32_t>(bk.base) + ((q > bk.thr) ? 1u : 0u);
-            xv[j] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(lut) + ((c << 8) | lane4));
+            xv[j] = *reinterpret_cast<const float *>(lut_lane + (c << 8));
         }
     } else {
 #pragma unroll
