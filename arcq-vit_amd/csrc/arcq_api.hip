@@ -115,7 +115,7 @@ static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds
                             w_code_sum, bias, w_hat_ws, y, y_dtype == ARCQ_F16, nullptr, false, static_cast<int>(M),
                             static_cast<int>(N), static_cast<int>(K), bits, 1.0e-6f};
         const int rc = arcq::launch_otf_rows(a, static_cast<hipStream_t>(stream));
-        if (rc != arcq::kNoCounter) return rc;
+        if (rc != arcq::kNotLaunched) return rc;
     }
     // Scratch-only workspaces and 512 rows or more: x_hat in the block layout, eight-wave weight-stationary GEMM
     // (bit-identical results; invalid arguments fall through to the entry points below, which report them).
@@ -185,7 +185,8 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
     if (a->x_hat_ws == a->x) return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: x_hat_ws must not alias x");
     if (a->residual && !arcq::aligned(a->residual, 16))
         return arcq::fail(ARCQ_ERR_ALIGN, "arcq_linear_otf_ex: residual must be 16-byte aligned");
-    if (a->w_hat_ws && a->x_dtype == ARCQ_F16 && arcq::otf_rows_pays(a->M, a->N, a->K) && a->x && a->a_thresholds &&
+    if (a->w_hat_ws && a->x_dtype == ARCQ_F16 &&
+        arcq::otf_rows_pays(a->M, a->N, a->K, a->producer == ARCQ_PRODUCER_LAYERNORM) && a->x && a->a_thresholds &&
         a->a_codebook && a->packed_w && a->w_codebook && a->w_center && a->w_scale && a->w_code_sum && a->y &&
         (a->y_dtype == ARCQ_F16 || a->y_dtype == ARCQ_F32) && arcq::aligned(a->x, 16) && arcq::aligned(a->y, 16) &&
         arcq::aligned(a->w_hat_ws, 128) && arcq::aligned(a->packed_w, 4) &&
@@ -197,7 +198,7 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
                             a->w_hat_ws, a->y, a->y_dtype == ARCQ_F16, a->residual, a->activation == ARCQ_ACT_GELU,
                             static_cast<int>(a->M), static_cast<int>(a->N), static_cast<int>(a->K), a->bits, 1.0e-6f};
         const int rc = arcq::launch_otf_rows(r, static_cast<hipStream_t>(stream));
-        if (rc != arcq::kNoCounter) return rc;
+        if (rc != arcq::kNotLaunched) return rc;
     }
     const bool carry = a->w_hat_ws && arcq::blocked_uses_workspace(a->N, a->K) && a->packed_w && a->w_codebook && a->w_center &&
                        a->w_scale && a->w_code_sum && arcq::aligned(a->w_hat_ws, 16) && arcq::aligned(a->packed_w, 16);

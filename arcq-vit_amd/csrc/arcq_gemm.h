@@ -84,12 +84,15 @@ struct OtfRowsArgs {
     int M, N, K, bits;
     float eps;
 };
-// Shapes the kernel can run (M >= 512, K a multiple of 64 up to 512, N a multiple of 32, everything within LDS).
-bool otf_rows_supported(int64_t M, int64_t N, int64_t K);
+// Shapes the kernels can run: M >= 512 and few enough rows that one workgroup per 64 of them is resident at once
+// (M <= 64 x compute units, twice that for K = 192), N a multiple of 32 and either K = 192 / 256 / 384 with everything
+// within LDS (otf_rows_kernel) or K = 768 / 1536 with N <= 384 and no LayerNorm in front (otf_rows_phased_kernel).
+bool otf_rows_supported(int64_t M, int64_t N, int64_t K, bool layernorm = false);
 // Whether the whole-layer entry points take it for this shape (fp16 input, both workspaces given).
-bool otf_rows_pays(int64_t M, int64_t N, int64_t K);
-// Returns kNoCounter (and launches nothing, records no error) when the stream cannot be given a counter.
-constexpr int kNoCounter = -1000;
+bool otf_rows_pays(int64_t M, int64_t N, int64_t K, bool layernorm = false);
+// Returns kNotLaunched (having launched nothing and recorded no error) when the stream cannot be given a counter or
+// the device would not hold all the launch's workgroups at once: the caller takes the two-launch path.
+constexpr int kNotLaunched = -1000;
 int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream);
 
 }  // namespace arcq

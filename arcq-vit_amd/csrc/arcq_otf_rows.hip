@@ -416,6 +416,259 @@ otf_rows_kernel(const RowsParams p)
     }
 }
 
+// The same layer for rows of PHASES * 64 G values (K = 768, 1536: fc2 of the small models) and at most 32 * 2 G
+// output columns: the row is taken in PHASES slices of G groups.  Two x_hat slice buffers alternate in LDS; while the
+// MFMAs of slice p run from one, stage 1 of slice p + 1 fills the other (stage 1 is bound by vector-ALU issue, the
+// product by the stream of w_hat through L1 -- different units, so waves of one SIMD that are in different halves
+// of the phase overlap: every second wave quad multiplies first and quantizes second).  Every wave owns one
+// 32-column block for the whole launch, so the accumulators stay in registers across the slices; k order per output
+// is ascending as everywhere else.  A lane pair reads its 64 inputs of the next slice straight from global memory
+// (two whole 64-byte halves of a 128-byte line) as soon as the registers of the current one are converted.
+template <int BITS, typename TOUT, int G, int PHASES>
+__global__ void __launch_bounds__(128 * G)
+otf_rows_phased_kernel(const RowsParams p)
+{
+    constexpr int L = 1 << BITS;
+    constexpr int W = 2 * G, GT = G * PHASES, K = 64 * GT, KS = 64 * G;
+    static_assert(G % 2 == 0, "the two-slot fragment ring must close on a slice boundary");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ float lut[L * 64];
+    __shared__ Bucket table[kMaxBuckets + 1];
+    __shared__ int slow_slots[W];
+    __shared__ int s_flag;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int nthreads = 64 * W;
+    constexpr int pitch = KS * 2 + 16;                           // bytes per x_hat row of a slice
+    constexpr int kBuf = 64 * pitch;
+    unsigned char *xs = smem;                                    // [2][64][pitch]
+    float *s_bias = reinterpret_cast<float *>(smem + 2 * kBuf);  // [32 W]
+    unsigned char *wave_lds = smem + wave * kWaveLds;            // output staging: reuses the slice buffers at the end
+    static_assert(W * kWaveLds <= 2 * kBuf, "output staging must fit into the slice buffers");
+    const int64_t pieces = static_cast<int64_t>(p.N) * (K / 8);
+    const int64_t row_base = static_cast<int64_t>(blockIdx.x) * 64;
+
+    // stage-1 role: wave = (row block rb2, group g of the slice); lane pair = one row
+    const int rb2 = wave / G, g = wave - rb2 * G;
+    const int row = lane >> 1, half = lane & 1;
+    uint4 raw[4];
+    auto load_slice = [&](int ph) {                              // rows past the tensor's end read as zeros
+        const int64_t my_row = row_base + rb2 * 32 + row;
+        const __half *src = p.x + my_row * K + ph * KS + g * 64 + half * 32;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            raw[i] = my_row < p.M ? *reinterpret_cast<const uint4 *>(src + i * 8) : make_uint4(0, 0, 0, 0);
+    };
+    load_slice(0);
+
+    // ---- this workgroup's share of w_hat and the lookup tables, as in otf_rows_kernel ----
+    constexpr int kBuilders = 3, kBuilder0 = 1;
+    constexpr int kPieceThreads = 64 * (W - 3);
+    const int ptid = wave == 0 ? lane : (wave >= 4 ? (wave - 3) * 64 + lane : -1);
+    int64_t share_lo = 0, share_hi = 0;
+    Piece pc{};
+    unsigned long long target = 0;
+    if (p.counter) {
+        int64_t per = (pieces + gridDim.x - 1) / gridDim.x;
+        per = (per + 7) & ~int64_t(7);
+        share_lo = blockIdx.x * per;
+        share_hi = share_lo + per < pieces ? share_lo + per : pieces;
+        if (ptid >= 0 && share_lo + ptid < share_hi) fetch_piece<BITS, GT>(p, share_lo + ptid, pc);
+    }
+    for (int i = tid; i < 32 * W; i += nthreads) s_bias[i] = (p.bias && i < p.N) ? p.bias[i] : 0.0f;
+    float th[L - 1], cbv[L];
+    load_quant_params<BITS>(p.thr, p.cb_a, th, cbv);
+    const BucketScale bq = pick_bucket_scale<BITS>(th);
+    if (wave >= kBuilder0 && wave < kBuilder0 + kBuilders)
+        build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid - 64 * kBuilder0, 64 * kBuilders);
+    if (p.counter) {
+        if (ptid >= 0 && share_lo + ptid < share_hi) finish_piece<BITS>(p, share_lo + ptid, pc);
+        for (int64_t idx = share_lo + kPieceThreads + ptid; ptid >= 0 && idx < share_hi; idx += kPieceThreads) {
+            fetch_piece<BITS, GT>(p, idx, pc);
+            finish_piece<BITS>(p, idx, pc);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // the written-through pieces have reached memory
+    }
+    __syncthreads();                                             // tables complete, and the workgroup's share of w_hat
+    if (p.counter && tid == 0) {
+        const unsigned long long inc = blockIdx.x == 0 ? kEpoch - (gridDim.x - 1) : 1ull;
+        const unsigned long long old = __hip_atomic_fetch_add(p.counter, inc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        target = (old & ~(kEpoch - 1)) + kEpoch;
+    }
+    bool table_ok = true;
+    for (int w = 0; w < kBuilders; ++w) table_ok = table_ok && (slow_slots[w] == 0);
+
+    // ---- product role: wave = 32-column block `wave` (idle in the product if the layer has fewer blocks) ----
+    const int lr = lane & 31, lh = lane >> 5;
+    const int ncb = p.N / 32;
+    const bool has_block = wave < ncb;
+    const char *w_col = reinterpret_cast<const char *>(p.w_blk) + lh * 2048 + lr * 16 +
+                        static_cast<int64_t>(has_block ? wave : 0) * (static_cast<int64_t>(K) * 64);
+    int ld_g = 0;
+    auto load_unit = [&](u32x4_t (&r)[4]) {      // the four fragments of the next group; past the last it re-reads the last
+        const char *q = w_col + (ld_g < GT ? ld_g : GT - 1) * 4096;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) r[kk] = *reinterpret_cast<const u32x4_t *>(q + kk * 512);
+        ++ld_g;
+    };
+    u32x4_t ring[2][4];
+    float16_t acc[2];
+
+    auto stage1 = [&](int ph) {                  // slice ph: registers -> xs[ph & 1]; then requests slice ph + 1
+        float xv[32];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w4[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                xv[8 * i + 2 * e] = __half2float(__ushort_as_half(static_cast<unsigned short>(w4[e] & 0xffffu)));
+                xv[8 * i + 2 * e + 1] = __half2float(__ushort_as_half(static_cast<unsigned short>(w4[e] >> 16)));
+            }
+        }
+        if (ph + 1 < PHASES) load_slice(ph + 1);
+        float mu, var, s, sum_codes;
+        group_stats32x2(xv, p.eps, mu, var, s);
+        group_codes32x2<BITS>(xv, mu, var, s, th, bq, table, lut, table_ok, lane, sum_codes);
+        const float code_mean = sum_codes * 0.015625f;
+        unsigned char *dst = xs + (ph & 1) * kBuf + (rb2 * 32 + row) * pitch + g * 128 + half * 64;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            u32x4_t o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int j = 8 * q4 + 2 * e;
+                const __half2 h = __floats2half2_rn(fma_f32(s, xv[j] - code_mean, mu), fma_f32(s, xv[j + 1] - code_mean, mu));
+                o[e] = *reinterpret_cast<const uint32_t *>(&h);
+            }
+            *reinterpret_cast<u32x4_t *>(dst + q4 * 16) = o;
+        }
+    };
+
+    auto product = [&](int ph) {                 // acc += x_hat slice ph * w_hat slice ph^T
+        const unsigned char *xb = xs + (ph & 1) * kBuf + lr * pitch + lh * 64;
+        half8_t xf[2][2];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) xf[0][rb] = *reinterpret_cast<const half8_t *>(xb + rb * 32 * pitch);
+#pragma unroll
+        for (int gl = 0; gl < G; ++gl) {
+            const u32x4_t (&cur_set)[4] = ring[gl % 2];
+            u32x4_t (&load_set)[4] = ring[(gl + 1) % 2];
+            const unsigned char *xsrc = xb + gl * 128;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const int t = kk + 1;              // the k-step whose x_hat fragments are read now; 4: first of the next group
+                const int off = t < 4 ? t * 16 : 128;                  // (past the slice on its last group: unused)
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb)
+                    xf[t % 2][rb] = *reinterpret_cast<const half8_t *>(xsrc + rb * 32 * pitch + off);
+                if (kk == 1) load_unit(load_set);
+                half8_t wf;
+                __builtin_memcpy(&wf, &cur_set[kk], 16);
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb)
+                    acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf, xf[kk % 2][rb], acc[rb], 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // 1 MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 // 1 LDS read
+                    if (kk == 1) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);    // 2 global loads
+                }
+            }
+        }
+    };
+
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[rb][v] = 0.0f;
+
+    // ---- the phases: iteration ph multiplies slice ph and quantizes slice ph + 1; iteration -1 only quantizes ----
+    const bool multiply_first = ((wave >> 2) & 1) != 0;
+    for (int ph = -1; ph < PHASES; ++ph) {
+        if (ph >= 0 && has_block && multiply_first) product(ph);
+        if (ph + 1 < PHASES) stage1(ph + 1);
+        if (ph >= 0 && has_block && !multiply_first) product(ph);
+        if (ph == -1) {
+            // ---- every share of w_hat written? ----
+            if (p.counter && tid == 0) {
+                int ok = 1;
+                const long long t0 = wall_clock64();
+                while (__hip_atomic_load(p.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+                    if (wall_clock64() - t0 > kSpinTicks) {
+                        ok = 0;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(4);
+                }
+                s_flag = ok;
+            }
+            if (p.counter && wave == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        }
+        __syncthreads();                         // slice ph + 1 of x_hat is complete, slice ph has been consumed
+        if (ph == -1) {
+            if (p.counter && !s_flag) {          // workgroup-uniform: the others are not resident; rebuild everything
+                for (int64_t idx = tid; idx < pieces; idx += nthreads) {
+                    fetch_piece<BITS, GT>(p, idx, pc);
+                    finish_piece<BITS>(p, idx, pc);
+                }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+            }
+            if (has_block) load_unit(ring[0]);
+        }
+    }
+
+    // ---- epilogue: as in otf_rows_kernel, one column block per wave ----
+    if (has_block) {
+    constexpr int kStageRow = 32 * static_cast<int>(sizeof(TOUT)) + 16;
+    constexpr int kVec = 16 / static_cast<int>(sizeof(TOUT));
+    constexpr int kPiecesPerRow = 32 / kVec;
+    constexpr int kRowsPerInstr = 64 / kPiecesPerRow;
+    TOUT *y = static_cast<TOUT *>(p.y);
+    const TOUT *residual = static_cast<const TOUT *>(p.residual);
+    const int cbk = wave;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+        float4 bv[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bv[q] = *reinterpret_cast<const float4 *>(s_bias + cbk * 32 + 8 * q + 4 * lh);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int cl = 8 * q + 4 * lh;
+            const float o0 = acc[rb][4 * q] + bv[q].x, o1 = acc[rb][4 * q + 1] + bv[q].y;
+            const float o2 = acc[rb][4 * q + 2] + bv[q].z, o3 = acc[rb][4 * q + 3] + bv[q].w;
+            unsigned char *dst = wave_lds + lr * kStageRow + cl * static_cast<int>(sizeof(TOUT));
+            if constexpr (sizeof(TOUT) == 2) {
+                const __half2 lo = __floats2half2_rn(o0, o1), hi = __floats2half2_rn(o2, o3);
+                u32x2_t pk;
+                pk[0] = *reinterpret_cast<const uint32_t *>(&lo);
+                pk[1] = *reinterpret_cast<const uint32_t *>(&hi);
+                *reinterpret_cast<u32x2_t *>(dst) = pk;
+            } else {
+                u32x4_t pk;
+                pk[0] = __float_as_uint(o0); pk[1] = __float_as_uint(o1);
+                pk[2] = __float_as_uint(o2); pk[3] = __float_as_uint(o3);
+                *reinterpret_cast<u32x4_t *>(dst) = pk;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        const int col = cbk * 32 + (lane % kPiecesPerRow) * kVec;
+#pragma unroll
+        for (int i = 0; i < 32 / kRowsPerInstr; ++i) {
+            const int r = i * kRowsPerInstr + lane / kPiecesPerRow;
+            u32x4_store_t v = *reinterpret_cast<const u32x4_store_t *>(wave_lds + r * kStageRow + (lane % kPiecesPerRow) * 16);
+            const int64_t grow = row_base + rb * 32 + r;
+            if (grow < p.M) {
+                if (residual || p.gelu)
+                    post_ops16<TOUT>(v, residual ? residual + grow * p.N + col : nullptr, p.gelu != 0, kVec);
+                store_streaming16(y + grow * p.N + col, v[0], v[1], v[2], v[3]);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    }
+}
+
 // One counter per stream (calls on one stream run one after another; calls on different streams may overlap and must
 // not count into the same word).  The counters live in device memory that is zero when the code object is loaded.
 constexpr int kCounterSlots = 256;
@@ -449,6 +702,41 @@ unsigned long long *counter_for(hipStream_t stream)
     return g_counters_ptr[dev] + slot;
 }
 
+// Workgroups of `Kernel` (threads, dynamic LDS bytes) the current device holds at once.  A launch must not be larger:
+// every workgroup waits for the weight shares of all the others, and those that are not resident write theirs only
+// after a resident one has given up waiting (correct, but milliseconds late).  Asked once per device, kernel and LDS
+// size; 0 if the runtime cannot tell.
+template <auto Kernel>
+int resident_workgroups(int threads, size_t smem)
+{
+    struct Entry { int dev; size_t smem; int blocks; };
+    static std::mutex mutex;
+    static std::vector<Entry> known;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    std::lock_guard<std::mutex> lock(mutex);
+    for (const Entry &e : known)
+        if (e.dev == dev && e.smem == smem) return e.blocks;
+    int per_cu = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(Kernel), threads, smem) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        per_cu = cus = 0;
+    known.push_back({dev, smem, per_cu * cus});
+    return per_cu * cus;
+}
+
+// Compute units of the current device (256 when there is none to ask: the host-side predicates also run without a GPU).
+int device_cus()
+{
+    static std::atomic<int> known[kMaxDevices];
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    if (const int c = known[dev].load(std::memory_order_relaxed)) return c;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 256;
+    known[dev].store(cus, std::memory_order_relaxed);
+    return cus;
+}
+
 size_t rows_lds_bytes(int N, int K)
 {
     const int G = K / 64;
@@ -456,11 +744,15 @@ size_t rows_lds_bytes(int N, int K)
            static_cast<size_t>(N) * sizeof(float);
 }
 
+// The launchers return false, having launched nothing, when the device would not hold the whole grid at once.
 template <int BITS, typename TOUT, int G, int RING, int AHEAD>
-void launch_rows_g(const RowsParams &p, size_t smem, hipStream_t stream)
+bool launch_rows_g(const RowsParams &p, size_t smem, hipStream_t stream)
 {
     allow_dynamic_lds<otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>>(160 * 1024 - 10 * 1024);
-    hipLaunchKernelGGL((otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>), dim3((p.M + 63) / 64), dim3(128 * G), smem, stream, p);
+    const int tiles = (p.M + 63) / 64;
+    if (resident_workgroups<otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>>(128 * G, smem) < tiles) return false;
+    hipLaunchKernelGGL((otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>), dim3(tiles), dim3(128 * G), smem, stream, p);
+    return true;
 }
 
 // Two fragment groups per wave (the one being multiplied and the next) and x_hat fragments read one k-step ahead:
@@ -468,29 +760,62 @@ void launch_rows_g(const RowsParams &p, size_t smem, hipStream_t stream)
 // shapes -- the stream from L2 is bound by throughput, not latency.  Streaming stores for y and the MFMA / LDS /
 // load interleave pinned with scheduling barriers are worth 7 % and 13 %.
 template <int BITS, typename TOUT>
-void launch_rows(const RowsParams &p, size_t smem, hipStream_t stream)
+bool launch_rows(const RowsParams &p, size_t smem, hipStream_t stream)
 {
-    if (p.G == 3) launch_rows_g<BITS, TOUT, 3, 2, 1>(p, smem, stream);
-    else if (p.G == 4) launch_rows_g<BITS, TOUT, 4, 2, 1>(p, smem, stream);
-    else launch_rows_g<BITS, TOUT, 6, 2, 1>(p, smem, stream);
+    if (p.G == 3) return launch_rows_g<BITS, TOUT, 3, 2, 1>(p, smem, stream);
+    if (p.G == 4) return launch_rows_g<BITS, TOUT, 4, 2, 1>(p, smem, stream);
+    return launch_rows_g<BITS, TOUT, 6, 2, 1>(p, smem, stream);
 }
+
+constexpr int kPhasedG = 6;                  // groups per slice of the phased kernel (twelve waves)
+constexpr size_t kPhasedLds = 2 * 64 * (64 * kPhasedG * 2 + 16) + 32 * 2 * kPhasedG * sizeof(float);
+
+template <int BITS, typename TOUT, int PHASES>
+bool launch_phased_p(const RowsParams &p, hipStream_t stream)
+{
+    allow_dynamic_lds<otf_rows_phased_kernel<BITS, TOUT, kPhasedG, PHASES>>(160 * 1024 - 10 * 1024);
+    const int tiles = (p.M + 63) / 64;
+    if (resident_workgroups<otf_rows_phased_kernel<BITS, TOUT, kPhasedG, PHASES>>(128 * kPhasedG, kPhasedLds) < tiles) return false;
+    hipLaunchKernelGGL((otf_rows_phased_kernel<BITS, TOUT, kPhasedG, PHASES>), dim3(tiles), dim3(128 * kPhasedG), kPhasedLds,
+                       stream, p);
+    return true;
+}
+
+template <int BITS, typename TOUT>
+bool launch_phased(const RowsParams &p, int K, hipStream_t stream)
+{
+    if (K == 768) return launch_phased_p<BITS, TOUT, 2>(p, stream);
+    return launch_phased_p<BITS, TOUT, 4>(p, stream);
+}
+
+bool phased_shape(int64_t N, int64_t K) { return (K == 768 || K == 1536) && N <= 32 * 2 * kPhasedG; }
 
 }  // namespace
 
-bool otf_rows_supported(int64_t M, int64_t N, int64_t K)
+bool otf_rows_supported(int64_t M, int64_t N, int64_t K, bool layernorm)
 {
-    // (at most 2^19 workgroups: what one launch adds to its counter must stay below the counter's epoch)
-    if (M < 512 || M > (int64_t(64) << 19) || (K != 192 && K != 256 && K != 384) || N < 32 || N % 32 != 0 ||
-        N > 16384)
-        return false;
+    if (M < 512 || N < 32 || N % 32 != 0 || N > 16384) return false;
+    // One workgroup per 64 rows, all of them resident at once: K = 192 leaves room for two per compute unit, longer
+    // rows for one (registers: twelve or eight waves of ~165 VGPRs; LDS: 100 KB and more).
+    const int64_t tiles = (M + 63) / 64;
+    if (tiles > static_cast<int64_t>(device_cus()) * (K == 192 ? 2 : 1)) return false;
+    if (phased_shape(N, K)) return !layernorm;
+    if (K != 192 && K != 256 && K != 384) return false;
     return rows_lds_bytes(static_cast<int>(N), static_cast<int>(K)) <= 160 * 1024 - 10 * 1024;
 }
 
-bool otf_rows_pays(int64_t M, int64_t N, int64_t K)
+bool otf_rows_pays(int64_t M, int64_t N, int64_t K, bool layernorm)
 {
-    if (!otf_rows_supported(M, N, K) || tuning().gemm_kernel) return false;
+    if (!otf_rows_supported(M, N, K, layernorm) || tuning().gemm_kernel) return false;
     const char *e = tuning().rows;
     if (e) return e[0] != '0';
+    if (phased_shape(N, K)) {
+        // The phased kernel takes the same time for any number of row tiles up to the device's compute units (stage 1
+        // of a whole row on one CU); the two launches it replaces spread stage 1 over all CUs and win while the grid
+        // is small.  Crossover measured at 128 row tiles for K = 1536 and at 90 for K = 768 (256 CUs).
+        const int64_t tiles = (M + 63) / 64;
+        return tiles * (K == 1536 ? 2 : 3) >= device_cus();
+    }
     return true;
 }
 
@@ -503,20 +828,31 @@ int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream)
     p.pw = a.pw, p.cb_w = a.w_cb, p.wc = a.wc, p.ws = a.ws, p.wcs = a.wcs;
     p.w_blk = static_cast<__half *>(a.w_hat_ws);
     p.counter = counter_for(stream);
-    if (!p.counter) return kNoCounter;       // more streams than counters: the caller takes the two-launch path
+    if (!p.counter) return kNotLaunched;     // more streams than counters: the caller takes the two-launch path
     p.bias = a.bias, p.y = a.y, p.residual = a.residual, p.gelu = a.gelu ? 1 : 0;
     p.M = a.M, p.N = a.N, p.G = a.K / 64;
-    const size_t smem = rows_lds_bytes(a.N, a.K);
-    if (a.y_f16) {
-        if (a.bits == 4) launch_rows<4, __half>(p, smem, stream);
-        else if (a.bits == 3) launch_rows<3, __half>(p, smem, stream);
-        else launch_rows<2, __half>(p, smem, stream);
+    bool launched;
+    if (phased_shape(a.N, a.K)) {
+        if (a.y_f16)
+            launched = a.bits == 4   ? launch_phased<4, __half>(p, a.K, stream)
+                       : a.bits == 3 ? launch_phased<3, __half>(p, a.K, stream)
+                                     : launch_phased<2, __half>(p, a.K, stream);
+        else
+            launched = a.bits == 4   ? launch_phased<4, float>(p, a.K, stream)
+                       : a.bits == 3 ? launch_phased<3, float>(p, a.K, stream)
+                                     : launch_phased<2, float>(p, a.K, stream);
     } else {
-        if (a.bits == 4) launch_rows<4, float>(p, smem, stream);
-        else if (a.bits == 3) launch_rows<3, float>(p, smem, stream);
-        else launch_rows<2, float>(p, smem, stream);
+        const size_t smem = rows_lds_bytes(a.N, a.K);
+        if (a.y_f16)
+            launched = a.bits == 4   ? launch_rows<4, __half>(p, smem, stream)
+                       : a.bits == 3 ? launch_rows<3, __half>(p, smem, stream)
+                                     : launch_rows<2, __half>(p, smem, stream);
+        else
+            launched = a.bits == 4   ? launch_rows<4, float>(p, smem, stream)
+                       : a.bits == 3 ? launch_rows<3, float>(p, smem, stream)
+                                     : launch_rows<2, float>(p, smem, stream);
     }
-    return launch_status("arcq_linear_otf");
+    return launched ? launch_status("arcq_linear_otf") : kNotLaunched;
 }
 
 }  // namespace arcq

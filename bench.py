@@ -120,19 +120,20 @@ class Layer:
     # The two halves of arcq_linear_otf_ws on their own.  Block-layout shapes: arcq_act_quant_blocked_with_weights
     # (stage 1 plus the weight reconstruction carried in the same launch) and arcq_linear_fused_blocked on weights
     # that are ready; other shapes: arcq_act_quant and arcq_linear_fused_ws.  A layer that runs as ONE launch
-    # ("rows": otf_rows_kernel, stage 1 + weight reconstruction + GEMM) has no halves: call_act does nothing and
-    # call_gemm is the whole layer.
+    # ("rows": otf_rows_kernel / otf_rows_phased_kernel, stage 1 + weight reconstruction + GEMM) has no halves:
+    # call_gemm is the whole layer, and call_act runs the stand-alone stage-1 kernel on the layer's input, which the
+    # step itself never launches (reported as a reference figure).
     def mode(self, lib, m):
         name = lib.arcq_linear_otf_ws_kernel(m, self.n, self.k, 1)
-        return ("rows" if name == b"otf_rows_kernel" else
+        return ("rows" if name in (b"otf_rows_kernel", b"otf_rows_phased_kernel") else
                 "copy" if name in (b"gemm_slab8_kernel<copy>", b"gemm_pair_kernel") else
                 "blocked" if b"slab8" in name else "rowmajor")
 
     def call_act(self, lib, x, ws, stream):
         from arcq_vit_amd._lib import ARCQ_F16
         mode = self.mode(lib, x.shape[0])
-        if mode == "rows":
-            return 0
+        if mode == "rows":       # no stage-1 launch of its own in the step: the stand-alone kernel, timed for reference
+            mode = "blocked"
         if mode == "copy":
             return lib.arcq_act_quant_blocked_with_weights(
                 x.data_ptr(), ARCQ_F16, self.thr.data_ptr(), self.cb.data_ptr(), ws.data_ptr(), x.shape[0], self.k,
@@ -310,10 +311,10 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
                             "shapes_nk": sorted({(l.n, l.k) for l in sub})}
 
     act_layers = [l for l in layers if l.mode(lib, m) != "rows"]          # layers with a stage-1 launch of their own
-    n_act = max(len(act_layers), 1)
+    n_act = len(layers)                                                   # (the stage-1 timing runs it for every layer)
     flops = sum(synth.algorithmic_flops(m, l.n, l.k) for l in layers)
     gemm_bytes = sum(synth.algorithmic_bytes(m, l.n, l.k, bits) for l in layers)
-    act_bytes = sum(2 * 2 * m * l.k for l in act_layers)          # fp16 in, fp16 out
+    act_bytes = sum(2 * 2 * m * l.k for l in layers)              # fp16 in, fp16 out
     res = {
         "batch": batch, "M": m, "layers": len(layers),
         "ms_per_step": t_full / steps * 1e3,
@@ -332,7 +333,7 @@ def run_config(model, bits, batch, steps, warmup, dev, use_graph=False):
         "act_kernel": {"copy": "act_quant_blocked2_kernel (block layout, weight reconstruction carried along)",
                        "blocked": "act_quant_blocked2_kernel (block layout)",
                        "rowmajor": "act_quant_g64_kernel / act_quant_small_kernel (row-major)"}[
-                           (act_layers or layers)[0].mode(lib, m) if act_layers else "copy"],
+                           act_layers[0].mode(lib, m) if act_layers else "blocked"],
     }
     return res, layers, inputs
 
@@ -471,6 +472,10 @@ def kernel_note(name):
     if name == "otf_rows_kernel":
         return ("the WHOLE layer in one launch: stage 1 of 64 rows into LDS, the fp16 weights reconstructed cooperatively "
                 "into the workspace, fp16 MFMA GEMM + bias; its duration includes stage 1 and the reconstruction")
+    if name == "otf_rows_phased_kernel":
+        return ("the WHOLE layer in one launch for K = 768 / 1536: the rows are quantized into LDS in slices of 384 values "
+                "while the MFMAs of the previous slice run; weights reconstructed cooperatively into the workspace; "
+                "its duration includes stage 1 and the reconstruction")
     if name in ("gemm_slab8_kernel<copy>", "gemm_pair_kernel"):
         return ("fp16 MFMA GEMM + bias on weights that the stage-1 launch of the same layer reconstructed into an "
                 "fp16 workspace (copied global -> LDS); its own launch does no dequantization")
@@ -515,6 +520,10 @@ def main():
     res, layers, inputs = run_config(args.model, args.bits, args.batch, args.steps, args.warmup, dev,
                                      use_graph=not args.eager)
     dom = max(res["gemm_kernels"], key=lambda k: res["gemm_kernels"][k]["ms_per_step"])
+    one = sum(v["launches_per_step"] for k, v in res["gemm_kernels"].items() if k.startswith("otf_rows"))
+    launch_note = ("every layer runs as ONE launch (stage 1 inside the GEMM kernel)" if one == res["layers"] else
+                   f"{one} of the {res['layers']} layers run as ONE launch (stage 1 inside the GEMM kernel), "
+                   f"the others as two (stage 1 + weight reconstruction, then the GEMM)")
     dk = res["gemm_kernels"][dom]
     out = {
         "metric": "DeiT-S W4A4 images/s at bs1/bs64; packed-linear % of MFMA/HBM roofline",
@@ -523,7 +532,7 @@ def main():
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"{args.model} {res['layers']} packed linears ({res['layers'] // 4} blocks x qkv/proj/fc1/fc2), W{args.bits}A{args.bits}, "
                                f"g=64, batch {args.batch} (M={res['M']}), fp16 in/out; per layer: stage 1 (activation quantize + reconstruct), the fp16 weights "
-                               f"reconstructed from the packed codes, an fp16 MFMA GEMM + bias -- one launch for K <= 384, two launches otherwise",
+                               f"reconstructed from the packed codes, an fp16 MFMA GEMM + bias -- {launch_note}",
                    "model_shapes": args.model, "bits": args.bits, "batch": args.batch, "group_size": 64},
         "roofline": {"bound": "mfma", "kernel": dom, "kernel_does": kernel_note(dom), "achieved": dk["tflops"],
                      "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": dk["tflops"] / PEAK_FP16_TFLOPS,
@@ -542,8 +551,10 @@ def main():
                      # all_fused_gemm_launches counts a one-launch layer whole (stage 1 included)
                      # whole layer = stage 1 (+ weight reconstruction) + GEMM, everything the step runs
                      "layer": layer_roofline(res, args.bits)},
+        # the stand-alone stage-1 kernel on every layer's input; the step launches it only for the two-launch layers
         "stage1": {"kernel": res["act_kernel"], "bound": "hbm", "achieved": res["act_gbs"], "peak": PEAK_HBM_GBS,
-                   "unit": "GB/s", "frac": res["act_gbs"] / PEAK_HBM_GBS, "avg_launch_us": res["act_us_per_launch"]},
+                   "unit": "GB/s", "frac": res["act_gbs"] / PEAK_HBM_GBS, "avg_launch_us": res["act_us_per_launch"],
+                   "launches_in_step": res["act_launches_per_step"], "timed_launches": res["layers"]},
         "detail_bs%d" % args.batch: res,
     }
     if not args.no_bs1:

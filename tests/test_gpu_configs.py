@@ -104,7 +104,7 @@ def test_benchmarked_layer_call_fullsize(cuda, oracle, name, k, n, bits):
         assert np.array_equal(_np(x_ws).view(np.uint16), _np(_to_blocked(torch.from_numpy(a))).view(np.uint16)), path
     if path.endswith("<copy>") or "pair" in path:       # the stage-1 launch rebuilt the weights
         assert np.array_equal(_np(w_ws).view(np.uint16), w16.reshape(-1).view(np.uint16)), path
-    if path == "otf_rows_kernel":                       # one launch: x_hat stays in LDS, w_hat in 32-column blocks
+    if path.startswith("otf_rows"):                     # one launch: x_hat stays in LDS, w_hat in 32-column blocks
         blocked = np.ascontiguousarray(w16.reshape(n // 32, 32, k // 8, 8).transpose(0, 2, 1, 3)).reshape(-1)
         assert np.array_equal(_np(w_ws).view(np.uint16), blocked.view(np.uint16)), path
     rows = torch.randint(0, m, (64,), generator=torch.Generator().manual_seed(3))

@@ -1,5 +1,6 @@
-"""GPU tests of the one-launch row-stationary layer kernel (``otf_rows_kernel``: stage 1 into LDS, weights rebuilt
-cooperatively into the workspace in 32-column blocks, product from there)."""
+"""GPU tests of the one-launch row-stationary layer kernels (``otf_rows_kernel``: stage 1 into LDS, weights rebuilt
+cooperatively into the workspace in 32-column blocks, product from there; ``otf_rows_phased_kernel``: the same for
+rows of 768 / 1536 values, quantized in slices of 384 while the previous slice is multiplied)."""
 import numpy as np
 import pytest
 import torch
@@ -31,7 +32,9 @@ def _w_blocked(w16):
 @pytest.mark.parametrize("m,n,k,bits,out", [(12608, 1152, 384, 4, torch.float16), (12608, 384, 384, 4, torch.float16),
                                             (12608, 1536, 384, 3, torch.float16), (12608, 576, 192, 4, torch.float16),
                                             (1001, 96, 192, 2, torch.float32), (3000, 1024, 256, 3, torch.float16),
-                                            (577, 32, 384, 4, torch.float32)])
+                                            (577, 32, 384, 4, torch.float32),
+                                            (12608, 384, 1536, 4, torch.float16), (12608, 192, 768, 3, torch.float32),
+                                            (9000, 96, 1536, 2, torch.float16), (6001, 384, 768, 4, torch.float32)])
 def test_rows_kernel_against_oracle_and_two_launch_path(cuda, oracle, monkeypatch, m, n, k, bits, out):
     """The kernel's y against the fp64 oracle on sampled rows (fp32-accumulation bound plus the output rounding),
     the weight workspace against the oracle's w_hat bit for bit (block layout), and y bit for bit against the
@@ -40,7 +43,8 @@ def test_rows_kernel_against_oracle_and_two_launch_path(cuda, oracle, monkeypatc
     x = synth.make_activation(m, k, 33, "ln").to(torch.float16)
     d = lambda t: t.to(cuda)
     args = (d(thr), d(cb), d(pw), d(cb), d(wc), d(ws), d(wcs), d(bias), bits, 64)
-    assert _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1) == b"otf_rows_kernel"
+    kernel = b"otf_rows_kernel" if k <= 384 else b"otf_rows_phased_kernel"
+    assert _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1) == kernel
     w_ws = torch.zeros(n * k, dtype=torch.float16, device=cuda)
     y = ops.linear_otf(d(x), *args, out_dtype=out, w_hat_ws=w_ws)
     torch.cuda.synchronize()
@@ -59,9 +63,27 @@ def test_rows_kernel_against_oracle_and_two_launch_path(cuda, oracle, monkeypatc
     y1 = ops.linear_otf(d(x), *args, out_dtype=out, w_hat_ws=off)
     assert torch.equal(y, y1) and np.array_equal(_np(off).view(np.uint16), w16.reshape(-1).view(np.uint16))
     monkeypatch.setenv("ARCQ_ROWS", "0")
-    assert _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1) != b"otf_rows_kernel"
+    assert _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1) != kernel
     y2 = ops.linear_otf(d(x), *args, out_dtype=out, w_hat_ws=torch.zeros_like(w_ws))
     assert torch.equal(y, y2)
+
+
+@pytest.mark.parametrize("m,n,k", [(16448, 384, 384), (20032, 384, 1536)])
+def test_more_row_tiles_than_the_device_holds_take_the_two_launch_path(cuda, oracle, monkeypatch, m, n, k):
+    """A workgroup of the one-launch kernels waits for the weight shares of all the others, so a launch larger than
+    the device holds at once would stall until the wait gives up.  Such calls must take the two-launch path: the
+    weight workspace then comes back row-major, and y has the bits of the call with the one-launch kernels off."""
+    cb, thr, pw, wc, ws, wcs, bias = _layer(oracle, n, k, 4, 71)
+    x = synth.make_activation(m, k, 73, "ln").to(torch.float16).to(cuda)
+    d = lambda t: t.to(cuda)
+    args = (d(thr), d(cb), d(pw), d(cb), d(wc), d(ws), d(wcs), d(bias), 4, 64)
+    assert not _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1).startswith(b"otf_rows")
+    w_ws = torch.zeros(n * k, dtype=torch.float16, device=cuda)
+    y = ops.linear_otf(x, *args, out_dtype=torch.float16, w_hat_ws=w_ws)
+    w16 = oracle.weight_dequant_c(pw.numpy(), cb, wc, ws, wcs, 4, 64, fma=True).astype(np.float16)
+    assert np.array_equal(_np(w_ws).view(np.uint16), w16.reshape(-1).view(np.uint16))
+    monkeypatch.setenv("ARCQ_ROWS", "0")
+    assert torch.equal(y, ops.linear_otf(x, *args, out_dtype=torch.float16, w_hat_ws=w_ws))
 
 
 @pytest.mark.parametrize("bits,out", [(4, torch.float16), (3, torch.float32)])
@@ -92,11 +114,40 @@ def test_rows_kernel_with_layernorm_gelu_residual(cuda, oracle, monkeypatch, bit
     assert float(close.float().mean()) > 0.999        # torch's LayerNorm may round a value differently: rare code flips
 
 
+@pytest.mark.parametrize("n,k,bits,out", [(384, 1536, 4, torch.float16), (192, 768, 3, torch.float32)])
+def test_phased_kernel_with_gelu_and_residual(cuda, oracle, monkeypatch, n, k, bits, out):
+    """arcq_linear_otf_ex on the fc2 shapes: GELU and the skip connection in the one-launch kernel's epilogue give the
+    bits of the two-launch path and of the separate torch operations behind the plain layer; a LayerNorm in front is
+    not something the kernel does, so that call takes the two-launch path (and still agrees)."""
+    m = 12608
+    cb, thr, pw, wc, ws, wcs, bias = _layer(oracle, n, k, bits, 81)
+    g = torch.Generator().manual_seed(19)
+    x = synth.make_activation(m, k, 83, "gelu").to(torch.float16).to(cuda)
+    res = torch.randn(m, n, generator=g).to(out).to(cuda)
+    d = lambda t: t.to(cuda)
+    args = (d(thr), d(cb), d(pw), d(cb), d(wc), d(ws), d(wcs), d(bias), bits, 64)
+    w_ws = torch.zeros(n * k, dtype=torch.float16, device=cuda)
+    assert _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1) == b"otf_rows_phased_kernel"
+    y = ops.linear_otf_ex(x, *args, out_dtype=out, gelu=True, residual=res, w_hat_ws=w_ws)
+    plain = ops.linear_otf(x, *args, out_dtype=out, w_hat_ws=w_ws)
+    near = lambda a, b: bool(((a.float() - b.float()).abs() <= 2.0 ** -9 * b.float().abs() + 1e-3).all())
+    assert near(y, torch.nn.functional.gelu(plain).to(out) + res)
+    assert near(ops.linear_otf_ex(x, *args, out_dtype=out, residual=res, w_hat_ws=w_ws), plain + res)
+    lw = (1 + 0.1 * torch.randn(k, generator=g)).to(cuda)
+    lb = (0.1 * torch.randn(k, generator=g)).to(cuda)
+    kw = dict(out_dtype=out, gelu=True, residual=res, w_hat_ws=w_ws)
+    y_ln = ops.linear_otf_ex(x, *args, layernorm=(lw, lb, 1e-6), **kw) if k <= 1024 else None
+    monkeypatch.setenv("ARCQ_ROWS", "0")
+    assert torch.equal(y, ops.linear_otf_ex(x, *args, **kw))
+    if y_ln is not None:
+        assert torch.equal(y_ln, ops.linear_otf_ex(x, *args, layernorm=(lw, lb, 1e-6), **kw))
+
+
 def test_rows_kernel_counter_protocol(cuda, oracle):
     """The cooperative weight reconstruction counts per stream and never resets: many calls in a row, layers of
     different sizes sharing one weight workspace (every call must find the other layer's weights replaced), two
     streams at once, and HIP graph replays with eager calls in between all give the first call's bits."""
-    shapes = [(12608, 1152, 384), (12608, 384, 384), (2000, 576, 192)]
+    shapes = [(12608, 1152, 384), (12608, 384, 384), (2000, 576, 192), (12608, 384, 1536)]
     layers = []
     for i, (m, n, k) in enumerate(shapes):
         cb, thr, pw, wc, ws, wcs, bias = _layer(oracle, n, k, 4, 50 + i)

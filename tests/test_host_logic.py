@@ -374,7 +374,25 @@ def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
     assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 1) == both8                     # the rebuild rides in stage 1
     monkeypatch.delenv("ARCQ_ROWS")
     assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 0) == b"gemm_slab8_kernel"
+    # One workgroup per 64 rows must be resident at once (256 compute units; two workgroups each for K = 192).
+    assert lib.arcq_linear_otf_ws_kernel(16384, 1152, 384, 1) == rows
+    assert lib.arcq_linear_otf_ws_kernel(16448, 1152, 384, 1) == both8
+    assert lib.arcq_linear_otf_ws_kernel(32768, 576, 192, 1) == rows
+    assert lib.arcq_linear_otf_ws_kernel(32832, 576, 192, 1) == both8
+    # Long rows and at most 384 outputs (fc2 of the small models): one launch, the row taken in slices of 384 values,
+    # from the number of row tiles on at which it beats the two launches.
+    phased = b"otf_rows_phased_kernel"
+    assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 1) == phased
+    assert lib.arcq_linear_otf_ws_kernel(12608, 192, 768, 1) == phased
+    assert lib.arcq_linear_otf_ws_kernel(8192, 384, 1536, 1) == phased                     # 128 row tiles
+    assert lib.arcq_linear_otf_ws_kernel(8128, 384, 1536, 1) == both8
+    assert lib.arcq_linear_otf_ws_kernel(5504, 384, 768, 1) == phased                      # 86 row tiles
+    assert lib.arcq_linear_otf_ws_kernel(5440, 384, 768, 1) != phased
+    assert lib.arcq_linear_otf_ws_kernel(16448, 384, 1536, 1) == both8                     # (not resident at once)
+    assert lib.arcq_linear_otf_ws_kernel(12608, 416, 1536, 1) == both8                     # (more than twelve column blocks)
+    monkeypatch.setenv("ARCQ_ROWS", "0")
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 1) == both8
+    monkeypatch.delenv("ARCQ_ROWS")
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 0) == b"gemm_slab8_kernel"
     pair = b"gemm_pair_kernel"        # several slices and at least eight row blocks per workgroup: two blocks per wave
     assert lib.arcq_linear_otf_ws_kernel(12608, 768, 768, 1) == pair                       # two slices, six slabs
