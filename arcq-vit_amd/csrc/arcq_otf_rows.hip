@@ -36,8 +36,7 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
-constexpr int kInPitch = 33;                 // dwords per row of a wave's stage-1 input tile (64 fp16 + 1 pad)
-constexpr int kWaveLds = 4608;               // bytes of LDS per wave: input tile (4224), later the output staging tile
+constexpr int kWaveLds = 4608;               // bytes of LDS per wave: the output staging tile (32 rows of 128 + 16 bytes)
 constexpr unsigned long long kEpoch = 1ull << 20;     // what one launch adds to its counter, whatever its grid
 constexpr long long kSpinTicks = 500000;     // bounded wait for the other workgroups' shares: 5 ms of the 100 MHz clock
 
@@ -125,17 +124,16 @@ otf_rows_kernel(const RowsParams p)
     const int64_t row_base = static_cast<int64_t>(blockIdx.x) * 64;
     const int64_t pieces = static_cast<int64_t>(p.N) * (K / 8);
 
-    // The wave's stage-1 tile (wave = (row block rb2, group g): 32 rows x 64 values) is requested first, so that it
-    // travels while the weights are rebuilt.
+    // The wave's stage-1 inputs (wave = (row block rb2, group g): 32 rows x 64 values; a lane pair holds one row's 64,
+    // each lane 64 contiguous bytes) are requested first, so that they travel while the weights are rebuilt.
     const int rb2 = wave / G, g = wave - rb2 * G;
     uint4 raw[4];
     {
-        const int64_t r0 = row_base + rb2 * 32 + lane / 8;
-        const __half *src = p.x + r0 * K + g * 64 + (lane % 8) * 8;
+        const int64_t r0 = row_base + rb2 * 32 + (lane >> 1);
+        const __half *src = p.x + r0 * K + g * 64 + (lane & 1) * 32;
 #pragma unroll
         for (int i = 0; i < 4; ++i)          // rows past the tensor's end read as zeros
-            raw[i] = (r0 + i * 8 < p.M) ? *reinterpret_cast<const uint4 *>(src + static_cast<int64_t>(i) * 8 * K)
-                                        : make_uint4(0, 0, 0, 0);
+            raw[i] = r0 < p.M ? *reinterpret_cast<const uint4 *>(src + i * 8) : make_uint4(0, 0, 0, 0);
     }
 
     // ---- this workgroup's share of w_hat: the inputs of this thread's first piece are requested here, the piece is
@@ -162,7 +160,6 @@ otf_rows_kernel(const RowsParams p)
     // ---- stage 1: wave = (row block rb2, group g), two lanes per (row, group) ----
     for (int i = tid; i < p.N; i += nthreads) s_bias[i] = p.bias ? p.bias[i] : 0.0f;
     {
-        uint32_t *tile = reinterpret_cast<uint32_t *>(wave_lds);
         float th[L - 1], cbv[L];
         load_quant_params<BITS>(p.thr, p.cb_a, th, cbv);
         const BucketScale bq = pick_bucket_scale<BITS>(th);
@@ -180,14 +177,6 @@ otf_rows_kernel(const RowsParams p)
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the written-through pieces have reached memory
         }
         const int row = lane >> 1, half = lane & 1;
-        {
-            uint32_t *dst = tile + (lane / 8) * kInPitch + (lane % 8) * 4;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                uint32_t *d = dst + i * 8 * kInPitch;
-                d[0] = raw[i].x; d[1] = raw[i].y; d[2] = raw[i].z; d[3] = raw[i].w;
-            }
-        }
         __syncthreads();                          // the tables are complete, and so is the workgroup's share of w_hat
         if (p.counter && tid == 0) {
             const unsigned long long inc = blockIdx.x == 0 ? kEpoch - (gridDim.x - 1) : 1ull;
@@ -195,13 +184,13 @@ otf_rows_kernel(const RowsParams p)
             target = (old & ~(kEpoch - 1)) + kEpoch;            // every launch adds kEpoch in total
         }
         float xv[32];
-        {
-            const uint32_t *src = tile + row * kInPitch + half * 16;
 #pragma unroll
-            for (int q = 0; q < 16; ++q) {
-                const uint32_t w = src[q];
-                xv[2 * q] = __half2float(__ushort_as_half(static_cast<unsigned short>(w & 0xffffu)));
-                xv[2 * q + 1] = __half2float(__ushort_as_half(static_cast<unsigned short>(w >> 16)));
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w4[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                xv[8 * i + 2 * e] = __half2float(__ushort_as_half(static_cast<unsigned short>(w4[e] & 0xffffu)));
+                xv[8 * i + 2 * e + 1] = __half2float(__ushort_as_half(static_cast<unsigned short>(w4[e] >> 16)));
             }
         }
         if (p.gamma) {
