@@ -146,10 +146,13 @@ int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const
  * y is bit-identical in every case; the contents of w_hat_ws after the call are unspecified.  arcq_linear_otf_ws treats
  * x_hat_ws as scratch too (unspecified contents afterwards: it may hold x_hat in the block layout described below, or
  * be left untouched); call arcq_linear_otf to get x_hat row-major in x_hat_ws.
- * With fp16 x, M >= 512, K = 192 / 256 / 384, N a multiple of 32 and w_hat_ws given (128-byte aligned),
- * arcq_linear_otf_ws runs the whole
- * layer as ONE launch (x_hat stays on chip; w_hat_ws is filled cooperatively, in 32-column blocks
- * [N/32][K/8][32][8]).  That launch counts in a word of the library's static device memory chosen by `stream`: calls
+ * With fp16 x, N a multiple of 32, w_hat_ws given (128-byte aligned) and 512 <= M <= 64 x the device's compute units
+ * (twice that for K = 192), arcq_linear_otf_ws runs the whole layer as ONE launch for K = 192 / 256 / 384, and for
+ * K = 768 / 1536 with N <= 384 from 86 / 128 blocks of 64 rows on (x_hat stays on chip; w_hat_ws is filled
+ * cooperatively, in 32-column blocks [N/32][K/8][32][8]).  The upper limit on M keeps every workgroup of the launch
+ * resident at once: each waits, for at most 5 ms, until all the others have written their share of w_hat; if the
+ * device is shared with other kernels at that moment the wait can run out, after which a workgroup rebuilds all of
+ * w_hat itself (same result, late).  That launch counts in a word of the library's static device memory chosen by `stream`: calls
  * on one stream run one after another as always; a HIP graph captured from a stream must not be replayed
  * concurrently with other calls made on that same stream; the first 256 streams a process uses for such calls on a
  * device get a word each, calls on further streams take the two-launch path.  ARCQ_ROWS=0 in the environment keeps
