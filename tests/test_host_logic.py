@@ -432,3 +432,27 @@ def test_block_layout_entry_points_validate_before_launching():
     assert lib.arcq_act_quant_blocked_with_weights(*wargs(8, None)) == -3
     assert lib.arcq_act_quant_blocked_with_weights(*wargs(8, p + 130)) == -7
     assert lib.arcq_act_quant_blocked_with_weights(*wargs(-1)) == -4
+
+
+def test_bench_host_side_contract():
+    """bench.py without a GPU: more than one GPU is refused with a message, and the committed rocprofv3 summaries
+    hold a traffic line for the kernel that dominates each benchmarked configuration (bench.py's roofline.traffic
+    is read from them, so a renamed kernel must not turn it into null unnoticed)."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    root = Path(__file__).resolve().parents[1]
+    proc = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert proc.returncode == 2 and "one GPU" in proc.stderr and not proc.stdout.strip()
+    sys.path.insert(0, str(root))
+    try:
+        import bench
+    finally:
+        sys.path.pop(0)
+    for (model, bits, batch), kernels in {("deit_small", 4, 64): ("otf_rows_kernel", "otf_rows_phased_kernel"),
+                                          ("deit_base", 4, 64): ("gemm_pair_kernel",),
+                                          ("vit_large", 3, 256): ("gemm_pair_kernel",)}.items():
+        for kernel in kernels:
+            traffic = bench.profiled_traffic(model, bits, batch, kernel)
+            assert traffic is not None and traffic > 1e6, (model, kernel)
+    assert bench.profiled_traffic("deit_small", 4, 64, "no_such_kernel") is None
