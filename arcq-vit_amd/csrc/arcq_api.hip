@@ -53,6 +53,11 @@ void read_tuning()
     g_tuning.view.otf_fused = grab("ARCQ_OTF_FUSED", g_tuning.otf_fused, sizeof(g_tuning.otf_fused));
     g_tuning.view.pair = grab("ARCQ_PAIR", g_tuning.pair, sizeof(g_tuning.pair));
     g_tuning.view.rows = grab("ARCQ_ROWS", g_tuning.rows, sizeof(g_tuning.rows));
+    // (ARCQ_ROWS_WAIT_TICKS=0 makes every workgroup of the one-launch kernels give up waiting at once and rebuild the
+    // weights itself: how the tests reach that path)
+    const char *ticks = getenv("ARCQ_ROWS_WAIT_TICKS");
+    g_tuning.view.rows_wait_ticks = ticks ? strtoll(ticks, nullptr, 10) : kRowsWaitTicks;
+    if (g_tuning.view.rows_wait_ticks < 0) g_tuning.view.rows_wait_ticks = kRowsWaitTicks;
 }
 }  // namespace
 

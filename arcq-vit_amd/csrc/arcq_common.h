@@ -26,7 +26,9 @@ struct Tuning {
     const char *otf_fused;     // "0" | "2"
     const char *pair;          // "0" | "1"
     const char *rows;          // "0" | "1": the one-launch row-stationary layer kernel off / wherever it can run
+    long long rows_wait_ticks; // bound of that kernel's wait for the other workgroups, in ticks of the 100 MHz clock
 };
+constexpr long long kRowsWaitTicks = 50000;     // 0.5 ms
 const Tuning &tuning();
 
 __host__ __device__ inline bool bits_ok(int bits) { return bits == 2 || bits == 3 || bits == 4; }

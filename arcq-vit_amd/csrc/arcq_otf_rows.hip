@@ -14,7 +14,7 @@
 // Weights: w_hat is rebuilt from the packed codes inside the same launch, cooperatively: every workgroup
 // reconstructs 1/gridDim of it into the workspace (16-byte pieces, written through to memory), adds to a counter,
 // does its stage 1, and then waits for the counter to show that all shares have been written.  The wait is bounded:
-// a workgroup that has not seen the others finish within a few milliseconds (they may not be resident) rebuilds
+// a workgroup that has not seen the others finish within half a millisecond (they may not be resident) rebuilds
 // the whole matrix itself -- same values, so a share written twice is harmless -- and goes on.  No workgroup ever
 // waits before it has contributed its share, so the counter always completes.
 //
@@ -38,7 +38,6 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kWaveLds = 4608;               // bytes of LDS per wave: the output staging tile (32 rows of 128 + 16 bytes)
 constexpr unsigned long long kEpoch = 1ull << 20;     // what one launch adds to its counter, whatever its grid
-constexpr long long kSpinTicks = 500000;     // bounded wait for the other workgroups' shares: 5 ms of the 100 MHz clock
 
 constexpr int gcd_of(int a, int b) { return b == 0 ? a : gcd_of(b, a % b); }
 
@@ -52,6 +51,7 @@ struct RowsParams {
     const float *cb_w, *wc, *ws, *wcs;
     __half *w_blk;                   // weight workspace, block layout
     unsigned long long *counter;     // nullptr: w_blk is complete already
+    long long wait_ticks;            // bound of the wait for the other workgroups' shares, ticks of the 100 MHz clock
     const float *bias;               // [N] or nullptr
     void *y;
     const void *residual;
@@ -260,7 +260,7 @@ otf_rows_kernel(const RowsParams p)
         int ok = 1;
         const long long t0 = wall_clock64();
         while (__hip_atomic_load(p.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-            if (wall_clock64() - t0 > kSpinTicks) {
+            if (wall_clock64() - t0 > p.wait_ticks) {
                 ok = 0;
                 break;
             }
@@ -583,7 +583,7 @@ otf_rows_phased_kernel(const RowsParams p)
                 int ok = 1;
                 const long long t0 = wall_clock64();
                 while (__hip_atomic_load(p.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-                    if (wall_clock64() - t0 > kSpinTicks) {
+                    if (wall_clock64() - t0 > p.wait_ticks) {
                         ok = 0;
                         break;
                     }
@@ -818,6 +818,7 @@ int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream)
     p.w_blk = static_cast<__half *>(a.w_hat_ws);
     p.counter = counter_for(stream);
     if (!p.counter) return kNotLaunched;     // more streams than counters: the caller takes the two-launch path
+    p.wait_ticks = tuning().rows_wait_ticks;
     p.bias = a.bias, p.y = a.y, p.residual = a.residual, p.gelu = a.gelu ? 1 : 0;
     p.M = a.M, p.N = a.N, p.G = a.K / 64;
     bool launched;

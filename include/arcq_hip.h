@@ -150,7 +150,7 @@ int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const
  * (twice that for K = 192), arcq_linear_otf_ws runs the whole layer as ONE launch for K = 192 / 256 / 384, and for
  * K = 768 / 1536 with N <= 384 from 86 / 128 blocks of 64 rows on (x_hat stays on chip; w_hat_ws is filled
  * cooperatively, in 32-column blocks [N/32][K/8][32][8]).  The upper limit on M keeps every workgroup of the launch
- * resident at once: each waits, for at most 5 ms, until all the others have written their share of w_hat; if the
+ * resident at once: each waits, for at most 0.5 ms, until all the others have written their share of w_hat; if the
  * device is shared with other kernels at that moment the wait can run out, after which a workgroup rebuilds all of
  * w_hat itself (same result, late).  That launch counts in a word of the library's static device memory chosen by `stream`: calls
  * on one stream run one after another as always; a HIP graph captured from a stream must not be replayed

@@ -195,3 +195,27 @@ def test_rows_kernel_counter_protocol(cuda, oracle):
         assert torch.equal(y, first[0]), rep
         assert torch.equal(ops.linear_otf(layers[1][0], *layers[1][1], out_dtype=torch.float16, w_hat_ws=shared), first[1])
         torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("m,n,k,bits", [(12608, 1152, 384, 4), (3000, 576, 192, 3), (12608, 384, 1536, 4)])
+def test_rows_kernels_when_nobody_waits(cuda, oracle, monkeypatch, m, n, k, bits):
+    """The wait for the other workgroups' weight shares is bounded; with the bound set to zero every workgroup gives
+    up at once and reconstructs all the weights itself (what happens, later, when part of a launch is not resident).
+    Same y, same weight workspace, and the calls that follow with the normal bound find the counter in order."""
+    cb, thr, pw, wc, ws, wcs, bias = _layer(oracle, n, k, bits, 91)
+    x = synth.make_activation(m, k, 93, "ln").to(torch.float16).to(cuda)
+    d = lambda t: t.to(cuda)
+    args = (d(thr), d(cb), d(pw), d(cb), d(wc), d(ws), d(wcs), d(bias), bits, 64)
+    assert _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1).startswith(b"otf_rows")
+    w_ws = torch.zeros(n * k, dtype=torch.float16, device=cuda)
+    want = ops.linear_otf(x, *args, out_dtype=torch.float16, w_hat_ws=w_ws)
+    w_want = w_ws.clone()
+    monkeypatch.setenv("ARCQ_ROWS_WAIT_TICKS", "0")
+    for _ in range(3):
+        w_ws.zero_()
+        assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float16, w_hat_ws=w_ws), want)
+        assert torch.equal(w_ws, w_want)
+    monkeypatch.delenv("ARCQ_ROWS_WAIT_TICKS")
+    w_ws.zero_()
+    assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float16, w_hat_ws=w_ws), want)
+    assert torch.equal(w_ws, w_want)
