@@ -1,6 +1,8 @@
-// Whole on-the-fly layer in ONE launch for short rows (K <= 512) and many of them: a workgroup owns 64 rows of x,
-// quantizes them into LDS (stage 1, optionally with the LayerNorm in front of it) and multiplies them with every
-// column of w_hat, which streams through the registers from a 32-column block layout in the weight workspace.
+// Whole on-the-fly layer in ONE launch for many rows of moderate length: a workgroup owns 64 rows of x, quantizes
+// them into LDS (stage 1, optionally with the LayerNorm in front of it) and multiplies them with every column of
+// w_hat, which streams through the registers from a 32-column block layout in the weight workspace.  Two kernels:
+// otf_rows_kernel (K = 192 / 256 / 384: the whole row at once) and otf_rows_phased_kernel (K = 768 / 1536, at most
+// 384 output columns: the row in slices of 384 values, stage 1 of a slice under the MFMAs of the one before).
 //
 //   y[M,N] = post( stage1( [LayerNorm] x )[M,K] * w_hat[N,K]^T + bias )
 //
@@ -9,7 +11,8 @@
 // are a third of the layer.  Here x_hat never leaves the CU (64 rows x K fp16 = 48 KB of LDS at K = 384), stage 1
 // runs on all twelve waves at once (wave = 32 rows x one group, two lanes per group), and the product starts the
 // moment the workgroup's own rows are done.  The price is that every workgroup reads all of w_hat from L2
-// (N*K*2 bytes, 0.9 MB for DeiT-S qkv) -- affordable only while K is short.
+// (N*K*2 bytes, 0.9 MB for DeiT-S qkv) -- affordable only while N*K is small -- and that the launch must not have
+// more workgroups than the device holds at once (see resident_workgroups below).
 //
 // Weights: w_hat is rebuilt from the packed codes inside the same launch, cooperatively: every workgroup
 // reconstructs 1/gridDim of it into the workspace (16-byte pieces, written through to memory), adds to a counter,
