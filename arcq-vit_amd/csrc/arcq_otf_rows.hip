@@ -16,7 +16,10 @@
 //
 // Weights: w_hat is rebuilt from the packed codes inside the same launch, cooperatively: every workgroup
 // reconstructs 1/gridDim of it into the workspace (16-byte pieces, written through to memory), adds to a counter,
-// does its stage 1, and then waits for the counter to show that all shares have been written.  The wait is bounded:
+// does its stage 1, and then waits for the counter to show that all shares have been written.  While the row tiles
+// leave compute units free, otf_rows_kernel's launch carries extra workgroups that do nothing but this
+// reconstruction, and the row workgroups only count (a quarter off the layer at 1 024 rows, nothing at 12 608).
+// The wait is bounded:
 // a workgroup that has not seen the others finish within half a millisecond (they may not be resident) rebuilds
 // the whole matrix itself -- same values, so a share written twice is harmless -- and goes on.  No workgroup ever
 // waits before it has contributed its share, so the counter always completes.
@@ -152,7 +155,26 @@ otf_rows_kernel(const RowsParams p)
     int64_t share_lo = 0, share_hi = 0;
     Piece pc{};
     unsigned long long target = 0;
-    if (p.counter) {
+    // Workgroups beyond the row tiles are helpers (the launcher adds them while compute units are free): they
+    // reconstruct all of w_hat between them, count, and are done; the row workgroups then only count.
+    const int row_wgs = (p.M + 63) / 64;
+    const int helpers = static_cast<int>(gridDim.x) - row_wgs;
+    if (static_cast<int>(blockIdx.x) >= row_wgs) {
+        int64_t per = (pieces + helpers - 1) / helpers;
+        per = (per + 7) & ~int64_t(7);
+        const int64_t lo = (static_cast<int>(blockIdx.x) - row_wgs) * per;
+        const int64_t hi = lo + per < pieces ? lo + per : pieces;
+        for (int64_t idx = lo + tid; idx < hi; idx += nthreads) {
+            fetch_piece<BITS, G>(p, idx, pc);
+            finish_piece<BITS>(p, idx, pc);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) __hip_atomic_fetch_add(p.counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    const bool own_share = p.counter && helpers == 0;
+    if (own_share) {
         int64_t per = (pieces + gridDim.x - 1) / gridDim.x;
         per = (per + 7) & ~int64_t(7);                          // whole 128-byte lines per workgroup
         share_lo = blockIdx.x * per;
@@ -171,7 +193,7 @@ otf_rows_kernel(const RowsParams p)
         // the phase).
         if (wave >= kBuilder0 && wave < kBuilder0 + kBuilders)
             build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slow_slots, tid - 64 * kBuilder0, 64 * kBuilders);
-        if (p.counter) {
+        if (own_share) {
             if (ptid >= 0 && share_lo + ptid < share_hi) finish_piece<BITS>(p, share_lo + ptid, pc);
             for (int64_t idx = share_lo + kPieceThreads + ptid; ptid >= 0 && idx < share_hi; idx += kPieceThreads) {     // (large N*K only)
                 fetch_piece<BITS, G>(p, idx, pc);
@@ -736,14 +758,27 @@ size_t rows_lds_bytes(int N, int K)
            static_cast<size_t>(N) * sizeof(float);
 }
 
+// Workgroups to add to a launch for the reconstruction of w_hat alone, given `spare` free places on the device: one
+// per `threads` pieces (every thread one piece), if at least half as many are to be had -- otherwise none, and the
+// row workgroups share the reconstruction.
+int helper_workgroups(const RowsParams &p, int spare, int threads)
+{
+    const int64_t pieces = static_cast<int64_t>(p.N) * p.G * 8;
+    const int want = static_cast<int>((pieces + threads - 1) / threads);
+    if (spare * 2 < want) return 0;
+    return spare < want ? spare : want;
+}
+
 // The launchers return false, having launched nothing, when the device would not hold the whole grid at once.
 template <int BITS, typename TOUT, int G, int RING, int AHEAD>
 bool launch_rows_g(const RowsParams &p, size_t smem, hipStream_t stream)
 {
     allow_dynamic_lds<otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>>(160 * 1024 - 10 * 1024);
     const int tiles = (p.M + 63) / 64;
-    if (resident_workgroups<otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>>(128 * G, smem) < tiles) return false;
-    hipLaunchKernelGGL((otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>), dim3(tiles), dim3(128 * G), smem, stream, p);
+    const int cap = resident_workgroups<otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>>(128 * G, smem);
+    if (cap < tiles) return false;
+    hipLaunchKernelGGL((otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>), dim3(tiles + helper_workgroups(p, cap - tiles, 128 * G)),
+                       dim3(128 * G), smem, stream, p);
     return true;
 }
 
