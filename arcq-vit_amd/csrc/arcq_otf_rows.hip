@@ -843,7 +843,11 @@ bool otf_rows_pays(int64_t M, int64_t N, int64_t K, bool layernorm)
         const int64_t tiles = (M + 63) / 64;
         return tiles * (K == 1536 ? 2 : 3) >= device_cus();
     }
-    return true;
+    // otf_rows_kernel takes about 8 us + 23 ps per weight whatever the number of rows (every workgroup streams all of
+    // w_hat); the two launches take about 12 us + 2.6 fs per multiply-add.  Fitted on N = 384 .. 1536, K = 192 .. 384,
+    // M = 512 .. 12608: one launch from about 6 200 rows on for DeiT-S qkv, 6 900 for fc1, always for proj.
+    const double weights = static_cast<double>(N) * static_cast<double>(K);
+    return static_cast<double>(M) >= 8800.0 - 1.15e9 / weights;
 }
 
 int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream)

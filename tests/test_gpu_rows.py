@@ -31,7 +31,7 @@ def _w_blocked(w16):
 
 @pytest.mark.parametrize("m,n,k,bits,out", [(12608, 1152, 384, 4, torch.float16), (12608, 384, 384, 4, torch.float16),
                                             (12608, 1536, 384, 3, torch.float16), (12608, 576, 192, 4, torch.float16),
-                                            (1001, 96, 192, 2, torch.float32), (3000, 1024, 256, 3, torch.float16),
+                                            (1001, 96, 192, 2, torch.float32), (5000, 1024, 256, 3, torch.float16),
                                             (577, 32, 384, 4, torch.float32),
                                             (12608, 384, 1536, 4, torch.float16), (12608, 192, 768, 3, torch.float32),
                                             (9000, 96, 1536, 2, torch.float16), (6001, 384, 768, 4, torch.float32)])
@@ -91,7 +91,8 @@ def test_rows_kernel_with_layernorm_gelu_residual(cuda, oracle, monkeypatch, bit
     """arcq_linear_otf_ex through the one-launch kernel: LayerNorm in front, GELU and the skip connection behind,
     bit for bit what the two-launch path gives (whose parts are checked against the oracle elsewhere) and what the
     separate torch operations give around the plain layer."""
-    m, n, k = 4000, 768, 384
+    m, n, k = 6016, 768, 384
+    assert _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1) == b"otf_rows_kernel"
     cb, thr, pw, wc, ws, wcs, bias = _layer(oracle, n, k, bits, 41)
     g = torch.Generator().manual_seed(9)
     x = (synth.make_activation(m, k, 43, "ln") * 1.7 + 0.3).to(torch.float16).to(cuda)

@@ -367,7 +367,13 @@ def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
     rows = b"otf_rows_kernel"         # short rows (K = 192 / 256 / 384) and both workspaces: the whole layer in one launch
     assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 1) == rows
     assert lib.arcq_linear_otf_ws_kernel(12608, 576, 192, 1) == rows
-    assert lib.arcq_linear_otf_ws_kernel(1000, 1024, 256, 1) == rows                        # any number of rows from 512 on
+    assert lib.arcq_linear_otf_ws_kernel(512, 576, 192, 1) == rows                          # few weights: from 512 rows on
+    assert lib.arcq_linear_otf_ws_kernel(1024, 384, 384, 1) == rows
+    assert lib.arcq_linear_otf_ws_kernel(6304, 1152, 384, 1) == rows                        # many weights: where it beats two launches
+    assert lib.arcq_linear_otf_ws_kernel(6144, 1152, 384, 1) == both8
+    assert lib.arcq_linear_otf_ws_kernel(6976, 1536, 384, 1) == rows
+    assert lib.arcq_linear_otf_ws_kernel(6720, 1536, 384, 1) == both8
+    assert lib.arcq_linear_otf_ws_kernel(4480, 1024, 256, 1) == rows
     assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 320, 1) == both8                     # (no instance for five groups)
     assert lib.arcq_linear_otf_ws_kernel(12608, 1000, 384, 1) == both8                     # (N must be whole 32-column blocks)
     monkeypatch.setenv("ARCQ_ROWS", "0")
