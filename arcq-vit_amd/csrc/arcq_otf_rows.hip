@@ -758,14 +758,15 @@ size_t rows_lds_bytes(int N, int K)
            static_cast<size_t>(N) * sizeof(float);
 }
 
-// Workgroups to add to a launch for the reconstruction of w_hat alone, given `spare` free places on the device: one
-// per `threads` pieces (every thread one piece), if at least half as many are to be had -- otherwise none, and the
-// row workgroups share the reconstruction.
-int helper_workgroups(const RowsParams &p, int spare, int threads)
+// Workgroups to add to a launch of `tiles` row workgroups for the reconstruction of w_hat alone, given `spare` free
+// places on the device: one per `threads` pieces (every thread one piece), if at least half as many are to be had and
+// the row tiles fill at most half the device -- otherwise none, and the row workgroups share the reconstruction
+// (with many row workgroups each one's share is small and hides under its load latency; helpers then cost 1 %).
+int helper_workgroups(const RowsParams &p, int tiles, int spare, int threads)
 {
     const int64_t pieces = static_cast<int64_t>(p.N) * p.G * 8;
     const int want = static_cast<int>((pieces + threads - 1) / threads);
-    if (spare * 2 < want) return 0;
+    if (spare < tiles || spare * 2 < want) return 0;
     return spare < want ? spare : want;
 }
 
@@ -777,7 +778,7 @@ bool launch_rows_g(const RowsParams &p, size_t smem, hipStream_t stream)
     const int tiles = (p.M + 63) / 64;
     const int cap = resident_workgroups<otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>>(128 * G, smem);
     if (cap < tiles) return false;
-    hipLaunchKernelGGL((otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>), dim3(tiles + helper_workgroups(p, cap - tiles, 128 * G)),
+    hipLaunchKernelGGL((otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>), dim3(tiles + helper_workgroups(p, tiles, cap - tiles, 128 * G)),
                        dim3(128 * G), smem, stream, p);
     return true;
 }
