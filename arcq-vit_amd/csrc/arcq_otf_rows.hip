@@ -308,21 +308,26 @@ otf_rows_kernel(const RowsParams p)
         }
     }
 
-    // ---- the product: wave tile = 64 rows x one 32-column block; blocks wave, wave + W, ... ----
+    // ---- the product: wave tile = 64 rows x one 32-column block; every wave a run of N / 32 / W blocks ----
     const int lr = lane & 31, lh = lane >> 5;
     const int ncb = p.N / 32;
     const unsigned char *xs_lane = xs + lr * pitch + lh * 64;
     const char *w_lane = reinterpret_cast<const char *>(p.w_blk) + lh * 2048 + lr * 16;
     const int64_t cb_bytes = static_cast<int64_t>(K) * 64;     // bytes per 32-column block
-    int ld_cb = wave, ld_g = 0;
+    // The wave's blocks are a run of adjacent ones: a row's 64-byte segments of two neighbouring blocks share a
+    // 128-byte line, and written by one wave shortly after each other they are more often merged on their way to
+    // memory than when twelve waves write them at unrelated times (qkv: 38.5 -> 35.7 MB written per launch).
+    const int bpw = (ncb + W - 1) / W;
+    const int cb_first = wave * bpw, cb_last = cb_first + bpw < ncb ? cb_first + bpw : ncb;
+    int ld_cb = cb_first, ld_g = 0;
     auto load_unit = [&](u32x4_t (&r)[4]) {      // the four fragments of one group; past the wave's last block it re-reads a valid one
-        const int c = ld_cb < ncb ? ld_cb : ncb - 1;
+        const int c = ld_cb < cb_last ? ld_cb : ncb - 1;
         const char *q = w_lane + c * cb_bytes + ld_g * 4096;
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) r[kk] = *reinterpret_cast<const u32x4_t *>(q + kk * 512);
         if (++ld_g == G) {
             ld_g = 0;
-            ld_cb += W;
+            ++ld_cb;
         }
     };
     // Ring of RING groups, walked with compile-time slot numbers: group number s (counted over the wave's column
@@ -342,11 +347,11 @@ otf_rows_kernel(const RowsParams p)
     TOUT *y = static_cast<TOUT *>(p.y);
     const TOUT *residual = static_cast<const TOUT *>(p.residual);
 
-    for (int cb0 = wave; cb0 < ncb; cb0 += kUnroll * W) {
+    for (int cb0 = cb_first; cb0 < cb_last; cb0 += kUnroll) {
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
-        const int cbk = cb0 + u * W;
-        if (cbk >= ncb) break;
+        const int cbk = cb0 + u;
+        if (cbk >= cb_last) break;
         float16_t acc[2];
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
