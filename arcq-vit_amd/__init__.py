@@ -22,6 +22,7 @@ from .packed_convert import (  # noqa: F401
     convert_arcq_linear_to_packed,
     count_packed_linear,
     load_packed_state_dict,
+    set_fp8_operands,
     share_buffers,
     to_on_the_fly,
 )
@@ -44,4 +45,5 @@ __all__ = [
     "FrozenARCQQuantizer", "convert_arcq_linear_to_packed", "count_packed_linear", "to_on_the_fly",
     "load_packed_state_dict", "infer_packed_hparams", "share_buffers", "clear_workspaces",
     "ARCQPackedPatchConv", "convert_arcq_conv_to_packed", "QuantConv2dPCARCQ", "QuantLinearLSQ", "LSQQuantizer",
+    "set_fp8_operands",
 ]

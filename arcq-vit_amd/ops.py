@@ -422,6 +422,94 @@ def linear_otf_ex(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch
     return y
 
 
+# ---------------------------------------------------------------------------------------------
+# the layer with FP8 operands -- no counterpart in the reference; a faster, less exact stage 3
+# ---------------------------------------------------------------------------------------------
+FP8_MAX = 448.0          # largest finite OCP E4M3 value
+
+
+def quantize_activation_fp8(x: torch.Tensor, thresholds: torch.Tensor, codebook: torch.Tensor, bits: int,
+                            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Stage 1 with the reconstruction rounded to FP8 (``torch.float8_e4m3fn``, row-major ``[M, K]``) instead of fp16;
+    group size 64.  Codes, ``mu`` and ``s`` are those of ``quantize_activation``."""
+    _check(x.is_cuda and x.dim() == 2, "x must be a CUDA tensor of shape [M, K]")
+    _check_bits(bits)
+    x = x.contiguous()
+    m, k = x.shape
+    if out is None:
+        out = torch.empty((m, k), dtype=torch.float8_e4m3fn, device=x.device)
+    else:
+        _check(out.dtype == torch.float8_e4m3fn and out.is_contiguous() and out.numel() >= m * k,
+               "out must be a contiguous float8_e4m3fn buffer of at least M*K elements")
+    thresholds, codebook = _f32c(thresholds), _f32c(codebook)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().arcq_act_quant_fp8(_ptr(x), _dtype_code(x, "x"), _ptr(thresholds), _ptr(codebook), _ptr(out),
+                                                  m, k, bits, 1.0e-6, _stream()))
+    return out
+
+
+def fp8_weight_multiplier(w_codebook: torch.Tensor, w_center: torch.Tensor, w_scale: torch.Tensor,
+                          w_code_sum: torch.Tensor) -> float:
+    """Power of two that moves a layer's reconstructed weights into FP8's normal range: the largest one that keeps a
+    bound on ``|w_hat|`` (``|center| + |scale| (max |cb| + |code_sum| / 64)`` over all groups) at or below half the
+    largest FP8 value.  Reads the metadata back to the host: compute it once per layer."""
+    cb = float(w_codebook.abs().max())
+    bound = float((w_center.abs() + w_scale.abs() * (cb + w_code_sum.abs() / 64.0)).max())
+    if not bound > 0.0:
+        return 1.0
+    import math
+    return float(2.0 ** math.floor(math.log2(FP8_MAX / 2.0 / bound)))
+
+
+def unpack_weight_fp8(packed: torch.Tensor, codebook: torch.Tensor, center: torch.Tensor, scale: torch.Tensor,
+                      code_sum: torch.Tensor, bits: int, w_mult: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Stage 2 with the weights rounded to FP8: ``fp8(w_mult * w_hat)``, row-major ``[N, K]``; group size 64."""
+    _check(packed.is_cuda and packed.dtype == torch.uint8, "packed must be a CUDA uint8 tensor")
+    _check_bits(bits)
+    n = packed.shape[0]
+    k = center.shape[1] * 64
+    _check(packed.shape[1] == (k * bits + 7) // 8, "packed row length does not match in_features*bits/8")
+    if out is None:
+        out = torch.empty((n, k), dtype=torch.float8_e4m3fn, device=packed.device)
+    else:
+        _check(out.dtype == torch.float8_e4m3fn and out.is_contiguous() and out.numel() >= n * k,
+               "out must be a contiguous float8_e4m3fn buffer of at least N*K elements")
+    packed = packed.contiguous()
+    codebook, center, scale, code_sum = _f32c(codebook), _f32c(center), _f32c(scale), _f32c(code_sum)
+    with torch.cuda.device(packed.device):
+        _lib.check(_lib.load().arcq_weight_dequant_fp8(_ptr(packed), _ptr(codebook), _ptr(center), _ptr(scale),
+                                                       _ptr(code_sum), _ptr(out), n, k, bits, 64, float(w_mult), _stream()))
+    return out
+
+
+def linear_otf_fp8(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Tensor, packed_w: torch.Tensor,
+                   w_codebook: torch.Tensor, w_center: torch.Tensor, w_scale: torch.Tensor, w_code_sum: torch.Tensor,
+                   bias: Optional[torch.Tensor], bits: int, out_dtype: torch.dtype = torch.float16,
+                   w_mult: Optional[float] = None, x8_ws: Optional[torch.Tensor] = None,
+                   w8_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The packed on-the-fly layer with FP8 operands: stage 1 and stage 2 as in ``linear_otf`` but rounded to FP8, the
+    product as the vendor library's FP8 GEMM with fp32 accumulation (``torch._scaled_mm``), ``y = x8 w8^T / w_mult +
+    bias``.  Faster where the layer is bound by the matrix units (the large models), NOT bit-compatible with the
+    reference: each operand carries a rounding error of up to 2^-4 relative (fp16: 2^-11).  Group size 64."""
+    _check(x.is_cuda and x.dim() == 2, "x must be a CUDA tensor of shape [M, K]")
+    m, k = x.shape
+    n = packed_w.shape[0]
+    _check(k % 16 == 0 and n % 16 == 0, "the FP8 GEMM needs K and N to be multiples of 16")
+    if w_mult is None:
+        w_mult = fp8_weight_multiplier(w_codebook, w_center, w_scale, w_code_sum)
+    x8 = quantize_activation_fp8(x, a_thresholds, a_codebook, bits, out=x8_ws)
+    w8 = unpack_weight_fp8(packed_w, w_codebook, w_center, w_scale, w_code_sum, bits, w_mult, out=w8_ws)
+    x8 = x8.view(-1)[:m * k].view(m, k)
+    w8 = w8.view(-1)[:n * k].view(n, k)
+    one = torch.ones((), dtype=torch.float32, device=x.device)
+    inv = torch.full((), 1.0 / float(w_mult), dtype=torch.float32, device=x.device)
+    has_bias = bias is not None and bias.numel() > 0
+    if has_bias and out_dtype == torch.float16:      # (the library adds a bias of the output's type; fp16 only)
+        return torch._scaled_mm(x8, w8.t(), scale_a=one, scale_b=inv, bias=bias.to(torch.float16), out_dtype=out_dtype)
+    y = torch._scaled_mm(x8, w8.t(), scale_a=one, scale_b=inv, out_dtype=out_dtype)
+    return y + bias.to(out_dtype) if has_bias else y
+
+
 def linear_fused_blocked(x_hat_blocked: torch.Tensor, m: int, k: int, packed_w: torch.Tensor, w_codebook: torch.Tensor,
                          w_center: torch.Tensor, w_scale: torch.Tensor, w_code_sum: torch.Tensor,
                          bias: Optional[torch.Tensor], bits: int, out_dtype: torch.dtype = torch.float16,

@@ -90,6 +90,10 @@ class ARCQPackedLinearOnTheFly(nn.Module):
             self.register_buffer("bias_tensor", torch.empty(0))
         self.out_dtype = torch.float16
         self._prep = None
+        # Opt-in: operands rounded to FP8 and the product on FP8 matrix units (ops.linear_otf_fp8).  Faster on the
+        # large models, not the reference's numerics; see set_fp8_operands in packed_convert.
+        self.fp8_operands = False
+        self._fp8_mult = None
 
     def _prepare(self):
         """Validated, fp32-contiguous views of the buffers and their raw pointers, built once and reused by every
@@ -105,6 +109,7 @@ class ARCQPackedLinearOnTheFly(nn.Module):
 
     def _load_from_state_dict(self, *args, **kwargs):
         self._prep = None
+        self._fp8_mult = None
         return super()._load_from_state_dict(*args, **kwargs)
 
     @classmethod
@@ -152,7 +157,7 @@ class ARCQPackedLinearOnTheFly(nn.Module):
         x2 = x2.contiguous()
         m = x2.shape[0]
         extras = layernorm is not None or activation is not None or residual is not None
-        fuse = (extras and m >= 512 and self.group_size == 64 and self.in_features % 64 == 0
+        fuse = (extras and not self.fp8_operands and m >= 512 and self.group_size == 64 and self.in_features % 64 == 0
                 and (layernorm is None or (self.in_features <= 1024 and layernorm.elementwise_affine
                                            and tuple(layernorm.normalized_shape) == (self.in_features,))))
         if extras and not fuse:          # separate operations around the plain layer
@@ -167,8 +172,19 @@ class ARCQPackedLinearOnTheFly(nn.Module):
         prep = self._prep
         if prep is None or prep[2] != self.packed_weight_codes.data_ptr():
             prep = self._prepare()
+            self._fp8_mult = None
         if prep[3] != x2.device:
             raise RuntimeError("x and the layer's buffers must be on the same device")
+        if self.fp8_operands:
+            if self.group_size != 64:
+                raise ValueError("fp8_operands needs group_size 64")
+            if self._fp8_mult is None:          # (reads the metadata back once per layer)
+                self._fp8_mult = ops.fp8_weight_multiplier(self.weight_codebook, self.weight_center, self.weight_scale,
+                                                           self.weight_code_sum)
+            t = prep[0]
+            y = ops.linear_otf_fp8(x2, t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7], self.bits,
+                                   out_dtype=self.out_dtype, w_mult=self._fp8_mult)
+            return y.reshape(*original_shape[:-1], self.out_features)
         ws = getattr(self, "_x_hat_buffer", None)       # a buffer the model owns (packed_convert.share_buffers)
         if ws is None or ws.numel() < x2.numel() or ws.device != x2.device:
             ws = _workspace(x2.device, x2.numel())

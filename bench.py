@@ -65,6 +65,9 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bs1", action="store_true")
     ap.add_argument("--no-model", action="store_true", help="skip the model_forward block (whole ViT forward)")
+    ap.add_argument("--fp8", action="store_true",
+                    help="also time the same step with FP8 operands (ops.linear_otf_fp8: not the reference's numerics; "
+                         "reported in a block of its own, never as `value`)")
     ap.add_argument("--eager", action="store_true",
                     help="launch every kernel from Python instead of replaying one HIP graph per step")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -468,6 +471,44 @@ def model_forward(model, bits, batches, steps, warmup, dev):
     return out
 
 
+def fp8_step(layers, inputs, m, steps, warmup):
+    """The same step with the operands rounded to FP8 (stage 1 -> FP8, stage 2 -> FP8, the vendor library's FP8 GEMM with
+    fp32 accumulation): ms/step under a HIP graph, and how far its outputs are from the fp16 path's."""
+    import torch
+    from arcq_vit_amd import ops
+    dev = layers[0].packed.device
+    x8 = torch.empty(m * max(l.k for l in layers), dtype=torch.float8_e4m3fn, device=dev)
+    w8 = torch.empty(max(l.n * l.k for l in layers), dtype=torch.float8_e4m3fn, device=dev)
+    mults = [ops.fp8_weight_multiplier(l.cb, l.center, l.scale, l.code_sum) for l in layers]
+
+    def run(l, mult):
+        x = inputs[l.name.rsplit(".", 1)[-1]]
+        return ops.linear_otf_fp8(x, l.thr, l.cb, l.packed, l.cb, l.center, l.scale, l.code_sum, l.bias, l.bits,
+                                  w_mult=mult, x8_ws=x8, w8_ws=w8)
+
+    def step():
+        for l, mult in zip(layers, mults):
+            run(l, mult)
+
+    step()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step()
+    t = time_loop(g.replay, steps, warmup)
+    rel = []
+    for l, mult in list(zip(layers, mults))[:4]:          # the four layer shapes of the first block
+        x = inputs[l.name.rsplit(".", 1)[-1]]
+        y16 = ops.linear_otf(x, l.thr, l.cb, l.packed, l.cb, l.center, l.scale, l.code_sum, l.bias, l.bits, 64,
+                             out_dtype=torch.float32)
+        rel.append(float((run(l, mult).float() - y16).norm() / y16.norm()))
+    flops = sum(2.0 * m * l.n * l.k for l in layers)
+    return {"ms_per_step": t / steps * 1e3, "tflops_whole_step": flops * steps / t / 1e12,
+            "relative_distance_from_fp16_path": rel,
+            "note": "operands rounded to OCP E4M3 (3 mantissa bits): NOT the reference's numerics; stage 3 is the vendor "
+                    "library's FP8 GEMM (torch._scaled_mm), stages 1 and 2 are this library's kernels"}
+
+
 def kernel_note(name):
     if name == "otf_rows_kernel":
         return ("the WHOLE layer in one launch: stage 1 of 64 rows into LDS, the fp16 weights reconstructed cooperatively "
@@ -566,6 +607,8 @@ def main():
         out["bs1"]["cold_cache"] = cold_cache_bs1(args.model, args.bits, max(args.steps, 50), max(args.warmup, 10), dev)
     if not args.no_model:
         out["model_forward"] = model_forward(args.model, args.bits, sorted({1, args.batch}), args.steps, args.warmup, dev)
+    if args.fp8:
+        out["fp8_operands"] = fp8_step(layers, inputs, res["M"], args.steps, args.warmup)
     out["launch_mode"] = "eager" if args.eager else "hip_graph_per_step"
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(layers, inputs, args.batch)

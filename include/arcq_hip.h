@@ -265,6 +265,20 @@ int arcq_linear_otf_static(const void *x, int x_dtype, const float *a_thresholds
                            const float *bias, void *y, int y_dtype,
                            int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
 
+/* The two operands of the layer rounded to FP8 (OCP E4M3, round to nearest even, clamped to +-448) instead of fp16, for
+ * a product on FP8 matrix units: the low-precision formulation that EXT/arcq_linear_kernel.cu:22-202 points at.  They
+ * have no counterpart in the reference and do NOT reproduce its numbers (3 mantissa bits per operand where fp16 has
+ * 10); codes, mu, s and the fp32 reconstruction are those of arcq_act_quant / arcq_weight_dequant.
+ *   arcq_act_quant_fp8:      x8[rows, cols]  = fp8(x_hat), row-major, cols a multiple of 64 (group size 64 only)
+ *   arcq_weight_dequant_fp8: w8[N, K]        = fp8(w_mult * w_hat), row-major; w_mult > 0, a power of two chosen by the
+ *                                              caller so that the weights fall into FP8's normal range (2^-6 .. 448)
+ * The product y = (x8 w8^T) / w_mult + bias is a plain FP8 GEMM with fp32 accumulation, left to a GEMM library. */
+int arcq_act_quant_fp8(const void *x, int x_dtype, const float *thresholds, const float *codebook, void *x8,
+                       int64_t rows, int64_t cols, int bits, float eps, void *stream);
+int arcq_weight_dequant_fp8(const uint8_t *packed, const float *codebook, const float *center, const float *scale,
+                            const float *code_sum, void *w8, int64_t N, int64_t K, int bits, int group_size,
+                            float w_mult, void *stream);
+
 /* Kernels arcq_linear_otf_ws runs after stage 1 for these sizes: "gemm_slab8_kernel", or, with the weights rebuilt
  * in the stage-1 launch and copied by the GEMM, "gemm_slab8_kernel<copy>" or "gemm_pair_kernel" (two row blocks per
  * wave), when it takes the block layout, else arcq_linear_fused_ws_kernel's answer.  A profiling aid with no

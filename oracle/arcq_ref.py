@@ -421,3 +421,24 @@ def gelu_f64_np(x) -> np.ndarray:
     x = np.asarray(x, dtype=np.float64)
     erf = np.vectorize(math.erf, otypes=[np.float64])
     return 0.5 * x * (1.0 + erf(x / math.sqrt(2.0)))
+
+
+# --------------------------------------------------------------------------
+# FP8 operands (the low-precision formulation of the layer; no reference counterpart)
+# --------------------------------------------------------------------------
+FP8_E4M3_MAX = 448.0
+
+
+def fp8_e4m3_np(v) -> np.ndarray:
+    """Round float values to OCP FP8 E4M3 (1 sign, 4 exponent bits with bias 7, 3 mantissa bits; no infinities,
+    largest finite value 448): clamp to +-448, then round to nearest, ties to the even mantissa.  Normal numbers
+    2^e (1 + m/8), e = -6 .. 8; below 2^-6 the spacing stays 2^-9 (subnormals).  Returns float32 holding the
+    rounded values exactly.  Pinned in tests by hand-computed ties and against torch's ``float8_e4m3fn`` cast."""
+    a = np.clip(np.asarray(v, dtype=np.float64), -FP8_E4M3_MAX, FP8_E4M3_MAX)
+    mag = np.abs(a)
+    e = np.floor(np.log2(np.where(mag > 0, mag, 1.0)))
+    e = np.clip(e, -6, 8)
+    step = np.exp2(e - 3)                      # spacing inside the binade (2^-9 for everything below 2^-6)
+    q = np.rint(mag / step)                    # numpy rounds halves to even
+    out = np.sign(a) * q * step                # (a mantissa carried to 16 steps is the next binade's first value)
+    return out.astype(np.float32)

@@ -356,3 +356,24 @@ def test_gelu_reference_matches_torch(oracle):
     x = torch.linspace(-8, 8, 4001, dtype=torch.float64)
     want = torch.nn.functional.gelu(x).numpy()
     assert np.max(np.abs(oracle.gelu_f64_np(x.numpy()) - want)) < 1e-14
+
+
+def test_fp8_e4m3_rounding_known_answers(oracle):
+    """The oracle's FP8 (OCP E4M3) rounding against values worked out by hand -- ties go to the even mantissa, the
+    subnormal spacing is 2^-9, everything beyond 448 saturates -- and against torch's float8_e4m3fn cast, an
+    independent implementation, on values across the range."""
+    f = oracle.fp8_e4m3_np
+    got = f([1.0, 1.0625, 1.1875, 1.3125, 449.0, -1000.0, 464.0, 0.001, 2.0 ** -10, 3 * 2.0 ** -10, 2.0 ** -6 * (1 + 1 / 16),
+             240.0, 15.5, -0.3])
+    want = [1.0, 1.0, 1.25, 1.25, 448.0, -448.0, 448.0, 2.0 ** -9, 0.0, 2.0 ** -8, 2.0 ** -6, 240.0, 16.0, -0.3125]
+    assert np.array_equal(got, np.asarray(want, dtype=np.float32))
+    g = np.random.default_rng(5)
+    v = np.concatenate([g.normal(size=50000) * 3, g.normal(size=50000) * 0.01, g.uniform(-448, 448, 50000)]).astype(np.float32)
+    assert np.array_equal(f(v), torch.from_numpy(v).to(torch.float8_e4m3fn).float().numpy())
+    # every FP8 value is a fixed point, and the rounding never moves a value by more than half a step
+    pos = [m * 2.0 ** -9 for m in range(1, 8)] + [2.0 ** e * (1 + m / 8) for e in range(-6, 9) for m in range(8)][:-1]
+    grid = np.asarray([-p for p in reversed(pos)] + [0.0] + pos, dtype=np.float32)       # all 253 finite values
+    assert grid.size == 253 and grid[-1] == 448.0 and np.array_equal(f(grid), grid)
+    assert set(np.unique(f(np.linspace(-448, 448, 400001))).tolist()) <= set(grid.tolist())      # and nothing else comes out
+    x = g.uniform(2.0 ** -6, 448, 10000)
+    assert np.all(np.abs(f(x) - x) <= np.exp2(np.floor(np.log2(x)) - 4) * (1 + 1e-12))
