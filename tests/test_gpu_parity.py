@@ -763,6 +763,61 @@ def test_index_linears_bitexact(cuda, oracle, bits, m, n, k):
         assert np.array_equal(_np(got8), want8)
 
 
+def _index_case(oracle, m, n, k, bits, gs, seed):
+    cb, packed_w, wc, ws, wcs = _packed_weight(oracle, n, k, bits, seed, gs=gs)
+    _, thr = _cb(bits)
+    x = synth.make_activation(m, k, seed)
+    bias = synth.make_bias(n, seed)
+    xa = oracle.act_quant_c(x.numpy(), thr, cb, bits, gs)
+    table = (cb.view(-1, 1) * (cb * 1.25).view(1, -1)).float().contiguous()      # asymmetric on purpose
+    wcodes = oracle.unpack_codes_u8_c(packed_w.numpy(), bits, k)
+    return xa, packed_w.numpy(), wcodes, wc, ws, wcs, table, bias
+
+
+def _index_both(cuda, oracle, case, bits, gs, k, n, rows=None):
+    """Run both index-space formats on the GPU on all rows and compare the rows in ``rows`` (all if None) with the
+    oracle evaluated on those rows only."""
+    xa, packed_w, wcodes, wc, ws, wcs, table, bias = case
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(cuda) if isinstance(a, np.ndarray) else a.to(cuda)
+    sel = slice(None) if rows is None else rows
+    got = ops.arcq_linear_forward(d(xa["packed"]), d(xa["center"]), d(xa["scale"]), d(xa["code_sum"]),
+                                  d(packed_w), d(wc), d(ws), d(wcs), d(table), d(bias), bits, gs, k, n)
+    want = oracle.linear_forward_packed_c(xa["packed"][sel], xa["center"][sel], xa["scale"][sel], xa["code_sum"][sel],
+                                          packed_w, wc, ws, wcs, table.numpy(), bias.numpy(), bits, gs, k, n)
+    assert got.dtype == torch.float32 and np.array_equal(_np(got)[sel], want)
+    got8 = ops.arcq_linear_forward_u8(d(xa["codes"]), d(xa["center"]), d(xa["scale"]), d(xa["code_sum"]),
+                                      d(wcodes), d(wc), d(ws), d(wcs), d(table), d(bias), gs)
+    want8 = oracle.linear_forward_u8_c(xa["codes"][sel], xa["center"][sel], xa["scale"][sel], xa["code_sum"][sel],
+                                       wcodes, wc, ws, wcs, table.numpy(), bias.numpy(), gs)
+    assert np.array_equal(_np(got8)[sel], want8)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("m,n,k", [(2100, 300, 384), (8195, 71, 128)])
+def test_index_linears_bitexact_many_tiles(cuda, oracle, bits, m, n, k):
+    """Launches of more than 512 tiles of 16 rows x 64 outputs give every thread four outputs (a different
+    instantiation from the one small launches take); rows % 16 and outputs % 64 are ragged on purpose."""
+    assert ((m + 15) // 16) * ((n + 63) // 64) > 512
+    _index_both(cuda, oracle, _index_case(oracle, m, n, k, bits, 64, 43), bits, 64, k, n)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_index_linears_bitexact_batch64_sampled_rows(cuda, oracle, bits):
+    """A DeiT-S projection at batch 64 (12 608 x 384 x 384: 4 728 tiles); the oracle is evaluated on 96 sampled rows
+    that include the first and last tile and the ragged tail."""
+    m, n, k = 12608, 384, 384
+    rng = np.random.default_rng(5)
+    rows = np.unique(np.concatenate([np.arange(0, 17), np.arange(m - 17, m), rng.integers(0, m, 62)]))
+    _index_both(cuda, oracle, _index_case(oracle, m, n, k, bits, 64, 45), bits, 64, k, n, rows=rows)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("gs,m,n,k", [(32, 70, 45, 96), (128, 37, 50, 256), (16, 19, 33, 48)])
+def test_index_linears_bitexact_other_group_sizes(cuda, oracle, bits, gs, m, n, k):
+    """Group sizes other than 64 run the one-thread-per-output kernels."""
+    _index_both(cuda, oracle, _index_case(oracle, m, n, k, bits, gs, 47), bits, gs, k, n)
+
+
 # ------------------------------------------------------------------------------------------------
 # argument errors surface as RuntimeError with the reference's wording
 # ------------------------------------------------------------------------------------------------
