@@ -181,15 +181,55 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
         return linear_otf_impl(a->x, a->x_dtype, a->a_thresholds, a->a_codebook, a->packed_w, a->w_codebook, a->w_center,
                                a->w_scale, a->w_code_sum, a->bias, a->x_hat_ws, a->w_hat_ws, true, a->y, a->y_dtype, a->M,
                                a->N, a->K, a->bits, a->group_size, stream);
-    if (a->group_size != 64 || !arcq::bits_ok(a->bits) || !arcq::otf_blocked_pays(a->M, a->N, a->K))
-        return arcq::fail(ARCQ_ERR_UNSUPPORTED,
-                          "arcq_linear_otf_ex: the fused options need group_size 64, bits 2/3/4 and at least 512 rows "
-                          "(got M=%lld K=%lld group_size=%d)", static_cast<long long>(a->M), static_cast<long long>(a->K),
-                          a->group_size);
+    if (a->group_size != 64 || !arcq::bits_ok(a->bits))
+        return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: the fused options need group_size 64 and bits 2/3/4 "
+                          "(got group_size=%d bits=%d)", a->group_size, a->bits);
     if (!a->x_hat_ws) return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf_ex: x_hat_ws must not be NULL");
     if (a->x_hat_ws == a->x) return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: x_hat_ws must not alias x");
     if (a->residual && !arcq::aligned(a->residual, 16))
         return arcq::fail(ARCQ_ERR_ALIGN, "arcq_linear_otf_ex: residual must be 16-byte aligned");
+    const bool want_ln = a->producer == ARCQ_PRODUCER_LAYERNORM;
+    if (want_ln && (!a->ln_weight || !a->ln_bias || !arcq::aligned(a->ln_weight, 16) || !arcq::aligned(a->ln_bias, 16)))
+        return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf_ex: ln_weight and ln_bias must be 16-byte aligned fp32 [K] tensors");
+    // A few hundred rows (batch 1): the whole layer, LayerNorm and post-operations included, in the one launch of the
+    // small-M kernel wherever that kernel can run (always with a LayerNorm: it is the only small-M kernel that has
+    // one); else stage 1 row-major + the split-K kernel with the post-operations in its epilogue.
+    if (a->M > 0 && a->M < 512 && a->N > 0 && a->N < (int64_t(1) << 30) && a->K >= 64 && a->K % 64 == 0) {
+        if (!a->x || !a->a_thresholds || !a->a_codebook || !a->packed_w || !a->w_codebook || !a->w_center || !a->w_scale ||
+            !a->w_code_sum || !a->y)
+            return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf_ex: NULL tensor pointer");
+        if ((a->x_dtype != ARCQ_F16 && a->x_dtype != ARCQ_F32) || (a->y_dtype != ARCQ_F16 && a->y_dtype != ARCQ_F32))
+            return arcq::fail(ARCQ_ERR_DTYPE, "arcq_linear_otf_ex: x and y must be float16 or float32");
+        if (!arcq::aligned(a->x, 16) || !arcq::aligned(a->x_hat_ws, 16) || !arcq::aligned(a->y, 16) ||
+            !arcq::aligned(a->packed_w, 16))
+            return arcq::fail(ARCQ_ERR_ALIGN, "arcq_linear_otf_ex: x, x_hat_ws, y and packed_w must be 16-byte aligned");
+        const char *e = arcq::tuning().otf_fused;
+        const bool one_launch = want_ln ? arcq::otf_small_supported(a->M, a->N, a->K, true)
+                                        : (!(e && e[0] == '0') && arcq::otf_small_supported(a->M, a->N, a->K, e && e[0] == '2'));
+        if (one_launch) {
+            arcq::OtfSmallArgs s{a->x, a->x_dtype == ARCQ_F16, a->a_thresholds, a->a_codebook, a->packed_w, a->w_codebook,
+                                 a->w_center, a->w_scale, a->w_code_sum, a->bias, a->x_hat_ws, a->y, a->y_dtype == ARCQ_F16,
+                                 static_cast<int>(a->M), static_cast<int>(a->N), static_cast<int>(a->K), a->bits, 1.0e-6f};
+            if (want_ln) s.ln_weight = a->ln_weight, s.ln_bias = a->ln_bias, s.ln_eps = a->ln_eps;
+            s.residual = a->residual;
+            s.gelu = a->activation == ARCQ_ACT_GELU;
+            arcq::launch_otf_small(s, static_cast<hipStream_t>(stream));
+            return arcq::launch_status("arcq_linear_otf_ex");
+        }
+        if (want_ln)
+            return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: below 512 rows the fused LayerNorm needs in_features <= 1536");
+        const int rc = arcq_act_quant(a->x, a->x_dtype, a->a_thresholds, a->a_codebook, nullptr, nullptr, nullptr, nullptr,
+                                      nullptr, a->x_hat_ws, ARCQ_F16, a->M, a->K, a->bits, 64, 1.0e-6f, stream);
+        if (rc != ARCQ_OK) return rc;
+        return arcq::linear_fused_post(a->x_hat_ws, a->packed_w, a->w_codebook, a->w_center, a->w_scale, a->w_code_sum, a->bias,
+                                       a->y, a->y_dtype, a->M, a->N, a->K, a->bits, 64, stream, a->residual,
+                                       a->activation == ARCQ_ACT_GELU);
+    }
+    if (!arcq::otf_blocked_pays(a->M, a->N, a->K))
+        return arcq::fail(ARCQ_ERR_UNSUPPORTED,
+                          "arcq_linear_otf_ex: the fused options need in_features a positive multiple of 64 and a shape the "
+                          "block-layout kernels run (got M=%lld K=%lld)", static_cast<long long>(a->M),
+                          static_cast<long long>(a->K));
     if (a->w_hat_ws && a->x_dtype == ARCQ_F16 &&
         arcq::otf_rows_pays(a->M, a->N, a->K, a->producer == ARCQ_PRODUCER_LAYERNORM) && a->x && a->a_thresholds &&
         a->a_codebook && a->packed_w && a->w_codebook && a->w_center && a->w_scale && a->w_code_sum && a->y &&

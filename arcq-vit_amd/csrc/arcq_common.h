@@ -157,6 +157,17 @@ template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ __half from_float<__half>(float v) { return __float2half_rn(v); }
 
+// The exact (erf) GELU in fp32, (x * 0.5) * (1 + erf(x * sqrt(1/2))), with the fp32 rounding of the last product made
+// visible: without the barrier the compiler may fuse that product with a following float->half conversion into one
+// instruction that rounds the exact product once to fp16, which differs from round-to-fp32-then-fp16 (what an
+// elementwise kernel computing in fp32 stores) on rare ties.
+__device__ __forceinline__ float gelu_f32(float x)
+{
+    float v = (x * 0.5f) * (1.0f + erff(x * 0.70710678118654752440f));
+    asm("" : "+v"(v));
+    return v;
+}
+
 // Optional elementwise work on a GEMM's outputs after they have been rounded to the output type, each step rounding
 // to that type again -- the values separate elementwise kernels on the stored tensor would produce:
 //   gelu:     y = round(gelu(y)),  gelu(v) = (v * 0.5) * (1 + erf(v * sqrt(1/2)))    (the exact, erf-based GELU)
@@ -172,8 +183,7 @@ __device__ __forceinline__ void post_ops16(u32x4_store_t &v, const TOUT *res, bo
     if (gelu) {
 #pragma unroll
         for (int i = 0; i < n; ++i) {
-            const float x = to_float(e[i]);
-            e[i] = from_float<TOUT>((x * 0.5f) * (1.0f + erff(x * 0.70710678118654752440f)));
+            e[i] = from_float<TOUT>(gelu_f32(to_float(e[i])));
         }
     }
     if (res) {
@@ -189,6 +199,17 @@ __device__ __forceinline__ void post_ops16(u32x4_store_t &v, const TOUT *res, bo
         for (int i = 0; i < n; ++i) e[i] = from_float<TOUT>(to_float(e[i]) + to_float(r[i]));
     }
     __builtin_memcpy(&v, e, 16);
+}
+
+// The same two steps on one output value (the small-M kernels, whose threads hold a few consecutive outputs each).
+template <typename TOUT>
+__device__ __forceinline__ TOUT post_op1(TOUT v, const TOUT *res, bool gelu)
+{
+    if (gelu) {
+        v = from_float<TOUT>(gelu_f32(to_float(v)));
+    }
+    if (res) v = from_float<TOUT>(to_float(v) + to_float(*res));
+    return v;
 }
 
 }  // namespace arcq

@@ -15,8 +15,9 @@ struct GemmArgs {
     void *y;                 // [M,N]
     bool y_f16;
     int M, N, K, bits;
-    // Post-operations on the rounded outputs (arcq_common.h, post_ops16); only the block-layout kernels
-    // (launch_gemm_slab8, launch_gemm_pair) apply them, the entry points keep them away from the others.
+    // Post-operations on the rounded outputs (arcq_common.h, post_ops16 / post_op1); only the block-layout kernels
+    // (launch_gemm_slab8, launch_gemm_pair) and the small-M kernel (launch_gemm_splitk) apply them, the entry points
+    // keep them away from the others.
     const void *residual = nullptr;   // [M,N] of y's type, or nullptr
     bool gelu = false;
 };
@@ -50,6 +51,12 @@ int linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_w, con
 
 // Small-M kernel (64 x 64 tiles, K split across the waves of a workgroup); requires K >= 64.
 void launch_gemm_splitk(const GemmArgs &g, hipStream_t stream);
+// arcq_linear_fused with GELU / a residual ([M,N] of y's type) on the rounded outputs; with either set it needs the
+// small-M kernel's shapes (fewer than 512 rows, K >= 64) and reports ARCQ_ERR_UNSUPPORTED otherwise.
+int linear_fused_post(const void *x_hat, const uint8_t *packed_w, const float *w_codebook, const float *w_center,
+                      const float *w_scale, const float *w_code_sum, const float *bias, void *y, int y_dtype,
+                      int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream,
+                      const void *residual, bool gelu);
 
 // Whole on-the-fly layer in one launch (activation quantizer + split-K product) for M < 512.
 struct OtfSmallArgs {
@@ -63,6 +70,12 @@ struct OtfSmallArgs {
     bool y_f16;
     int M, N, K, bits;
     float eps;
+    // Optional work fused around the layer: a LayerNorm over the rows of x in front of stage 1 (fp32 weight / bias
+    // [K], 16-byte aligned; nullptr: none) and GELU / a residual ([M,N] of y's type) on the rounded outputs.
+    const float *ln_weight = nullptr, *ln_bias = nullptr;
+    float ln_eps = 0.0f;
+    const void *residual = nullptr;
+    bool gelu = false;
 };
 bool otf_small_supported(int64_t M, int64_t N, int64_t K, bool any_supported);
 void launch_otf_small(const OtfSmallArgs &a, hipStream_t stream);

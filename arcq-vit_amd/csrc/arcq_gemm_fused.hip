@@ -282,11 +282,12 @@ ARCQ_API const char *arcq_linear_fused_kernel(int64_t M, int64_t N, int64_t K)
     }
 }
 
-ARCQ_API int arcq_linear_fused(const void *x_hat,
-                               const uint8_t *packed_w, const float *w_codebook,
-                               const float *w_center, const float *w_scale, const float *w_code_sum,
-                               const float *bias, void *y, int y_dtype,
-                               int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
+// arcq_linear_fused, optionally with GELU / a residual on the rounded outputs; those are built into the small-M
+// kernel only (the large-M row-major kernels do not have them: callers with 512 rows or more use the block layout).
+int arcq::linear_fused_post(const void *x_hat, const uint8_t *packed_w, const float *w_codebook, const float *w_center,
+                            const float *w_scale, const float *w_code_sum, const float *bias, void *y, int y_dtype,
+                            int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream,
+                            const void *residual, bool gelu)
 {
     if (!bits_ok(bits)) return fail(ARCQ_ERR_BITS, "arcq_linear_fused: bits must be 2, 3, or 4");
     if (M < 0 || N < 0 || K < 0 || group_size <= 0) return fail(ARCQ_ERR_SHAPE, "arcq_linear_fused: bad sizes");
@@ -308,6 +309,15 @@ ARCQ_API int arcq_linear_fused(const void *x_hat,
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
     GemmArgs g{x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype == ARCQ_F16, m, n, k, bits};
+    if (residual || gelu) {
+        if (pick_kernel(M, N, K) != kSplitK)
+            return fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_fused: GELU / residual on row-major x_hat need fewer than 512 rows "
+                        "and in_features >= 64");
+        if (residual && !aligned(residual, 16))
+            return fail(ARCQ_ERR_ALIGN, "arcq_linear_fused: residual must be 16-byte aligned");
+        g.residual = residual;
+        g.gelu = gelu;
+    }
     switch (pick_kernel(M, N, K)) {
     case kSplitK: launch_gemm_splitk(g, st); break;
     case kSlab: launch_gemm_slab(g, st); break;
@@ -319,6 +329,16 @@ ARCQ_API int arcq_linear_fused(const void *x_hat,
             launch_out<float>(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, m, n, k, bits, st);
     }
     return launch_status("arcq_linear_fused");
+}
+
+ARCQ_API int arcq_linear_fused(const void *x_hat,
+                               const uint8_t *packed_w, const float *w_codebook,
+                               const float *w_center, const float *w_scale, const float *w_code_sum,
+                               const float *bias, void *y, int y_dtype,
+                               int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream)
+{
+    return linear_fused_post(x_hat, packed_w, w_codebook, w_center, w_scale, w_code_sum, bias, y, y_dtype, M, N, K, bits,
+                             group_size, stream, nullptr, false);
 }
 
 // Whether arcq_linear_fused_ws, given a workspace, rebuilds the weights into it and runs the copying slab kernel.

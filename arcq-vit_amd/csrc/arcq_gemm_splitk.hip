@@ -63,7 +63,8 @@ template <int BITS, typename TOUT, int NW, int RB, int CB>
 __global__ void __launch_bounds__(NW * 64)
 gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw, const float *__restrict__ cb,
                    const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
-                   const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K)
+                   const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K,
+                   const TOUT *residual, int gelu)
 {
     constexpr int L = 1 << BITS;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -202,11 +203,18 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
     const int gr = m0 + row, gc = n0 + col;
     if (gr < M && gc < N) {
         TOUT *dst = y + static_cast<int64_t>(gr) * N + gc;
+        // Optional GELU / residual on the rounded output (post_op1): what separate elementwise kernels would store.
+        const TOUT *res = residual ? residual + static_cast<int64_t>(gr) * N + gc : nullptr;
+        const bool post = res || gelu;
         constexpr int BYTES = E * static_cast<int>(sizeof(TOUT));
         if (gc + E <= N && (N % E) == 0 && BYTES % 8 == 0) {
             TOUT out[E];
 #pragma unroll
             for (int e = 0; e < E; ++e) out[e] = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
+            if (post) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) out[e] = post_op1<TOUT>(out[e], res ? res + e : nullptr, gelu != 0);
+            }
             if constexpr (BYTES % 16 == 0) {
 #pragma unroll
                 for (int b = 0; b < BYTES; b += 16)
@@ -218,7 +226,11 @@ gemm_splitk_kernel(const __half *__restrict__ a, const uint8_t *__restrict__ pw,
         } else {
 #pragma unroll
             for (int e = 0; e < E; ++e)
-                if (gc + e < N) dst[e] = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
+                if (gc + e < N) {
+                    TOUT o = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
+                    if (post) o = post_op1<TOUT>(o, res ? res + e : nullptr, gelu != 0);
+                    dst[e] = o;
+                }
         }
     }
 }
@@ -236,7 +248,8 @@ static void launch_splitk_rb(const GemmArgs &g, hipStream_t stream)
     allow_dynamic_lds<gemm_splitk_kernel<BITS, TOUT, NW, RB, CB>>(static_cast<int>(smem));
     const dim3 grid((g.N + kSkTile - 1) / kSkTile, (g.M + RT - 1) / RT);
     hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), smem, stream, static_cast<const __half *>(g.x_hat), g.pw, g.cb, g.wc,
-                       g.ws, g.wcs, g.bias, static_cast<TOUT *>(g.y), g.M, g.N, g.K);
+                       g.ws, g.wcs, g.bias, static_cast<TOUT *>(g.y), g.M, g.N, g.K, static_cast<const TOUT *>(g.residual),
+                       g.gelu ? 1 : 0);
 }
 
 template <int BITS, typename TOUT>

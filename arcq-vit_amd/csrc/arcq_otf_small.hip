@@ -98,7 +98,9 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
                  const uint8_t *__restrict__ pw, const float *__restrict__ w_cb,
                  const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
                  const float *__restrict__ bias, __half *__restrict__ x_hat_ws, TOUT *__restrict__ y,
-                 int M, int N, int K, float eps, int tile_bytes, int partial_off)
+                 int M, int N, int K, float eps, int tile_bytes, int partial_off,
+                 const float *__restrict__ ln_w, const float *__restrict__ ln_b, float ln_eps, int ln_off,
+                 const TOUT *residual, int gelu)
 {
     constexpr int L = 1 << BITS;
     constexpr int RT = 32 * RB;
@@ -154,11 +156,16 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     // each lane holding EL consecutive inputs.  With two lanes per group the per-lane instruction chain, which is
     // what a launch this small waits for, is half as long (arcq_act_quant_core.h); it is used while the row tile is
     // at most eight such tiles (K <= 512 for 32 rows), i.e. while it does not add a round.
-    constexpr int EL = 64 / LPG, GPT = 64 / LPG;
+    // With a LayerNorm in front (ln_w != nullptr) a wave tile holds whole rows only (floor(slots / G) rows, the
+    // remaining slots idle), so that a row's sums never leave the wave.
+    constexpr int EL = 64 / LPG, SLOTS = 64 / LPG;
     const int groups = RT * G;
+    const int gpt = ln_w ? (SLOTS / G) * G : SLOTS;      // groups per wave tile
+    const int slot = lane / LPG;
+    auto tile_group = [&](int t) { return slot < gpt ? t * gpt + slot : groups; };      // `groups`: this lane idles
     OsGroupRegs<TIN, EL> in;
-    auto fetch_x = [&](int t0) {
-        const int f = t0 + lane / LPG;
+    auto fetch_x = [&](int t) {
+        const int f = tile_group(t);
         const int row = f / G, g = f - row * G;
         os_fetch_group<TIN, EL>(x + static_cast<int64_t>(min(m0 + row, M - 1)) * K + g * 64 + (lane % LPG) * EL,
                                f < groups && m0 + row < M, in);
@@ -168,14 +175,77 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     auto stats = [&]() {
         os_convert_group<TIN, EL>(in, xv);
     };
+    // LayerNorm of the rows of tile t, on xv in place: arithmetic and summation order of the stand-alone LayerNorm +
+    // stage-1 kernel (act_quant_rows_ln_kernel): every half group of 32 values is summed serially, a row's 2 G
+    // partial sums are added in order, mean = sum / K, var = the same sum over (x - mean)^2, / K,
+    // y = ((x - mean) * (1 / sqrt(var + eps))) * weight + bias, rounded to x's type.  The partial sums of a wave's
+    // rows meet in a wave-private piece of LDS (LDS operations of one wave execute in order: no barrier needed).
+    float *ln_part = reinterpret_cast<float *>(smem + ln_off) + wave * 128;
+    auto layernorm = [&](int t) {
+        constexpr int H = EL / 32;                    // half groups per lane
+        const int f = tile_group(t);
+        const bool act = f < groups;
+        const int fl = act ? slot : 0;                // idle lanes read the first row's sums and write nothing
+        const int rl = fl / G, g = fl - rl * G;
+        const int base = rl * 2 * G;
+        const int mine = base + 2 * g + (LPG == 2 ? (lane & 1) : 0);
+        auto row_total = [&](const float (&ps)[H]) {
+            if (act) {
+#pragma unroll
+                for (int h = 0; h < H; ++h) ln_part[mine + h] = ps[h];
+            }
+            __builtin_amdgcn_wave_barrier();
+            float acc = 0.0f;
+            for (int i = 0; i < 2 * G; ++i) acc += ln_part[base + i];
+            __builtin_amdgcn_wave_barrier();
+            return acc;
+        };
+        const float fk = static_cast<float>(K);
+        float ps[H];
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            float a = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 32; ++j) a += xv[32 * h + j];
+            ps[h] = a;
+        }
+        const float mean = row_total(ps) / fk;
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            float q = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 32; ++j) {
+                xv[32 * h + j] -= mean;
+                const float sq = xv[32 * h + j] * xv[32 * h + j];
+                q += sq;
+            }
+            ps[h] = q;
+        }
+        const float var_row = row_total(ps) / fk;
+        const float rstd = 1.0f / sqrtf(var_row + ln_eps);
+        const float4 *gp = reinterpret_cast<const float4 *>(ln_w + g * 64 + (lane % LPG) * EL);
+        const float4 *bp = reinterpret_cast<const float4 *>(ln_b + g * 64 + (lane % LPG) * EL);
+#pragma unroll
+        for (int j4 = 0; j4 < EL / 4; ++j4) {
+            const float4 gv = gp[j4], bv = bp[j4];
+            const float g4[4] = {gv.x, gv.y, gv.z, gv.w}, b4[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float tt = xv[4 * j4 + e] * rstd;
+                const float u = tt * g4[e];
+                if constexpr (sizeof(TIN) == 2) xv[4 * j4 + e] = __half2float(__float2half_rn(u + b4[e]));
+                else xv[4 * j4 + e] = u + b4[e];
+            }
+        }
+    };
     // Wave w owns the tiles w, w + 8, ... of the row tile.  With fewer than eight tiles the waves without one build
     // the lookup tables while the others take their statistics, and one barrier joins the two halves; otherwise all
     // eight waves build the tables between the two halves of their first tile.
-    const int n_tiles = (groups + GPT - 1) / GPT;
+    const int n_tiles = (groups + gpt - 1) / gpt;
     const bool spare_waves = n_tiles < kOsWaves;
     const int tile_waves = spare_waves ? n_tiles : kOsWaves;
     const bool has_tile = wave < n_tiles;
-    if (has_tile) fetch_x(wave * GPT);
+    if (has_tile) fetch_x(wave);
     float th[L - 1], cbv[L];
     load_quant_params<BITS>(a_thr, a_cb, th, cbv);
     const BucketScale bq = pick_bucket_scale<BITS>(th);
@@ -187,7 +257,8 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     }
     if (has_tile) {
         stats();
-        if (wave + kOsWaves < n_tiles) fetch_x((wave + kOsWaves) * GPT);      // the next tile's inputs, one round ahead
+        if (wave + kOsWaves < n_tiles) fetch_x(wave + kOsWaves);      // the next tile's inputs, one round ahead
+        if (ln_w) layernorm(wave);
         if constexpr (LPG == 1) group_stats64(xv, eps, mu, var, s);
         else group_stats32x2(xv, eps, mu, var, s);
     }
@@ -199,11 +270,12 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     for (int t = wave; t < n_tiles; t += kOsWaves) {
         if (t != wave) {                       // later tiles of this wave: their inputs were requested a round ago
             stats();
-            if (t + kOsWaves < n_tiles) fetch_x((t + kOsWaves) * GPT);
+            if (t + kOsWaves < n_tiles) fetch_x(t + kOsWaves);
+            if (ln_w) layernorm(t);
             if constexpr (LPG == 1) group_stats64(xv, eps, mu, var, s);
             else group_stats32x2(xv, eps, mu, var, s);
         }
-        const int f = t * GPT + lane / LPG;
+        const int f = tile_group(t);
         const int row = f / G, g = f - row * G;
         const bool valid = f < groups && m0 + row < M;
         float sum_codes;
@@ -321,11 +393,18 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     const int gr = m0 + row, gc = n0 + col;
     if (gr < M && gc < N) {
         TOUT *dst = y + static_cast<int64_t>(gr) * N + gc;
+        // Optional GELU / residual on the rounded output (post_op1): what separate elementwise kernels would store.
+        const TOUT *res = residual ? residual + static_cast<int64_t>(gr) * N + gc : nullptr;
+        const bool post = res || gelu;
         constexpr int BYTES = E * static_cast<int>(sizeof(TOUT));
         if (gc + E <= N && (N % E) == 0 && BYTES % 8 == 0) {
             TOUT out[E];
 #pragma unroll
             for (int e = 0; e < E; ++e) out[e] = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
+            if (post) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) out[e] = post_op1<TOUT>(out[e], res ? res + e : nullptr, gelu != 0);
+            }
             if constexpr (BYTES % 16 == 0) {
 #pragma unroll
                 for (int b = 0; b < BYTES; b += 16)
@@ -337,7 +416,11 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
         } else {
 #pragma unroll
             for (int e = 0; e < E; ++e)
-                if (gc + e < N) dst[e] = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
+                if (gc + e < N) {
+                    TOUT o = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
+                    if (post) o = post_op1<TOUT>(o, res ? res + e : nullptr, gelu != 0);
+                    dst[e] = o;
+                }
         }
     }
 }
@@ -353,16 +436,21 @@ static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
     const int xhat_bytes = RT * os_row_pitch(G);
     const int partial_bytes = kOsWaves * RT * kOsRedPitch;
     const int tile_bytes = xhat_bytes;
+    // (lookup tables, per-wave flags, and -- with a LayerNorm in front -- 128 floats per wave for the rows' partial sums)
     const size_t tables = 2 * L * 64 * sizeof(float) + (kMaxBuckets + 64) * sizeof(Bucket) + 64;
+    const size_t ln_bytes = a.ln_weight ? kOsWaves * 128 * sizeof(float) : 0;
     // Both regions side by side while they fit 160 KB of LDS; else the partial tiles reuse the x_hat tile's space.
-    const int partial_off = (tile_bytes + partial_bytes + tables <= 160 * 1024) ? tile_bytes : 0;
-    const size_t smem = (partial_off ? tile_bytes + partial_bytes : (tile_bytes > partial_bytes ? tile_bytes : partial_bytes)) + tables;
+    const int partial_off = (tile_bytes + partial_bytes + tables + ln_bytes <= 160 * 1024) ? tile_bytes : 0;
+    const size_t front = partial_off ? tile_bytes + partial_bytes : (tile_bytes > partial_bytes ? tile_bytes : partial_bytes);
+    const int ln_off = static_cast<int>(front + tables);
+    const size_t smem = front + tables + ln_bytes;
     auto kernel = otf_small_kernel<TIN, BITS, TOUT, RB, LPG, CB>;
     allow_dynamic_lds<otf_small_kernel<TIN, BITS, TOUT, RB, LPG, CB>>(160 * 1024);      // (the size varies with K: allow the CU's whole LDS)
     const dim3 grid((a.N + kOsCols - 1) / kOsCols, (a.M + RT - 1) / RT);
     hipLaunchKernelGGL(kernel, grid, dim3(kOsWaves * 64), smem, stream, static_cast<const TIN *>(a.x), a.a_thr, a.a_cb,
                        a.pw, a.w_cb, a.wc, a.ws, a.wcs, a.bias, static_cast<__half *>(a.x_hat_ws),
-                       static_cast<TOUT *>(a.y), a.M, a.N, a.K, a.eps, tile_bytes, partial_off);
+                       static_cast<TOUT *>(a.y), a.M, a.N, a.K, a.eps, tile_bytes, partial_off, a.ln_weight, a.ln_bias,
+                       a.ln_eps, ln_off, static_cast<const TOUT *>(a.residual), a.gelu ? 1 : 0);
 }
 
 template <typename TIN, int BITS, typename TOUT>

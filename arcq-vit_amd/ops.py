@@ -385,7 +385,9 @@ def linear_otf_ex(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch
                   x_hat_ws: Optional[torch.Tensor] = None, w_hat_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``residual + gelu(linear(stage1(LayerNorm(x))))`` with the optional parts fused into the layer's two launches
     (``arcq_linear_otf_ex``): ``layernorm = (weight, bias, eps)`` or None, ``residual`` ``[M, N]`` of ``out_dtype`` or
-    None.  Raises ``RuntimeError`` where the library does not fuse (fewer than 512 rows, K > 1024 with LayerNorm)."""
+    None.  Below 512 rows the whole layer with its options is one launch (or stage 1 + the split-K kernel with the
+    GELU / residual in its epilogue); from 512 rows on the block-layout path.  Raises ``RuntimeError`` where the
+    library does not fuse (LayerNorm with K > 1024 from 512 rows on, K > 1536 below)."""
     _check(x.is_cuda and packed_w.is_cuda, "x and packed_w must be CUDA tensors")
     _check(x.dim() == 2, "x must have shape [M, K]")
     _check_bits(bits)

@@ -2,14 +2,18 @@
 benchmarks), constructor and buffers as FQ/arcq_packed_on_the_fly.py:93-135.
 
 Reference forward (:137-161): fp16 copy of x -> Triton quantize+reconstruct in place -> Triton
-unpack of the whole weight into an fp16 buffer in HBM -> cuBLAS ``F.linear``.  Here: one HIP
-stage-1 kernel writes x_hat (fp16) into a workspace, and one HIP kernel streams the packed
-codes, rebuilds the weight tile by tile in LDS and feeds fp16 MFMA; by default the dense weight
-never exists in HBM.  ``_weight_buffer`` (the flat fp16 scratch the reference's benchmark shares
-between all layers, scripts/benchmark_arcq_on_the_fly.py:182-191, read at :148-158) is honoured as
-an optional workspace: when it is set and the shape is one where rebuilding the weight once beats
-rebuilding it per row tile, the library reconstructs the weight into it and the GEMM copies from
-there; the result is bit-identical either way.
+unpack of the whole weight into an fp16 buffer in HBM -> cuBLAS ``F.linear``.  Here the layer is one
+or two HIP launches (``arcq_linear_otf_ws`` / ``arcq_linear_otf_ex``): stage 1 writes x_hat (fp16)
+into a workspace or keeps it in LDS, and the fused unpack + fp16 MFMA GEMM follows.  Where the
+dense weight lives depends on ``_weight_buffer`` (the flat fp16 scratch the reference's benchmark
+shares between all layers, scripts/benchmark_arcq_on_the_fly.py:182-191, read at :148-158):
+  * not set: the GEMM kernel rebuilds the weight tile by tile in LDS; the dense weight never exists
+    in HBM;
+  * set (what ``packed_convert.share_buffers`` and ``bench.py`` do): from 512 rows on the fp16
+    weight is reconstructed into it inside the layer's first (or only) launch and the GEMM reads it
+    from there, i.e. it does pass through memory (L2-resident, a few MB) -- the reference's
+    unpack-then-GEMM order without a launch of its own; below 512 rows it is not used.
+The result is bit-identical either way.
 
 Differences from the reference module that a caller can observe (all on the side of more accuracy;
 for these cases "same indices as the reference" is not pinned by any test):
@@ -141,9 +145,9 @@ class ARCQPackedLinearOnTheFly(nn.Module):
                 residual: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``residual + activation(linear(stage1(layernorm(x))))``.  The three optional parts (the LayerNorm in front
         of the layer, ``activation="gelu"`` and the skip connection behind it, as they surround the block linears in
-        timm's ``Block``, FQ/timm_quant_models.py:63-121) are fused into the layer's two launches where the library
-        can (512 rows or more, group size 64, K <= 1024 for the LayerNorm) and run as separate torch operations
-        otherwise; without them this is the reference module's forward."""
+        timm's ``Block``, FQ/timm_quant_models.py:63-121) are fused into the layer's launches where the library can
+        (group size 64; for the LayerNorm K <= 1024 from 512 rows on and K <= 1536 below) and run as separate torch
+        operations otherwise; without them this is the reference module's forward."""
         original_shape = x.shape
         if original_shape[-1] != self.in_features:
             raise ValueError(f"expected last dim {self.in_features}, got {original_shape[-1]}")
@@ -157,8 +161,9 @@ class ARCQPackedLinearOnTheFly(nn.Module):
         x2 = x2.contiguous()
         m = x2.shape[0]
         extras = layernorm is not None or activation is not None or residual is not None
-        fuse = (extras and not self.fp8_operands and m >= 512 and self.group_size == 64 and self.in_features % 64 == 0
-                and (layernorm is None or (self.in_features <= 1024 and layernorm.elementwise_affine
+        fuse = (extras and not self.fp8_operands and m > 0 and self.group_size == 64 and self.in_features % 64 == 0
+                and (layernorm is None or (self.in_features <= (1024 if m >= 512 else 1536)
+                                           and layernorm.elementwise_affine
                                            and tuple(layernorm.normalized_shape) == (self.in_features,))))
         if extras and not fuse:          # separate operations around the plain layer
             if layernorm is not None:

@@ -380,6 +380,74 @@ def cold_cache_bs1(model, bits, steps, warmup, dev, footprint_bytes=512 << 20):
             "hbm_frac": nbytes * n / t / 1e9 / PEAK_HBM_GBS}
 
 
+def chained_step(model, bits, batch, steps, warmup, dev):
+    """The packed linears of the model as a dependency chain: every layer reads what the layer before it wrote (the
+    step of `run_config` runs the layers on fixed inputs, so nothing in it waits for a predecessor).  Per block:
+    qkv(x) -> q; proj(the first M*dim values of q, standing in for the attention output) -> p; fc1(p) -> h; fc2(h) -> x.
+    Two figures under one HIP graph per step: `plain` (arcq_linear_otf_ws per layer) and `fused` (arcq_linear_otf_ex:
+    LayerNorm in front of qkv / fc1, GELU behind fc1, the skip connections behind proj / fc2 -- the work that sits
+    between the packed linears of a transformer block, inside their launches)."""
+    import ctypes
+    import torch
+    from arcq_vit_amd import _lib, synth
+    from arcq_vit_amd._lib import ARCQ_F16
+    lib = _lib.load()
+    m, layers, inputs, ws, _ = build_workload(model, bits, batch, dev)
+    dim, hid = synth.MODEL_DIMS[model]["dim"], synth.MODEL_DIMS[model]["mlp"]
+    x0 = inputs["qkv"].clone()
+    ring = [torch.empty_like(x0) for _ in range(3)]       # the residual stream after attention / after the MLP, rotating
+    q = torch.empty(m * 3 * dim, dtype=torch.float16, device=dev)
+    h = torch.empty(m * hid, dtype=torch.float16, device=dev)
+    ln_w = torch.ones(max(dim, hid), dtype=torch.float32, device=dev)
+    ln_b = torch.zeros(max(dim, hid), dtype=torch.float32, device=dev)
+    keep = []
+
+    def ex(l, x, y, ln=False, gelu=False, res=None):
+        a = _lib.LinearExArgs()
+        a.struct_size = ctypes.sizeof(_lib.LinearExArgs)
+        a.x_dtype = a.y_dtype = ARCQ_F16
+        a.bits, a.group_size, a.M, a.N, a.K = l.bits, 64, m, l.n, l.k
+        a.x, a.y, a.x_hat_ws, a.w_hat_ws = x.data_ptr(), y.data_ptr(), ws.data_ptr(), Layer.W_WS.data_ptr()
+        if ln:
+            a.producer, a.ln_weight, a.ln_bias, a.ln_eps = _lib.ARCQ_PRODUCER_LAYERNORM, ln_w.data_ptr(), ln_b.data_ptr(), 1e-6
+        a.activation = _lib.ARCQ_ACT_GELU if gelu else _lib.ARCQ_ACT_NONE
+        a.residual = None if res is None else res.data_ptr()
+        a.a_thresholds, a.a_codebook, a.packed_w, a.w_codebook = l.thr.data_ptr(), l.cb.data_ptr(), l.packed.data_ptr(), l.cb.data_ptr()
+        a.w_center, a.w_scale, a.w_code_sum, a.bias = l.center.data_ptr(), l.scale.data_ptr(), l.code_sum.data_ptr(), l.bias.data_ptr()
+        keep.append(a)
+        return a
+
+    def run(fused, stream):
+        cur, r = x0, 0
+        for b in range(len(layers) // 4):
+            qkv, proj, fc1, fc2 = layers[4 * b:4 * b + 4]
+            mid, nxt = ring[r % 3], ring[(r + 1) % 3]       # cur is x0 or ring[(r + 2) % 3]
+            r += 2
+            calls = ([ex(qkv, cur, q, ln=True), ex(proj, q, mid, res=cur), ex(fc1, mid, h, ln=True, gelu=True),
+                      ex(fc2, h, nxt, res=mid)] if fused else
+                     [ex(qkv, cur, q), ex(proj, q, mid), ex(fc1, mid, h), ex(fc2, h, nxt)])
+            for a in calls:
+                rc = lib.arcq_linear_otf_ex(ctypes.byref(a), stream)
+                if rc:
+                    _lib.check(rc)
+            cur = nxt
+
+    out = {}
+    for name, fused in (("plain", False), ("fused", True)):
+        run(fused, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            run(fused, torch.cuda.current_stream().cuda_stream)
+        t = time_loop(g.replay, steps, warmup)
+        out[name + "_ms_per_step"] = t / steps * 1e3
+        out[name + "_images_per_s"] = batch * steps / t
+        del g
+    out["note"] = ("every layer reads its predecessor's output; fused = LayerNorm / GELU / skip connections inside the "
+                   "packed layers' launches (arcq_linear_otf_ex)")
+    return out
+
+
 def cpu_baseline(layers, inputs, batch, budget_s=12.0):
     """Oracle restatement of QuantLinearPCARCQ.forward (FQ/quant_backends.py:312-322) on host cores: the four linears
     of ONE block at the benchmark's batch, repeated while the time budget lasts (at least once); images/s = batch /
@@ -433,7 +501,7 @@ def model_forward(model, bits, batches, steps, warmup, dev):
     images: the protocol of scripts/benchmark_arcq_on_the_fly.py:202-243 (HIP graph at batch 1, eager otherwise; both
     figures are given for every batch).  Two models: the block's LayerNorms, GELU and skip connections
     as separate torch kernels (`unfused`, the reference's structure) and inside the packed layers' launches
-    (`fused_elementwise`; below 512 rows the layers run them separately, so batch 1 shows no difference)."""
+    (`fused_elementwise`)."""
     import torch
     from arcq_vit_amd import synth
     from arcq_vit_amd.vit import build_packed_vit
@@ -445,8 +513,6 @@ def model_forward(model, bits, batches, steps, warmup, dev):
         part = {}
         with torch.no_grad():
             for b in batches:
-                if fuse and b * synth.TOKENS < 512:
-                    continue
                 x = synth.make_images(b, 1).to(dev).half()
                 n = max(steps // (4 if b > 1 else 1), 5)
                 res = {}
@@ -605,6 +671,7 @@ def main():
                       "gemm_hbm_frac_warm": r1["gemm_gbs"] / PEAK_HBM_GBS, "act_us_per_launch": r1["act_us_per_launch"],
                       "hip_graph": True}
         out["bs1"]["cold_cache"] = cold_cache_bs1(args.model, args.bits, max(args.steps, 50), max(args.warmup, 10), dev)
+        out["bs1"]["chained"] = chained_step(args.model, args.bits, 1, max(args.steps, 50), max(args.warmup, 10), dev)
     if not args.no_model:
         out["model_forward"] = model_forward(args.model, args.bits, sorted({1, args.batch}), args.steps, args.warmup, dev)
     if args.fp8:

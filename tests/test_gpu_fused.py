@@ -76,7 +76,19 @@ def test_layernorm_stage1_bitexact(cuda, oracle, bits, m, k, in_dtype):
     (12608, 768, 3072, 3, False, False, True),      # DeiT-B fc2 at W3: the two-blocks-per-wave kernel
     (12608, 3072, 768, 4, True, True, False),       # DeiT-B fc1
     (1000, 200, 448, 4, True, True, True),          # ragged rows and columns, everything at once
-    (600, 100, 1024, 3, True, False, True)])
+    (600, 100, 1024, 3, True, False, True),
+    # fewer than 512 rows (batch 1): one launch with everything inside, or stage 1 + split-K with the post-operations
+    (197, 1152, 384, 4, True, False, False),        # qkv of DeiT-S at batch 1
+    (197, 384, 384, 4, False, False, True),         # proj
+    (197, 1536, 384, 4, True, True, False),         # fc1
+    (197, 384, 1536, 4, False, False, True),        # fc2: two launches, residual in the split-K epilogue
+    (197, 2304, 768, 3, True, False, False),        # DeiT-B qkv: one lane per group
+    (197, 3072, 768, 4, True, True, False),         # DeiT-B fc1: the one-launch kernel because of the LayerNorm
+    (394, 768, 192, 4, True, True, True),           # DeiT-tiny, batch 2
+    (100, 200, 1024, 4, True, True, True),          # ragged rows and columns
+    (37, 96, 1536, 3, True, False, True),           # LayerNorm over a long row: two rounds of stage-1 tiles
+    (197, 100, 1536, 2, False, True, True),         # split-K epilogue, ragged columns
+    (1, 64, 64, 4, True, True, True)])
 def test_linear_otf_ex_equals_the_unfused_sequence(cuda, oracle, m, n, k, bits, ln, gelu, res):
     """arcq_linear_otf_ex == LayerNorm (oracle, rounded to fp16) -> arcq_linear_otf_ws -> torch GELU -> torch add, every
     step in fp16 as the unfused model runs them: bit for bit; sampled rows of the linear part against the fp64 oracle."""
@@ -131,12 +143,22 @@ def test_linear_otf_ex_fp32_and_limits(cuda, oracle):
     assert torch.equal(y, torch.nn.functional.gelu(lin) + r)
     assert torch.equal(ops.linear_otf_ex(x, *args, out_dtype=torch.float32), lin)      # no option: the plain layer
     small = x[:197].contiguous()
-    assert torch.equal(ops.linear_otf_ex(small, *args, out_dtype=torch.float32),
-                       ops.linear_otf(small, *args, out_dtype=torch.float32))
-    with pytest.raises(RuntimeError, match="at least 512 rows"):
-        ops.linear_otf_ex(small, *args, out_dtype=torch.float32, gelu=True)
+    lin_small = ops.linear_otf(small, *args, out_dtype=torch.float32)
+    assert torch.equal(ops.linear_otf_ex(small, *args, out_dtype=torch.float32), lin_small)
+    assert torch.equal(ops.linear_otf_ex(small, *args, out_dtype=torch.float32, gelu=True, residual=r[:197].contiguous()),
+                       torch.nn.functional.gelu(lin_small) + r[:197])
+    # fp32 input with a LayerNorm in front, below 512 rows: the LayerNorm's result is not rounded to fp16
+    lw, lb = _ln_params(k, 8)
+    xln = torch.from_numpy(oracle.layernorm_rows_np(small.cpu().numpy(), lw.numpy(), lb.numpy(), 1e-6, out_f16=False))
+    assert torch.equal(ops.linear_otf_ex(small, *args, out_dtype=torch.float32, layernorm=(d(lw), d(lb), 1e-6)),
+                       ops.linear_otf(d(xln), *args, out_dtype=torch.float32))
     with pytest.raises(RuntimeError, match="residual"):
         ops.linear_otf_ex(x, *args, out_dtype=torch.float32, residual=r.half())
+    wide = synth.make_activation(8, 2048, 44).to(cuda)
+    pw2, _, wc2, ws2, wcs2 = _weights(oracle, 64, 2048, bits, 45)
+    with pytest.raises(RuntimeError, match="in_features <= 1536"):
+        ops.linear_otf_ex(wide, d(thr), d(cb), d(pw2), d(cb), d(wc2), d(ws2), d(wcs2), None, bits, 64,
+                          layernorm=(torch.ones(2048, device=cuda), torch.zeros(2048, device=cuda), 1e-6))
 
 
 @pytest.mark.parametrize("model,batch", [("deit_small", 64), ("deit_tiny", 2)])
@@ -144,8 +166,8 @@ def test_vit_block_fusion(cuda, oracle, model, batch):
     """The ViT skeleton with LayerNorm / GELU / skip connections inside the packed layers' launches: every packed layer's
     output, captured by forward hooks, equals the oracle's value of the same fused layer on the captured input
     (LayerNorm restatement -> stage 1 -> fp64 product -> GELU / residual in fp16), and the logits stay close to the
-    unfused model's (whose LayerNorm is torch's kernel: another summation order, so codes may differ at ties).  At
-    batch 2 (394 rows) the layers fall back to separate operations and must equal the unfused model exactly."""
+    unfused model's (whose LayerNorm is torch's kernel: another summation order, so codes may differ at ties).  Batch 2
+    (394 rows) takes the small-M kernels: one launch per layer with everything inside, fc2 as stage 1 + split-K."""
     kw = dict(num_classes=100, device="cuda", half_chain=True, depth=2, shared_buffers=True, max_rows=batch * synth.TOKENS)
     fused = build_packed_vit(model, 4, fuse_elementwise=True, **kw)
     plain = build_packed_vit(model, 4, fuse_elementwise=False, **kw)
@@ -167,9 +189,6 @@ def test_vit_block_fusion(cuda, oracle, model, batch):
     for h in hooks:
         h.remove()
     assert bool(torch.isfinite(lf).all())
-    if batch * synth.TOKENS < 512:
-        assert torch.equal(lf, lp)
-        return
     assert len(captured) == 8
     for mod, ln, act, x2, r2, y in captured:
         k = mod.in_features
