@@ -103,8 +103,9 @@ static int linear_otf_impl(const void *x, int x_dtype, const float *a_thresholds
             w_codebook && w_center && w_scale && w_code_sum && y && (x_dtype == ARCQ_F16 || x_dtype == ARCQ_F32) &&
             (y_dtype == ARCQ_F16 || y_dtype == ARCQ_F32) && arcq::aligned(x, 16) && arcq::aligned(x_hat_ws, 16) &&
             arcq::aligned(y, 16) && arcq::aligned(packed_w, 16)) {
+            // (with scratch-only workspaces nobody reads x_hat afterwards: the kernel then keeps it in LDS only)
             arcq::OtfSmallArgs a{x, x_dtype == ARCQ_F16, a_thresholds, a_codebook, packed_w, w_codebook, w_center, w_scale,
-                                 w_code_sum, bias, x_hat_ws, y, y_dtype == ARCQ_F16, static_cast<int>(M),
+                                 w_code_sum, bias, scratch_only ? nullptr : x_hat_ws, y, y_dtype == ARCQ_F16, static_cast<int>(M),
                                  static_cast<int>(N), static_cast<int>(K), bits, 1.0e-6f};
             arcq::launch_otf_small(a, static_cast<hipStream_t>(stream));
             return arcq::launch_status("arcq_linear_otf");
@@ -208,7 +209,7 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
                                         : (!(e && e[0] == '0') && arcq::otf_small_supported(a->M, a->N, a->K, e && e[0] == '2'));
         if (one_launch) {
             arcq::OtfSmallArgs s{a->x, a->x_dtype == ARCQ_F16, a->a_thresholds, a->a_codebook, a->packed_w, a->w_codebook,
-                                 a->w_center, a->w_scale, a->w_code_sum, a->bias, a->x_hat_ws, a->y, a->y_dtype == ARCQ_F16,
+                                 a->w_center, a->w_scale, a->w_code_sum, a->bias, nullptr, a->y, a->y_dtype == ARCQ_F16,
                                  static_cast<int>(a->M), static_cast<int>(a->N), static_cast<int>(a->K), a->bits, 1.0e-6f};
             if (want_ln) s.ln_weight = a->ln_weight, s.ln_bias = a->ln_bias, s.ln_eps = a->ln_eps;
             s.residual = a->residual;

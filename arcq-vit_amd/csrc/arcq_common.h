@@ -201,14 +201,13 @@ __device__ __forceinline__ void post_ops16(u32x4_store_t &v, const TOUT *res, bo
     __builtin_memcpy(&v, e, 16);
 }
 
-// The same two steps on one output value (the small-M kernels, whose threads hold a few consecutive outputs each).
+// The same two steps on one output value (the small-M kernels, whose threads hold a few consecutive outputs each);
+// `r` is the residual value, used when `has_res`.
 template <typename TOUT>
-__device__ __forceinline__ TOUT post_op1(TOUT v, const TOUT *res, bool gelu)
+__device__ __forceinline__ TOUT post_op1(TOUT v, bool has_res, TOUT r, bool gelu)
 {
-    if (gelu) {
-        v = from_float<TOUT>(gelu_f32(to_float(v)));
-    }
-    if (res) v = from_float<TOUT>(to_float(v) + to_float(*res));
+    if (gelu) v = from_float<TOUT>(gelu_f32(to_float(v)));
+    if (has_res) v = from_float<TOUT>(to_float(v) + to_float(r));
     return v;
 }
 

@@ -201,6 +201,16 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
             return acc;
         };
         const float fk = static_cast<float>(K);
+        const float4 *gp = reinterpret_cast<const float4 *>(ln_w + g * 64 + (lane % LPG) * EL);
+        const float4 *bp = reinterpret_cast<const float4 *>(ln_b + g * 64 + (lane % LPG) * EL);
+        // Half a group per lane: weight and bias are requested before the sums (64 registers); a whole group per lane
+        // has no registers to spare and loads them where they are used.
+        constexpr int PRE = LPG == 2 ? EL / 4 : 1;
+        float4 gpre[PRE], bpre[PRE];
+        if constexpr (LPG == 2) {
+#pragma unroll
+            for (int j4 = 0; j4 < PRE; ++j4) gpre[j4] = gp[j4], bpre[j4] = bp[j4];
+        }
         float ps[H];
 #pragma unroll
         for (int h = 0; h < H; ++h) {
@@ -223,11 +233,11 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
         }
         const float var_row = row_total(ps) / fk;
         const float rstd = 1.0f / sqrtf(var_row + ln_eps);
-        const float4 *gp = reinterpret_cast<const float4 *>(ln_w + g * 64 + (lane % LPG) * EL);
-        const float4 *bp = reinterpret_cast<const float4 *>(ln_b + g * 64 + (lane % LPG) * EL);
 #pragma unroll
         for (int j4 = 0; j4 < EL / 4; ++j4) {
-            const float4 gv = gp[j4], bv = bp[j4];
+            float4 gv, bv;
+            if constexpr (LPG == 2) gv = gpre[j4], bv = bpre[j4];
+            else gv = gp[j4], bv = bp[j4];
             const float g4[4] = {gv.x, gv.y, gv.z, gv.w}, b4[4] = {bv.x, bv.y, bv.z, bv.w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -309,6 +319,40 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     }
     __syncthreads();
 
+    // The thread's outputs in the epilogue (E consecutive ones of a row) are known now: their bias and residual values
+    // are requested here, so that the loads travel under the product instead of after it.
+    constexpr int E = RT * kOsCols / (kOsWaves * 64);            // outputs per thread, consecutive in a row (8, 4 or 2)
+    constexpr int TPR = kOsCols / E;                       // threads per row
+    constexpr int BYTES = E * static_cast<int>(sizeof(TOUT));
+    const int row = tid / TPR, col = (tid % TPR) * E;
+    const int gr = m0 + row, gc = n0 + col;
+    const bool vec_out = gr < M && gc + E <= N && (N % E) == 0 && BYTES % 4 == 0;
+    float bv[E];
+    TOUT rv[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) bv[e] = 0.0f, rv[e] = from_float<TOUT>(0.0f);
+    if (vec_out) {
+        if (bias) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) bv[e] = bias[gc + e];
+        }
+        if (residual) {    // (N % E == 0 and a 16-byte aligned tensor: the E values are aligned 4-, 8- or 16-byte loads)
+            const TOUT *rp = residual + static_cast<int64_t>(gr) * N + gc;
+            if constexpr (BYTES % 16 == 0) {
+#pragma unroll
+                for (int b = 0; b < BYTES / 16; ++b) {
+                    const u32x4_t v = reinterpret_cast<const u32x4_t *>(rp)[b];
+                    __builtin_memcpy(reinterpret_cast<char *>(rv) + 16 * b, &v, 16);
+                }
+            } else if constexpr (BYTES == 8) {
+                const u32x2_t v = *reinterpret_cast<const u32x2_t *>(rp);
+                __builtin_memcpy(rv, &v, 8);
+            } else {
+                const uint32_t v = *reinterpret_cast<const uint32_t *>(rp);
+                __builtin_memcpy(rv, &v, 4);
+            }
+        }
+    }
     // ---- stages 2+3: split-K product, wave w takes groups w, w+8, ... --------------------------------------
     float16_t acc[RB][CB];
 #pragma unroll
@@ -370,9 +414,6 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
                 *reinterpret_cast<f32x4_t *>(mine + (i * 32 + lr) * kOsRedPitch + (j * 32 + 8 * q + 4 * lh) * 4) = v;
             }
     __syncthreads();
-    constexpr int E = RT * kOsCols / (kOsWaves * 64);      // outputs per thread, consecutive in a row (8, 4 or 2)
-    constexpr int TPR = kOsCols / E;
-    const int row = tid / TPR, col = (tid % TPR) * E;
     float sum[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) sum[e] = 0.0f;
@@ -390,35 +431,36 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
             for (int e = 0; e < E; ++e) sum[e] += *reinterpret_cast<const float *>(src + e * 4);
         }
     }
-    const int gr = m0 + row, gc = n0 + col;
     if (gr < M && gc < N) {
         TOUT *dst = y + static_cast<int64_t>(gr) * N + gc;
         // Optional GELU / residual on the rounded output (post_op1): what separate elementwise kernels would store.
-        const TOUT *res = residual ? residual + static_cast<int64_t>(gr) * N + gc : nullptr;
-        const bool post = res || gelu;
-        constexpr int BYTES = E * static_cast<int>(sizeof(TOUT));
-        if (gc + E <= N && (N % E) == 0 && BYTES % 8 == 0) {
+        const bool post = residual || gelu;
+        if (vec_out) {
             TOUT out[E];
 #pragma unroll
-            for (int e = 0; e < E; ++e) out[e] = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
+            for (int e = 0; e < E; ++e) out[e] = from_float<TOUT>(sum[e] + bv[e]);
             if (post) {
 #pragma unroll
-                for (int e = 0; e < E; ++e) out[e] = post_op1<TOUT>(out[e], res ? res + e : nullptr, gelu != 0);
+                for (int e = 0; e < E; ++e) out[e] = post_op1<TOUT>(out[e], residual != nullptr, rv[e], gelu != 0);
             }
             if constexpr (BYTES % 16 == 0) {
 #pragma unroll
                 for (int b = 0; b < BYTES; b += 16)
                     *reinterpret_cast<u32x4_t *>(reinterpret_cast<char *>(dst) + b) =
                         *reinterpret_cast<const u32x4_t *>(reinterpret_cast<const char *>(out) + b);
-            } else {
+            } else if constexpr (BYTES == 8) {
                 *reinterpret_cast<u32x2_t *>(dst) = *reinterpret_cast<const u32x2_t *>(out);
+            } else {
+                static_assert(BYTES == 4, "outputs per thread");
+                *reinterpret_cast<uint32_t *>(dst) = *reinterpret_cast<const uint32_t *>(out);
             }
         } else {
+            const TOUT *res = residual ? residual + static_cast<int64_t>(gr) * N + gc : nullptr;
 #pragma unroll
             for (int e = 0; e < E; ++e)
                 if (gc + e < N) {
                     TOUT o = from_float<TOUT>(sum[e] + (bias ? bias[gc + e] : 0.0f));
-                    if (post) o = post_op1<TOUT>(o, res ? res + e : nullptr, gelu != 0);
+                    if (post) o = post_op1<TOUT>(o, res != nullptr, res ? res[e] : o, gelu != 0);
                     dst[e] = o;
                 }
         }
