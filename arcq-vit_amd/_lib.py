@@ -63,6 +63,11 @@ _SIGNATURES = {
     "arcq_act_quant_blocked": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32, _c_ptr],
     "arcq_act_quant_fp8": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32, _c_ptr],
     "arcq_weight_dequant_fp8": [_c_ptr] * 6 + [_c_i64, _c_i64, _c_int, _c_int, _c_f32, _c_ptr],
+    "arcq_act_quant_fp8_blocked": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32,
+                                   _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_f32, _c_ptr],
+    "arcq_linear_fp8_blocked": [_c_ptr, _c_ptr, _c_ptr, _c_f32, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_ptr],
+    "arcq_linear_otf_fp8": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_f32,
+                            _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr],
     "arcq_act_quant_blocked_with_weights": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32,
                                             _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr],
     "arcq_linear_fused_blocked": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int,

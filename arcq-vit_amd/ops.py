@@ -484,19 +484,62 @@ def unpack_weight_fp8(packed: torch.Tensor, codebook: torch.Tensor, center: torc
     return out
 
 
+def fp8_padded_k(k: int) -> int:
+    """Row length of the FP8 GEMM's operands: ``k`` rounded up to a multiple of 128 (the padding is zero)."""
+    return (int(k) + 127) // 128 * 128
+
+
 def linear_otf_fp8(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Tensor, packed_w: torch.Tensor,
                    w_codebook: torch.Tensor, w_center: torch.Tensor, w_scale: torch.Tensor, w_code_sum: torch.Tensor,
                    bias: Optional[torch.Tensor], bits: int, out_dtype: torch.dtype = torch.float16,
                    w_mult: Optional[float] = None, x8_ws: Optional[torch.Tensor] = None,
                    w8_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The packed on-the-fly layer with FP8 operands: stage 1 and stage 2 as in ``linear_otf`` but rounded to FP8, the
-    product as the vendor library's FP8 GEMM with fp32 accumulation (``torch._scaled_mm``), ``y = x8 w8^T / w_mult +
-    bias``.  Faster where the layer is bound by the matrix units (the large models), NOT bit-compatible with the
-    reference: each operand carries a rounding error of up to 2^-4 relative (fp16: 2^-11).  Group size 64."""
+    """The packed on-the-fly layer with FP8 operands (``arcq_linear_otf_fp8``, two launches): stage 1 and stage 2 as in
+    ``linear_otf`` but rounded to FP8 (the weights first multiplied by ``w_mult``), then the library's own FP8 MFMA GEMM
+    with fp32 accumulation, ``y = x8 w8^T / w_mult + bias``.  Faster where the layer is bound by the matrix units (the
+    large models), NOT bit-compatible with the reference: each operand carries a rounding error of up to 2^-4 relative
+    (fp16: 2^-11).  Group size 64.  ``x8_ws`` / ``w8_ws``: scratch of at least ``M * Kp`` / ``N * Kp`` bytes
+    (``Kp = fp8_padded_k(K)``), any 1-byte dtype."""
+    _check(x.is_cuda and x.dim() == 2, "x must be a CUDA tensor of shape [M, K]")
+    _check_bits(bits)
+    x = x.contiguous()
+    m, k = x.shape
+    n = packed_w.shape[0]
+    _check(k % 64 == 0 and k > 0, "in_features must be a positive multiple of the group size 64")
+    _check(packed_w.shape[1] == (k * bits + 7) // 8, "packed_w row length does not match K*bits/8")
+    if w_mult is None:
+        w_mult = fp8_weight_multiplier(w_codebook, w_center, w_scale, w_code_sum)
+    kp = fp8_padded_k(k)
+    if x8_ws is None:
+        x8_ws = torch.empty(max(m * kp, 1), dtype=torch.uint8, device=x.device)
+    if w8_ws is None:
+        w8_ws = torch.empty(max(n * kp, 1), dtype=torch.uint8, device=x.device)
+    for t, need, name in ((x8_ws, m * kp, "x8_ws"), (w8_ws, n * kp, "w8_ws")):
+        _check(t.is_cuda and t.is_contiguous() and t.element_size() == 1 and t.numel() >= need,
+               f"{name} must be a contiguous 1-byte CUDA buffer of at least {need} elements")
+    y = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    a = [_f32c(a_thresholds), _f32c(a_codebook)]
+    w = [packed_w.contiguous(), _f32c(w_codebook), _f32c(w_center), _f32c(w_scale), _f32c(w_code_sum)]
+    b = None if bias is None or bias.numel() == 0 else _f32c(bias)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().arcq_linear_otf_fp8(
+            _ptr(x), _dtype_code(x, "x"), *[_ptr(t) for t in a], *[_ptr(t) for t in w], _ptr(b), float(w_mult),
+            _ptr(x8_ws), _ptr(w8_ws), _ptr(y), _dtype_code(y, "y"), m, n, k, bits, _stream()))
+    return y
+
+
+def linear_otf_fp8_library_gemm(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Tensor,
+                                packed_w: torch.Tensor, w_codebook: torch.Tensor, w_center: torch.Tensor,
+                                w_scale: torch.Tensor, w_code_sum: torch.Tensor, bias: Optional[torch.Tensor], bits: int,
+                                out_dtype: torch.dtype = torch.float16, w_mult: Optional[float] = None,
+                                x8_ws: Optional[torch.Tensor] = None, w8_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The same layer with the product left to the vendor library's FP8 GEMM (``torch._scaled_mm``) on row-major
+    operands, three launches: kept as a timing and cross-check reference for ``linear_otf_fp8``, not used by the
+    modules."""
     _check(x.is_cuda and x.dim() == 2, "x must be a CUDA tensor of shape [M, K]")
     m, k = x.shape
     n = packed_w.shape[0]
-    _check(k % 16 == 0 and n % 16 == 0, "the FP8 GEMM needs K and N to be multiples of 16")
+    _check(k % 16 == 0 and n % 16 == 0, "the library's FP8 GEMM needs K and N to be multiples of 16")
     if w_mult is None:
         w_mult = fp8_weight_multiplier(w_codebook, w_center, w_scale, w_code_sum)
     x8 = quantize_activation_fp8(x, a_thresholds, a_codebook, bits, out=x8_ws)

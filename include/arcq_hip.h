@@ -272,12 +272,37 @@ int arcq_linear_otf_static(const void *x, int x_dtype, const float *a_thresholds
  *   arcq_act_quant_fp8:      x8[rows, cols]  = fp8(x_hat), row-major, cols a multiple of 64 (group size 64 only)
  *   arcq_weight_dequant_fp8: w8[N, K]        = fp8(w_mult * w_hat), row-major; w_mult > 0, a power of two chosen by the
  *                                              caller so that the weights fall into FP8's normal range (2^-6 .. 448)
- * The product y = (x8 w8^T) / w_mult + bias is a plain FP8 GEMM with fp32 accumulation, left to a GEMM library. */
+ * The product y = (x8 w8^T) / w_mult + bias on these row-major operands is a plain FP8 GEMM with fp32 accumulation that
+ * any GEMM library can run; arcq_linear_otf_fp8 below is the layer on this library's own FP8 kernel. */
 int arcq_act_quant_fp8(const void *x, int x_dtype, const float *thresholds, const float *codebook, void *x8,
                        int64_t rows, int64_t cols, int bits, float eps, void *stream);
 int arcq_weight_dequant_fp8(const uint8_t *packed, const float *codebook, const float *center, const float *scale,
                             const float *code_sum, void *w8, int64_t N, int64_t K, int bits, int group_size,
                             float w_mult, void *stream);
+
+/* The FP8-operand layer end to end on hand-written kernels (no counterpart in the reference; same caveat: FP8 operands
+ * do not reproduce its numbers).  Kp below is K rounded up to a multiple of 128.
+ *   arcq_act_quant_fp8_blocked: stage 1 with x8 in the FP8 GEMM's block layout, 16-byte pieces
+ *       x8_blocked[((row / 32) * (Kp / 16) + k / 16) * 32 + row % 32][k % 16]
+ *     (a last block of r = rows % 32 rows compactly as [(k / 16) * r + row % 32][k % 16]); the pieces from K to Kp are
+ *     written as zeros; rows * Kp bytes in all.  packed_w != NULL: extra workgroups of the same launch also write
+ *     w8[N, Kp] = fp8(w_mult * w_hat), rows Kp bytes apart, zero from K to Kp (what arcq_weight_dequant_fp8 computes).
+ *   arcq_linear_fp8_blocked: y[M,N] = (x8 w8^T) / w_mult + bias on v_mfma_f32_32x32x64_f8f6f4 (fp32 accumulation in
+ *     ascending k; bias fp32 or NULL, added in fp32 before the one output rounding; y ARCQ_F16 or ARCQ_F32).  K here is
+ *     the padded length Kp (a multiple of 128); x8_blocked and w8 as written by arcq_act_quant_fp8_blocked.
+ *   arcq_linear_otf_fp8: the two of them, i.e. the whole layer in two launches.  x8_ws: M * Kp bytes, w8_ws: N * Kp
+ *     bytes, both 16-byte aligned scratch. */
+int arcq_act_quant_fp8_blocked(const void *x, int x_dtype, const float *thresholds, const float *codebook,
+                               void *x8_blocked, int64_t rows, int64_t cols, int bits, float eps,
+                               const uint8_t *packed_w, const float *w_codebook, const float *w_center,
+                               const float *w_scale, const float *w_code_sum, void *w8, int64_t N, float w_mult,
+                               void *stream);
+int arcq_linear_fp8_blocked(const void *x8_blocked, const void *w8, const float *bias, float w_mult, void *y, int y_dtype,
+                            int64_t M, int64_t N, int64_t K, void *stream);
+int arcq_linear_otf_fp8(const void *x, int x_dtype, const float *a_thresholds, const float *a_codebook,
+                        const uint8_t *packed_w, const float *w_codebook, const float *w_center, const float *w_scale,
+                        const float *w_code_sum, const float *bias, float w_mult, void *x8_ws, void *w8_ws, void *y,
+                        int y_dtype, int64_t M, int64_t N, int64_t K, int bits, void *stream);
 
 /* Kernels arcq_linear_otf_ws runs after stage 1 for these sizes: "gemm_slab8_kernel", or, with the weights rebuilt
  * in the stage-1 launch and copied by the GEMM, "gemm_slab8_kernel<copy>" or "gemm_pair_kernel" (two row blocks per

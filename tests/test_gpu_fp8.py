@@ -1,5 +1,5 @@
 """GPU tests of the layer with FP8 operands (``ops.linear_otf_fp8``: stage 1 and stage 2 rounded to OCP E4M3, the
-product as the vendor library's FP8 GEMM).  The path has no counterpart in the reference and does not reproduce its
+product on the library's own FP8 MFMA kernel).  The path has no counterpart in the reference and does not reproduce its
 numbers; what is checked is that it is exactly what it says: the operands are the oracle's fp32 reconstructions
 rounded to FP8 bit for bit, and the product is their exact product within fp32 accumulation error."""
 import numpy as np
@@ -83,6 +83,79 @@ def test_fp8_layer_is_the_exact_product_of_its_operands(cuda, oracle, m, n, k, b
     assert 1e-4 < rel < 0.05, rel
 
 
+def _fp8_blocked(a: np.ndarray, kp: int) -> np.ndarray:
+    """[M, K] bytes -> the FP8 GEMM's block layout [M/32][kp/16][rows][16] (zero padding from K to kp), flat."""
+    m, k = a.shape
+    pad = np.zeros((m, kp), dtype=np.uint8)
+    pad[:, :k] = a
+    parts = []
+    for r0 in range(0, m, 32):
+        blk = pad[r0:r0 + 32]
+        parts.append(np.ascontiguousarray(blk.reshape(blk.shape[0], kp // 16, 16).transpose(1, 0, 2)).reshape(-1))
+    return np.concatenate(parts)
+
+
+@pytest.mark.parametrize("m,n,k,bits,dtype", [(197, 96, 192, 4, torch.float16), (1000, 200, 384, 3, torch.float32),
+                                              (4099, 64, 1536, 2, torch.float16), (33, 40, 64, 4, torch.float32)])
+def test_stage1_fp8_blocked_with_weights(cuda, oracle, m, n, k, bits, dtype):
+    """arcq_act_quant_fp8_blocked: the bytes of the row-major kernel in the block layout, zero padding to a multiple of
+    128, and -- carried in the same launch -- the FP8 weights with the same padding."""
+    cb, thr, pw, wc, ws, wcs, _ = _layer(oracle, n, k, bits, 13)
+    x = synth.make_activation(m, k, 7, "ln").to(dtype)
+    kp = ops.fp8_padded_k(k)
+    mult = ops.fp8_weight_multiplier(cb, wc, ws, wcs)
+    d = lambda t: t.to(cuda)
+    x8 = torch.full((m * kp + 16,), 0x5a, dtype=torch.uint8, device=cuda)
+    w8 = torch.full((n * kp + 16,), 0x5a, dtype=torch.uint8, device=cuda)
+    lib = A._lib.load()
+    xd, td, cd = d(x), d(thr), d(cb)
+    wts = [d(t) for t in (pw, cb, wc, ws, wcs)]
+    code = A._lib.ARCQ_F16 if dtype == torch.float16 else A._lib.ARCQ_F32
+    A._lib.check(lib.arcq_act_quant_fp8_blocked(xd.data_ptr(), code, td.data_ptr(), cd.data_ptr(), x8.data_ptr(), m, k, bits,
+                                               1e-6, *[t.data_ptr() for t in wts], w8.data_ptr(), n, mult, 0))
+    torch.cuda.synchronize()
+    want_x = _fp8_bytes(oracle.fp8_e4m3_np(oracle.act_quant_c(x.float().numpy(), thr, cb, bits, 64)["x_hat"]))
+    assert np.array_equal(_np(x8)[:m * kp], _fp8_blocked(want_x, kp))
+    w = oracle.weight_dequant_c(pw.numpy(), cb, wc, ws, wcs, bits, 64, fma=True)
+    want_w = np.zeros((n, kp), dtype=np.uint8)
+    want_w[:, :k] = _fp8_bytes(oracle.fp8_e4m3_np(w * np.float32(mult)))
+    assert np.array_equal(_np(w8)[:n * kp].reshape(n, kp), want_w)
+    assert bool((x8[m * kp:] == 0x5a).all()) and bool((w8[n * kp:] == 0x5a).all())
+
+
+@pytest.mark.parametrize("m,n,k,out", [(50, 64, 128, torch.float32), (197, 384, 1536, torch.float16),
+                                       (1000, 200, 256, torch.float32),       # ragged rows and columns
+                                       (3000, 768, 768, torch.float16), (12608, 1152, 384, torch.float16),
+                                       (8191, 4096, 1024, torch.float16)])    # sixteen row blocks and more per workgroup
+def test_fp8_gemm_kernel_against_fp64(cuda, oracle, m, n, k, out):
+    """arcq_linear_fp8_blocked on random FP8 operands against their fp64 product (fp32 accumulation bound + the output
+    rounding) on sampled rows, and against the vendor library's FP8 GEMM on the same operands."""
+    g = torch.Generator().manual_seed(5)
+    a = (torch.randn(m, k, generator=g) * 1.5).to(torch.float8_e4m3fn)
+    w = (torch.randn(n, k, generator=g) * 4.0).to(torch.float8_e4m3fn)
+    bias = torch.randn(n, generator=g)
+    mult = 16.0
+    xb = torch.from_numpy(_fp8_blocked(a.view(torch.uint8).numpy(), k)).to(cuda)
+    wd = w.to(cuda)
+    y = torch.empty((m, n), dtype=out, device=cuda)
+    A._lib.check(A._lib.load().arcq_linear_fp8_blocked(xb.data_ptr(), wd.data_ptr(), bias.to(cuda).data_ptr(), mult, y.data_ptr(),
+                                                      A._lib.ARCQ_F16 if out == torch.float16 else A._lib.ARCQ_F32, m, n, k, 0))
+    rows = torch.randint(0, m, (40,), generator=torch.Generator().manual_seed(3))
+    rows[0], rows[1], rows[2] = 0, m - 1, (m // 32) * 32 - 1
+    y64, mag = oracle.linear_f64_c(a[rows].float().numpy(), w.float().numpy(), None)
+    y64, mag = y64 / mult + bias.numpy().astype(np.float64), mag / mult
+    ulp = 2.0 ** -11 if out == torch.float16 else 2.0 ** -24
+    # (the matrix unit sums the 64 products of one instruction internally, not as a chain of correctly rounded fp32
+    # additions: twice the serial-fp32 bound is allowed for it; measured worst case 1.4 x)
+    tol = 2 * (k + 2) * 2.0 ** -24 * mag + np.abs(y64) * ulp + 2.0 ** -24
+    err = np.abs(_np(y[rows.to(cuda)]).astype(np.float64) - y64)
+    assert np.all(err <= tol), float((err / tol).max())
+    if out == torch.float16 and n % 16 == 0:
+        one = torch.ones((), device=cuda)
+        lib_y = torch._scaled_mm(a.to(cuda), wd.t(), scale_a=one, scale_b=one / mult, bias=bias.half().to(cuda), out_dtype=out)
+        assert float((y.float() - lib_y.float()).abs().max()) <= 4e-3 * float(lib_y.float().abs().max())
+
+
 def test_fp8_entry_points_reject_bad_arguments(cuda):
     lib = A._lib.load()
     x = torch.zeros(64 * 64, dtype=torch.float16, device=cuda)
@@ -97,6 +170,11 @@ def test_fp8_entry_points_reject_bad_arguments(cuda):
     assert lib.arcq_weight_dequant_fp8(*args, 8, 64, 4, 32, 1.0, 0) != 0                        # group size 64 only
     assert lib.arcq_weight_dequant_fp8(*args, 8, 64, 4, 64, 0.0, 0) != 0                        # multiplier must be positive
     assert lib.arcq_weight_dequant_fp8(*args, 8, 64, 7, 64, 1.0, 0) != 0
+    y = torch.zeros(64 * 64, dtype=torch.float16, device=cuda)
+    assert lib.arcq_linear_fp8_blocked(out.data_ptr(), out.data_ptr(), None, 1.0, y.data_ptr(), F16, 32, 64, 64, 0) != 0   # K % 128
+    assert lib.arcq_linear_fp8_blocked(out.data_ptr(), out.data_ptr(), None, 0.0, y.data_ptr(), F16, 32, 64, 128, 0) != 0  # multiplier
+    assert lib.arcq_linear_fp8_blocked(None, out.data_ptr(), None, 1.0, y.data_ptr(), F16, 32, 64, 128, 0) != 0
+    assert lib.arcq_linear_fp8_blocked(None, None, None, 1.0, None, F16, 0, 64, 128, 0) == 0                              # nothing to do
 
 
 def test_model_with_fp8_operands(cuda):
