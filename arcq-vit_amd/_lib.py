@@ -32,10 +32,11 @@ class LinearExArgs(ctypes.Structure):
                 ("a_thresholds", ctypes.c_void_p), ("a_codebook", ctypes.c_void_p), ("packed_w", ctypes.c_void_p),
                 ("w_codebook", ctypes.c_void_p), ("w_center", ctypes.c_void_p), ("w_scale", ctypes.c_void_p),
                 ("w_code_sum", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("residual", ctypes.c_void_p),
-                ("x_hat_ws", ctypes.c_void_p), ("w_hat_ws", ctypes.c_void_p), ("y", ctypes.c_void_p)]
+                ("x_hat_ws", ctypes.c_void_p), ("w_hat_ws", ctypes.c_void_p), ("y", ctypes.c_void_p),
+                ("next_a_thresholds", ctypes.c_void_p), ("next_a_codebook", ctypes.c_void_p)]
 
 
-ARCQ_PRODUCER_NONE, ARCQ_PRODUCER_LAYERNORM = 0, 1
+ARCQ_PRODUCER_NONE, ARCQ_PRODUCER_LAYERNORM, ARCQ_PRODUCER_XHAT = 0, 1, 2
 ARCQ_ACT_NONE, ARCQ_ACT_GELU = 0, 1
 
 # name -> argtypes, in the order of include/arcq_hip.h
@@ -58,6 +59,7 @@ _SIGNATURES = {
     "arcq_linear_otf_static": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
     "arcq_linear_otf_ex": [ctypes.POINTER(LinearExArgs), _c_ptr],
+    "arcq_xhat_layout": [_c_i64],
     "arcq_act_quant_blocked_ln": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int,
                                   _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr],
     "arcq_act_quant_blocked": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_f32, _c_ptr],

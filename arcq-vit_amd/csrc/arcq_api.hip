@@ -1,6 +1,7 @@
 // Library-level pieces of libarcq_hip.so: version, per-thread error text and
 // the whole-layer entry point that chains stage 1 into the fused stages 2+3.
 #include <stdarg.h>
+#include <stddef.h>
 #include <string.h>
 
 #include <stdlib.h>
@@ -170,14 +171,20 @@ ARCQ_API int arcq_linear_otf_ws(const void *x, int x_dtype, const float *a_thres
 ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
 {
     if (!a) return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf_ex: args must not be NULL");
-    if (a->struct_size < sizeof(arcq_linear_ex_args))
+    constexpr size_t kFirstVersion = offsetof(arcq_linear_ex_args, next_a_thresholds);
+    if (a->struct_size < kFirstVersion)
         return arcq::fail(ARCQ_ERR_SHAPE, "arcq_linear_otf_ex: struct_size %u is smaller than this library's %zu",
-                          a->struct_size, sizeof(arcq_linear_ex_args));
-    if (a->producer != ARCQ_PRODUCER_NONE && a->producer != ARCQ_PRODUCER_LAYERNORM)
+                          a->struct_size, kFirstVersion);
+    const bool has_next = a->struct_size >= sizeof(arcq_linear_ex_args);
+    const float *next_thr = has_next ? a->next_a_thresholds : nullptr;
+    const float *next_cb = has_next ? a->next_a_codebook : nullptr;
+    if ((next_thr == nullptr) != (next_cb == nullptr))
+        return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf_ex: next_a_thresholds and next_a_codebook go together");
+    if (a->producer != ARCQ_PRODUCER_NONE && a->producer != ARCQ_PRODUCER_LAYERNORM && a->producer != ARCQ_PRODUCER_XHAT)
         return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: unknown producer %d", a->producer);
     if (a->activation != ARCQ_ACT_NONE && a->activation != ARCQ_ACT_GELU)
         return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: unknown activation %d", a->activation);
-    const bool options = a->producer != ARCQ_PRODUCER_NONE || a->activation != ARCQ_ACT_NONE || a->residual;
+    const bool options = a->producer != ARCQ_PRODUCER_NONE || a->activation != ARCQ_ACT_NONE || a->residual || next_thr;
     if (!options)
         return linear_otf_impl(a->x, a->x_dtype, a->a_thresholds, a->a_codebook, a->packed_w, a->w_codebook, a->w_center,
                                a->w_scale, a->w_code_sum, a->bias, a->x_hat_ws, a->w_hat_ws, true, a->y, a->y_dtype, a->M,
@@ -185,8 +192,16 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
     if (a->group_size != 64 || !arcq::bits_ok(a->bits))
         return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: the fused options need group_size 64 and bits 2/3/4 "
                           "(got group_size=%d bits=%d)", a->group_size, a->bits);
-    if (!a->x_hat_ws) return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf_ex: x_hat_ws must not be NULL");
-    if (a->x_hat_ws == a->x) return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: x_hat_ws must not alias x");
+    const bool from_xhat = a->producer == ARCQ_PRODUCER_XHAT;
+    if (from_xhat && a->x_dtype != ARCQ_F16)
+        return arcq::fail(ARCQ_ERR_DTYPE, "arcq_linear_otf_ex: ARCQ_PRODUCER_XHAT needs x as float16 (it is x_hat)");
+    if (next_thr && (a->y_dtype != ARCQ_F16 || a->N % 64 != 0))
+        return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: quantizing the output for the next layer needs a float16 y "
+                          "and out_features a multiple of 64");
+    if (!from_xhat) {
+        if (!a->x_hat_ws) return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf_ex: x_hat_ws must not be NULL");
+        if (a->x_hat_ws == a->x) return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: x_hat_ws must not alias x");
+    }
     if (a->residual && !arcq::aligned(a->residual, 16))
         return arcq::fail(ARCQ_ERR_ALIGN, "arcq_linear_otf_ex: residual must be 16-byte aligned");
     const bool want_ln = a->producer == ARCQ_PRODUCER_LAYERNORM;
@@ -196,16 +211,27 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
     // small-M kernel wherever that kernel can run (always with a LayerNorm: it is the only small-M kernel that has
     // one); else stage 1 row-major + the split-K kernel with the post-operations in its epilogue.
     if (a->M > 0 && a->M < 512 && a->N > 0 && a->N < (int64_t(1) << 30) && a->K >= 64 && a->K % 64 == 0) {
-        if (!a->x || !a->a_thresholds || !a->a_codebook || !a->packed_w || !a->w_codebook || !a->w_center || !a->w_scale ||
-            !a->w_code_sum || !a->y)
+        if (!a->x || (!from_xhat && (!a->a_thresholds || !a->a_codebook)) || !a->packed_w || !a->w_codebook || !a->w_center ||
+            !a->w_scale || !a->w_code_sum || !a->y)
             return arcq::fail(ARCQ_ERR_NULL, "arcq_linear_otf_ex: NULL tensor pointer");
         if ((a->x_dtype != ARCQ_F16 && a->x_dtype != ARCQ_F32) || (a->y_dtype != ARCQ_F16 && a->y_dtype != ARCQ_F32))
             return arcq::fail(ARCQ_ERR_DTYPE, "arcq_linear_otf_ex: x and y must be float16 or float32");
-        if (!arcq::aligned(a->x, 16) || !arcq::aligned(a->x_hat_ws, 16) || !arcq::aligned(a->y, 16) ||
+        if (!arcq::aligned(a->x, 16) || (!from_xhat && !arcq::aligned(a->x_hat_ws, 16)) || !arcq::aligned(a->y, 16) ||
             !arcq::aligned(a->packed_w, 16))
             return arcq::fail(ARCQ_ERR_ALIGN, "arcq_linear_otf_ex: x, x_hat_ws, y and packed_w must be 16-byte aligned");
+        if (from_xhat) {          // x is this layer's x_hat, row-major: stages 2+3 only
+            if (next_thr)
+                return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: below 512 rows a layer that starts from x_hat cannot "
+                                  "quantize its output for the next one");
+            return arcq::linear_fused_post(a->x, a->packed_w, a->w_codebook, a->w_center, a->w_scale, a->w_code_sum, a->bias,
+                                           a->y, a->y_dtype, a->M, a->N, a->K, a->bits, 64, stream, a->residual,
+                                           a->activation == ARCQ_ACT_GELU);
+        }
+        if (next_thr && !arcq::otf_small_supported(a->M, a->N, a->K, true))
+            return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: below 512 rows quantizing the output for the next layer "
+                              "needs in_features <= 1536");
         const char *e = arcq::tuning().otf_fused;
-        const bool one_launch = want_ln ? arcq::otf_small_supported(a->M, a->N, a->K, true)
+        const bool one_launch = next_thr ? true : want_ln ? arcq::otf_small_supported(a->M, a->N, a->K, true)
                                         : (!(e && e[0] == '0') && arcq::otf_small_supported(a->M, a->N, a->K, e && e[0] == '2'));
         if (one_launch) {
             arcq::OtfSmallArgs s{a->x, a->x_dtype == ARCQ_F16, a->a_thresholds, a->a_codebook, a->packed_w, a->w_codebook,
@@ -214,6 +240,7 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
             if (want_ln) s.ln_weight = a->ln_weight, s.ln_bias = a->ln_bias, s.ln_eps = a->ln_eps;
             s.residual = a->residual;
             s.gelu = a->activation == ARCQ_ACT_GELU;
+            s.next_thr = next_thr, s.next_cb = next_cb;
             arcq::launch_otf_small(s, static_cast<hipStream_t>(stream));
             return arcq::launch_status("arcq_linear_otf_ex");
         }
@@ -226,6 +253,8 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
                                        a->y, a->y_dtype, a->M, a->N, a->K, a->bits, 64, stream, a->residual,
                                        a->activation == ARCQ_ACT_GELU);
     }
+    if (from_xhat || next_thr)
+        return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: chaining two layers through x_hat is built for fewer than 512 rows");
     if (!arcq::otf_blocked_pays(a->M, a->N, a->K))
         return arcq::fail(ARCQ_ERR_UNSUPPORTED,
                           "arcq_linear_otf_ex: the fused options need in_features a positive multiple of 64 and a shape the "
@@ -268,6 +297,8 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
                                       a->w_hat_ws, carry, a->y, a->y_dtype, a->M, a->N, a->K, a->bits, a->group_size, stream,
                                       a->residual, a->activation == ARCQ_ACT_GELU);
 }
+
+ARCQ_API int arcq_xhat_layout(int64_t M) { return M < 512 ? 0 : 1; }
 
 // ---- the same layer for callers that cannot allocate --------------------------------------------------------
 // Both scratch buffers of arcq_linear_otf_ws live in a file-scope device array instead of caller memory.  Every GPU

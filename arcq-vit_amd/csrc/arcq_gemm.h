@@ -76,6 +76,9 @@ struct OtfSmallArgs {
     float ln_eps = 0.0f;
     const void *residual = nullptr;
     bool gelu = false;
+    // Quantize-the-output mode: y (fp16, N a multiple of 64) receives not the layer's output but stage 1 of the layer
+    // that consumes it (that layer's activation thresholds / codebook, same bits), row-major.
+    const float *next_thr = nullptr, *next_cb = nullptr;
 };
 bool otf_small_supported(int64_t M, int64_t N, int64_t K, bool any_supported);
 void launch_otf_small(const OtfSmallArgs &a, hipStream_t stream);

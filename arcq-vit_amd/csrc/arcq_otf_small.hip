@@ -100,7 +100,7 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
                  const float *__restrict__ bias, __half *__restrict__ x_hat_ws, TOUT *__restrict__ y,
                  int M, int N, int K, float eps, int tile_bytes, int partial_off,
                  const float *__restrict__ ln_w, const float *__restrict__ ln_b, float ln_eps, int ln_off,
-                 const TOUT *residual, int gelu)
+                 const TOUT *residual, int gelu, const float *__restrict__ nx_thr, const float *__restrict__ nx_cb, int nx_off)
 {
     constexpr int L = 1 << BITS;
     constexpr int RT = 32 * RB;
@@ -277,6 +277,20 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
     const bool write_ws = (x_hat_ws != nullptr) && blockIdx.x == 0;
     bool table_ok = true;
     for (int w = 0; w < (spare_waves ? kOsWaves - tile_waves : kOsWaves); ++w) table_ok = table_ok && (slow_slots[w] == 0);
+    // Quantize-the-output mode (nx_thr != nullptr: y receives stage 1 of the layer that consumes this one's output):
+    // that layer's lookup tables are built by the waves without a stage-1 tile while the others run theirs, or, when
+    // every wave has a tile, by all of them behind it.
+    float *n_lut = reinterpret_cast<float *>(smem + nx_off);
+    Bucket *n_table = reinterpret_cast<Bucket *>(n_lut + L * 64);
+    int *n_slots = reinterpret_cast<int *>(n_table + kMaxBuckets + 64);
+    const int n_builders = spare_waves ? kOsWaves - tile_waves : kOsWaves;
+    auto build_next_tables = [&]() {
+        float nth[L - 1], ncb[L];
+        load_quant_params<BITS>(nx_thr, nx_cb, nth, ncb);
+        const BucketScale nbq = pick_bucket_scale<BITS>(nth);
+        build_quant_tables_by<BITS>(nth, ncb, nbq, n_lut, n_table, n_slots, tid - (kOsWaves - n_builders) * 64, n_builders * 64);
+    };
+    if (nx_thr && spare_waves && !has_tile) build_next_tables();
     for (int t = wave; t < n_tiles; t += kOsWaves) {
         if (t != wave) {                       // later tiles of this wave: their inputs were requested a round ago
             stats();
@@ -317,6 +331,7 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
             for (int i = 0; i < EL / 8; ++i) dst[i] = out[i];
         }
     }
+    if (nx_thr && !spare_waves) build_next_tables();
     __syncthreads();
 
     // The thread's outputs in the epilogue (E consecutive ones of a row) are known now: their bias and residual values
@@ -431,6 +446,57 @@ otf_small_kernel(const TIN *__restrict__ x, const float *__restrict__ a_thr, con
             for (int e = 0; e < E; ++e) sum[e] += *reinterpret_cast<const float *>(src + e * 4);
         }
     }
+    if constexpr (CB == 2 && sizeof(TOUT) == 2) {
+        if (nx_thr) {          // workgroup-uniform; the launcher guarantees N % 64 == 0 (the tile is 32 rows x one group)
+            // The tile's outputs, rounded (and post-processed) as they would have been stored, meet in LDS; wave 0 then
+            // quantizes them as the consuming layer's stage 1 would -- two lanes per group -- and stores x_hat row-major.
+            TOUT out[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                out[e] = post_op1<TOUT>(from_float<TOUT>(sum[e] + bv[e]), residual != nullptr, rv[e], gelu != 0);
+            __syncthreads();                         // every thread is done reading the partial tiles
+            unsigned char *yt = partial;             // [32 rows][128 + 16 bytes]
+            *reinterpret_cast<u32x2_t *>(yt + row * 144 + col * 2) = *reinterpret_cast<const u32x2_t *>(out);
+            __syncthreads();
+            if (wave == 0) {
+                float nth[L - 1], ncb[L];
+                load_quant_params<BITS>(nx_thr, nx_cb, nth, ncb);
+                const BucketScale nbq = pick_bucket_scale<BITS>(nth);
+                bool n_ok = true;
+                for (int w = 0; w < n_builders; ++w) n_ok = n_ok && (n_slots[w] == 0);
+                const int r2 = lane >> 1, half = lane & 1;
+                float v[32];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const u32x4_t q = *reinterpret_cast<const u32x4_t *>(yt + r2 * 144 + half * 64 + i * 16);
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        v[8 * i + 2 * d] = __half2float(__ushort_as_half(static_cast<unsigned short>(q[d] & 0xffffu)));
+                        v[8 * i + 2 * d + 1] = __half2float(__ushort_as_half(static_cast<unsigned short>(q[d] >> 16)));
+                    }
+                }
+                float nmu, nvar, ns, nsum;
+                group_stats32x2(v, eps, nmu, nvar, ns);
+                group_codes32x2<BITS>(v, nmu, nvar, ns, nth, nbq, n_table, n_lut, n_ok, lane, nsum);
+                const float code_mean = nsum * 0.015625f;
+                if (m0 + r2 < M) {
+                    u32x4_t *dst = reinterpret_cast<u32x4_t *>(y + static_cast<int64_t>(m0 + r2) * N + n0 + half * 32);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        u32x4_t o;
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            const int j = 8 * i + 2 * d;
+                            const __half2 h = __floats2half2_rn(fma_f32(ns, v[j] - code_mean, nmu), fma_f32(ns, v[j + 1] - code_mean, nmu));
+                            o[d] = *reinterpret_cast<const uint32_t *>(&h);
+                        }
+                        dst[i] = o;
+                    }
+                }
+            }
+            return;
+        }
+    }
     if (gr < M && gc < N) {
         TOUT *dst = y + static_cast<int64_t>(gr) * N + gc;
         // Optional GELU / residual on the rounded output (post_op1): what separate elementwise kernels would store.
@@ -482,17 +548,21 @@ static void launch_os(const OtfSmallArgs &a, hipStream_t stream)
     const size_t tables = 2 * L * 64 * sizeof(float) + (kMaxBuckets + 64) * sizeof(Bucket) + 64;
     const size_t ln_bytes = a.ln_weight ? kOsWaves * 128 * sizeof(float) : 0;
     // Both regions side by side while they fit 160 KB of LDS; else the partial tiles reuse the x_hat tile's space.
-    const int partial_off = (tile_bytes + partial_bytes + tables + ln_bytes <= 160 * 1024) ? tile_bytes : 0;
+    const size_t nx_need = a.next_thr ? L * 64 * sizeof(float) + (kMaxBuckets + 64) * sizeof(Bucket) + 64 : 0;
+    const int partial_off = (tile_bytes + partial_bytes + tables + ln_bytes + nx_need <= 160 * 1024) ? tile_bytes : 0;
     const size_t front = partial_off ? tile_bytes + partial_bytes : (tile_bytes > partial_bytes ? tile_bytes : partial_bytes);
     const int ln_off = static_cast<int>(front + tables);
-    const size_t smem = front + tables + ln_bytes;
+    // (quantize-the-output mode: a second set of lookup tables, for the consuming layer's codebook)
+    const size_t nx_bytes = a.next_thr ? L * 64 * sizeof(float) + (kMaxBuckets + 64) * sizeof(Bucket) + 64 : 0;
+    const int nx_off = static_cast<int>(front + tables + ln_bytes);
+    const size_t smem = front + tables + ln_bytes + nx_bytes;
     auto kernel = otf_small_kernel<TIN, BITS, TOUT, RB, LPG, CB>;
     allow_dynamic_lds<otf_small_kernel<TIN, BITS, TOUT, RB, LPG, CB>>(160 * 1024);      // (the size varies with K: allow the CU's whole LDS)
     const dim3 grid((a.N + kOsCols - 1) / kOsCols, (a.M + RT - 1) / RT);
     hipLaunchKernelGGL(kernel, grid, dim3(kOsWaves * 64), smem, stream, static_cast<const TIN *>(a.x), a.a_thr, a.a_cb,
                        a.pw, a.w_cb, a.wc, a.ws, a.wcs, a.bias, static_cast<__half *>(a.x_hat_ws),
                        static_cast<TOUT *>(a.y), a.M, a.N, a.K, a.eps, tile_bytes, partial_off, a.ln_weight, a.ln_bias,
-                       a.ln_eps, ln_off, static_cast<const TOUT *>(a.residual), a.gelu ? 1 : 0);
+                       a.ln_eps, ln_off, static_cast<const TOUT *>(a.residual), a.gelu ? 1 : 0, a.next_thr, a.next_cb, nx_off);
 }
 
 template <typename TIN, int BITS, typename TOUT>
@@ -502,7 +572,8 @@ static void launch_os_rb(const OtfSmallArgs &a, hipStream_t stream)
     // 32-column tiles while their grid fits the chip in one wave of workgroups: half the weight rows to rebuild per wave
     // and half the reduction, at the price of twice as many workgroups repeating stage 1 (M = 197, K = 384:
     // N = 1152, 252 tiles, 8.9 -> 8.0 us; N = 384 8.7 -> 7.6; N = 1536, 336 tiles, 8.7-9.4 -> 10.0).  Bit-identical.
-    const bool narrow = static_cast<int64_t>((a.N + 31) / 32) * ((a.M + 31) / 32) <= 256;
+    // (quantizing the output for the next layer needs a whole group per tile row: 64 columns)
+    const bool narrow = !a.next_thr && static_cast<int64_t>((a.N + 31) / 32) * ((a.M + 31) / 32) <= 256;
     if (32 * (a.K / 64) <= 8 * 32) {
         if (narrow) launch_os<TIN, BITS, TOUT, 1, 2, 1>(a, stream);
         else launch_os<TIN, BITS, TOUT, 1, 2, 2>(a, stream);

@@ -378,16 +378,26 @@ def quantize_activation_blocked_ln(x: torch.Tensor, ln_weight: torch.Tensor, ln_
     return out
 
 
+def xhat_layout(m: int) -> int:
+    """Layout of an ``x_hat`` passed between two chained layers (``linear_otf_ex`` with ``next_quant`` / ``x_is_xhat``):
+    0 = row-major, 1 = the 32-row block layout."""
+    return int(_lib.load().arcq_xhat_layout(int(m)))
+
+
 def linear_otf_ex(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch.Tensor, packed_w: torch.Tensor,
                   w_codebook: torch.Tensor, w_center: torch.Tensor, w_scale: torch.Tensor, w_code_sum: torch.Tensor,
                   bias: Optional[torch.Tensor], bits: int, group_size: int, out_dtype: torch.dtype = torch.float16,
                   layernorm=None, gelu: bool = False, residual: Optional[torch.Tensor] = None,
-                  x_hat_ws: Optional[torch.Tensor] = None, w_hat_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  x_hat_ws: Optional[torch.Tensor] = None, w_hat_ws: Optional[torch.Tensor] = None,
+                  next_quant=None, x_is_xhat: bool = False) -> torch.Tensor:
     """``residual + gelu(linear(stage1(LayerNorm(x))))`` with the optional parts fused into the layer's two launches
     (``arcq_linear_otf_ex``): ``layernorm = (weight, bias, eps)`` or None, ``residual`` ``[M, N]`` of ``out_dtype`` or
     None.  Below 512 rows the whole layer with its options is one launch (or stage 1 + the split-K kernel with the
     GELU / residual in its epilogue); from 512 rows on the block-layout path.  Raises ``RuntimeError`` where the
-    library does not fuse (LayerNorm with K > 1024 from 512 rows on, K > 1536 below)."""
+    library does not fuse (LayerNorm with K > 1024 from 512 rows on, K > 1536 below).
+    ``next_quant = (thresholds, codebook)`` of the layer that consumes the output: the result is that layer's ``x_hat``
+    (stage 1 applied to the rounded output) in the layout ``xhat_layout(M)`` instead of the output itself; that layer is
+    then called with ``x_is_xhat=True`` (its own stage 1 is skipped)."""
     _check(x.is_cuda and packed_w.is_cuda, "x and packed_w must be CUDA tensors")
     _check(x.dim() == 2, "x must have shape [M, K]")
     _check_bits(bits)
@@ -410,6 +420,13 @@ def linear_otf_ex(x: torch.Tensor, a_thresholds: torch.Tensor, a_codebook: torch
         lw, lb = _f32c(lw), _f32c(lb)
         keep += [lw, lb]
         a.producer, a.ln_weight, a.ln_bias, a.ln_eps = _lib.ARCQ_PRODUCER_LAYERNORM, _ptr(lw), _ptr(lb), float(eps)
+    if x_is_xhat:
+        _check(layernorm is None and x.dtype == torch.float16, "x_is_xhat: x must be float16 and takes no LayerNorm")
+        a.producer = _lib.ARCQ_PRODUCER_XHAT
+    if next_quant is not None:
+        nt, nc = _f32c(next_quant[0]), _f32c(next_quant[1])
+        keep += [nt, nc]
+        a.next_a_thresholds, a.next_a_codebook = _ptr(nt), _ptr(nc)
     a.activation = _lib.ARCQ_ACT_GELU if gelu else _lib.ARCQ_ACT_NONE
     (a.a_thresholds, a.a_codebook, a.packed_w, a.w_codebook, a.w_center, a.w_scale, a.w_code_sum,
      a.bias) = [_ptr(t) or None for t in keep[:8]]

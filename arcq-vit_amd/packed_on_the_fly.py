@@ -141,13 +141,24 @@ class ARCQPackedLinearOnTheFly(nn.Module):
                 self._buffers[name] = orig.to(device=new.device)
         return self
 
+    def can_quantize_for(self, consumer: nn.Module, rows: int) -> bool:
+        """Whether ``forward(..., quantize_for=consumer)`` is available: this layer's launch then ends with the
+        consumer's stage 1 (the consumer is called with ``input_is_xhat=True``).  Built for fewer than 512 rows."""
+        return (isinstance(consumer, ARCQPackedLinearOnTheFly) and not self.fp8_operands and not consumer.fp8_operands
+                and 0 < rows < 512 and self.group_size == 64 and consumer.group_size == 64 and self.bits == consumer.bits
+                and consumer.in_features == self.out_features and self.out_features % 64 == 0
+                and self.in_features % 64 == 0 and self.in_features <= 1536 and self.out_dtype == torch.float16)
+
     def forward(self, x: torch.Tensor, layernorm: Optional[nn.LayerNorm] = None, activation: Optional[str] = None,
-                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+                residual: Optional[torch.Tensor] = None, quantize_for: Optional[nn.Module] = None,
+                input_is_xhat: bool = False) -> torch.Tensor:
         """``residual + activation(linear(stage1(layernorm(x))))``.  The three optional parts (the LayerNorm in front
         of the layer, ``activation="gelu"`` and the skip connection behind it, as they surround the block linears in
         timm's ``Block``, FQ/timm_quant_models.py:63-121) are fused into the layer's launches where the library can
         (group size 64; for the LayerNorm K <= 1024 from 512 rows on and K <= 1536 below) and run as separate torch
-        operations otherwise; without them this is the reference module's forward."""
+        operations otherwise; without them this is the reference module's forward.  ``quantize_for=consumer`` (see
+        ``can_quantize_for``): the result is the consumer's ``x_hat`` instead of this layer's output, to be passed to
+        ``consumer(..., input_is_xhat=True)``, which skips its own stage 1."""
         original_shape = x.shape
         if original_shape[-1] != self.in_features:
             raise ValueError(f"expected last dim {self.in_features}, got {original_shape[-1]}")
@@ -160,11 +171,18 @@ class ARCQPackedLinearOnTheFly(nn.Module):
             x2 = x2.to(torch.float16)
         x2 = x2.contiguous()
         m = x2.shape[0]
-        extras = layernorm is not None or activation is not None or residual is not None
+        chain = quantize_for is not None or input_is_xhat
+        if quantize_for is not None and not self.can_quantize_for(quantize_for, m):
+            raise ValueError("quantize_for: not available for this pair of layers / number of rows (see can_quantize_for)")
+        if input_is_xhat and (x2.dtype != torch.float16 or layernorm is not None or self.fp8_operands):
+            raise ValueError("input_is_xhat: x must be the float16 x_hat a producer made for this layer")
+        ln_fusable = layernorm is None or (self.in_features <= (1024 if m >= 512 else 1536) and layernorm.elementwise_affine
+                                           and tuple(layernorm.normalized_shape) == (self.in_features,))
+        if chain and not ln_fusable:     # (a chained call cannot fall back as a whole: only the LayerNorm runs apart)
+            x2, layernorm, ln_fusable = layernorm(x2).contiguous(), None, True
+        extras = layernorm is not None or activation is not None or residual is not None or chain
         fuse = (extras and not self.fp8_operands and m > 0 and self.group_size == 64 and self.in_features % 64 == 0
-                and (layernorm is None or (self.in_features <= (1024 if m >= 512 else 1536)
-                                           and layernorm.elementwise_affine
-                                           and tuple(layernorm.normalized_shape) == (self.in_features,))))
+                and ln_fusable)
         if extras and not fuse:          # separate operations around the plain layer
             if layernorm is not None:
                 x2 = layernorm(x2)
@@ -224,6 +242,14 @@ class ARCQPackedLinearOnTheFly(nn.Module):
                 a.activation = _lib.ARCQ_ACT_GELU if activation == "gelu" else _lib.ARCQ_ACT_NONE
                 (a.a_thresholds, a.a_codebook, a.packed_w, a.w_codebook, a.w_center, a.w_scale, a.w_code_sum,
                  a.bias) = [v or None for v in p]
+                if input_is_xhat:
+                    a.producer = _lib.ARCQ_PRODUCER_XHAT
+                if quantize_for is not None:
+                    nprep = quantize_for._prep
+                    if nprep is None or nprep[2] != quantize_for.packed_weight_codes.data_ptr():
+                        nprep = quantize_for._prepare()
+                        quantize_for._fp8_mult = None
+                    a.next_a_thresholds, a.next_a_codebook = nprep[1][0], nprep[1][1]
                 if residual is not None:
                     r2 = residual.reshape(-1, self.out_features)
                     if r2.dtype != self.out_dtype or tuple(r2.shape) != (m, self.out_features) or r2.device != x2.device:

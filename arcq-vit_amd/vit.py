@@ -72,12 +72,21 @@ class Block(nn.Module):
         # True (and the four linears on-the-fly packed layers): the LayerNorms, the GELU and the two skip connections
         # run inside the packed layers' launches (ARCQPackedLinearOnTheFly.forward's optional arguments).
         self.fuse_elementwise = False
+        # With fuse_elementwise: let fc1's launch end with fc2's stage 1 where the layers can (the GELU output then never
+        # exists as a tensor); results are the same bits either way.
+        self.chain_mlp = True
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.fuse_elementwise and isinstance(self.mlp.act, nn.GELU) and self.mlp.act.approximate == "none":
             a = self.attn
             x = a.proj(a.mix(a.qkv(x, layernorm=self.norm1)), residual=x)
-            return self.mlp.fc2(self.mlp.fc1(x, layernorm=self.norm2, activation="gelu"), residual=x)
+            fc1, fc2 = self.mlp.fc1, self.mlp.fc2
+            rows = x.numel() // x.shape[-1]
+            if self.chain_mlp and hasattr(fc1, "can_quantize_for") and fc1.can_quantize_for(fc2, rows):
+                # the GELU output is only ever consumed quantized: fc1's launch ends with fc2's stage 1
+                h = fc1(x, layernorm=self.norm2, activation="gelu", quantize_for=fc2)
+                return fc2(h, residual=x, input_is_xhat=True)
+            return fc2(fc1(x, layernorm=self.norm2, activation="gelu"), residual=x)
         x = x + self.attn(self.norm1(x))
         return x + self.mlp(self.norm2(x))
 

@@ -387,7 +387,8 @@ def chained_step(model, bits, batch, steps, warmup, dev):
     qkv(x) -> q; proj(the first M*dim values of q, standing in for the attention output) -> p; fc1(p) -> h; fc2(h) -> x.
     Two figures under one HIP graph per step: `plain` (arcq_linear_otf_ws per layer) and `fused` (arcq_linear_otf_ex:
     LayerNorm in front of qkv / fc1, GELU behind fc1, the skip connections behind proj / fc2 -- the work that sits
-    between the packed linears of a transformer block, inside their launches)."""
+    between the packed linears of a transformer block, inside their launches), and the latter with fc2's stage 1 inside
+    fc1's launch as well."""
     import ctypes
     import torch
     from arcq_vit_amd import _lib, synth
@@ -403,7 +404,7 @@ def chained_step(model, bits, batch, steps, warmup, dev):
     ln_b = torch.zeros(max(dim, hid), dtype=torch.float32, device=dev)
     keep = []
 
-    def ex(l, x, y, ln=False, gelu=False, res=None):
+    def ex(l, x, y, ln=False, gelu=False, res=None, nxt_layer=None, from_xhat=False):
         a = _lib.LinearExArgs()
         a.struct_size = ctypes.sizeof(_lib.LinearExArgs)
         a.x_dtype = a.y_dtype = ARCQ_F16
@@ -411,6 +412,10 @@ def chained_step(model, bits, batch, steps, warmup, dev):
         a.x, a.y, a.x_hat_ws, a.w_hat_ws = x.data_ptr(), y.data_ptr(), ws.data_ptr(), Layer.W_WS.data_ptr()
         if ln:
             a.producer, a.ln_weight, a.ln_bias, a.ln_eps = _lib.ARCQ_PRODUCER_LAYERNORM, ln_w.data_ptr(), ln_b.data_ptr(), 1e-6
+        if from_xhat:
+            a.producer = _lib.ARCQ_PRODUCER_XHAT
+        if nxt_layer is not None:
+            a.next_a_thresholds, a.next_a_codebook = nxt_layer.thr.data_ptr(), nxt_layer.cb.data_ptr()
         a.activation = _lib.ARCQ_ACT_GELU if gelu else _lib.ARCQ_ACT_NONE
         a.residual = None if res is None else res.data_ptr()
         a.a_thresholds, a.a_codebook, a.packed_w, a.w_codebook = l.thr.data_ptr(), l.cb.data_ptr(), l.packed.data_ptr(), l.cb.data_ptr()
@@ -424,9 +429,14 @@ def chained_step(model, bits, batch, steps, warmup, dev):
             qkv, proj, fc1, fc2 = layers[4 * b:4 * b + 4]
             mid, nxt = ring[r % 3], ring[(r + 1) % 3]       # cur is x0 or ring[(r + 2) % 3]
             r += 2
-            calls = ([ex(qkv, cur, q, ln=True), ex(proj, q, mid, res=cur), ex(fc1, mid, h, ln=True, gelu=True),
-                      ex(fc2, h, nxt, res=mid)] if fused else
-                     [ex(qkv, cur, q), ex(proj, q, mid), ex(fc1, mid, h), ex(fc2, h, nxt)])
+            if fused == "xhat":       # fc1's launch ends with fc2's stage 1; fc2 starts from that x_hat
+                calls = [ex(qkv, cur, q, ln=True), ex(proj, q, mid, res=cur),
+                         ex(fc1, mid, h, ln=True, gelu=True, nxt_layer=fc2), ex(fc2, h, nxt, res=mid, from_xhat=True)]
+            elif fused:
+                calls = [ex(qkv, cur, q, ln=True), ex(proj, q, mid, res=cur), ex(fc1, mid, h, ln=True, gelu=True),
+                         ex(fc2, h, nxt, res=mid)]
+            else:
+                calls = [ex(qkv, cur, q), ex(proj, q, mid), ex(fc1, mid, h), ex(fc2, h, nxt)]
             for a in calls:
                 rc = lib.arcq_linear_otf_ex(ctypes.byref(a), stream)
                 if rc:
@@ -434,7 +444,10 @@ def chained_step(model, bits, batch, steps, warmup, dev):
             cur = nxt
 
     out = {}
-    for name, fused in (("plain", False), ("fused", True)):
+    variants = [("plain", False), ("fused", True)]
+    if lib.arcq_xhat_layout(m) == 0:          # (chaining fc1 -> fc2 through x_hat is built for fewer than 512 rows)
+        variants.append(("fused_mlp_chained_through_x_hat", "xhat"))
+    for name, fused in variants:
         run(fused, torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()

@@ -220,6 +220,7 @@ int arcq_linear_fused_blocked(const void *x_hat_blocked,
  * struct_size = sizeof(arcq_linear_ex_args). */
 #define ARCQ_PRODUCER_NONE 0
 #define ARCQ_PRODUCER_LAYERNORM 1
+#define ARCQ_PRODUCER_XHAT 2
 #define ARCQ_ACT_NONE 0
 #define ARCQ_ACT_GELU 1
 typedef struct arcq_linear_ex_args {
@@ -234,8 +235,24 @@ typedef struct arcq_linear_ex_args {
     const float *w_codebook, *w_center, *w_scale, *w_code_sum, *bias;
     const void *residual;
     void *x_hat_ws, *w_hat_ws, *y;
+    /* fields added after the first version of this struct (a caller that passes the shorter struct_size gets NULL) */
+    const float *next_a_thresholds, *next_a_codebook;
 } arcq_linear_ex_args;
 int arcq_linear_otf_ex(const arcq_linear_ex_args *args, void *stream);
+
+/* Two layers chained through their quantizer (fc1 -> GELU -> fc2 of the block: the GELU output is only ever consumed
+ * quantized, FQ/arcq_packed_on_the_fly.py:139-145 is the stage-1 call that disappears).
+ *   next_a_thresholds / next_a_codebook set (the activation quantizer of the layer that consumes y; same bits, group
+ *   size 64, N a multiple of 64, y_dtype ARCQ_F16): y receives, instead of the layer's output, that output's
+ *   reconstruction x_hat = stage1(post-processed, fp16-rounded output), fp16, in the layout arcq_xhat_layout(M) --
+ *   exactly what the consuming layer's stage 1 would have produced from the stored output, bit for bit.
+ *   producer == ARCQ_PRODUCER_XHAT on the consuming layer's call: x [M,K] fp16 already is that x_hat in
+ *   arcq_xhat_layout(M); stage 1 is skipped (a_thresholds / a_codebook are not read) and the call runs stages 2+3 with
+ *   the optional GELU / residual.
+ * arcq_xhat_layout: 0 = row-major [M,K] (fewer than 512 rows), 1 = the 32-row block layout described above.
+ * Both return ARCQ_ERR_UNSUPPORTED for shapes the kernels that hold a whole group per output row do not serve; the
+ * caller then runs the two layers the ordinary way. */
+int arcq_xhat_layout(int64_t M);
 
 /* LayerNorm + stage 1 into the block layout in one launch (the first half of arcq_linear_otf_ex with
  * ARCQ_PRODUCER_LAYERNORM), exposed so that it can be called and tested on its own; no counterpart in the

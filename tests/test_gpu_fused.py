@@ -129,6 +129,32 @@ def test_linear_otf_ex_equals_the_unfused_sequence(cuda, oracle, m, n, k, bits, 
         assert np.all(np.abs(got - g64) <= step)
 
 
+@pytest.mark.parametrize("m,k,h,bits", [(197, 384, 1536, 4), (100, 384, 1536, 3), (197, 192, 768, 4), (33, 768, 3072, 4),
+                                        (1, 64, 64, 2)])
+def test_two_layers_chained_through_x_hat(cuda, oracle, m, k, h, bits):
+    """fc1 -> GELU -> fc2 with fc2's stage 1 inside fc1's launch (next_quant / x_is_xhat): the x_hat handed over equals
+    the oracle's stage 1 of the stored GELU output bit for bit, and fc2's result equals the unfused sequence's."""
+    pw1, cb, wc1, ws1, wcs1 = _weights(oracle, h, k, bits, 51)
+    pw2, _, wc2, ws2, wcs2 = _weights(oracle, k, h, bits, 52)
+    _, thr = _cb(bits)
+    cb2 = cb * 1.1                                   # the consumer's own quantizer, different from the producer's
+    thr2 = synth.midpoint_thresholds(cb2)
+    b1, b2 = synth.make_bias(h, 51), synth.make_bias(k, 52)
+    lw, lb = _ln_params(k, 9)
+    x = (synth.make_activation(m, k, 53, "ln") * 1.2).to(torch.float16)
+    d = lambda t: t.to(cuda)
+    a1 = (d(thr), d(cb), d(pw1), d(cb), d(wc1), d(ws1), d(wcs1), d(b1), bits, 64)
+    a2 = (d(thr2), d(cb2), d(pw2), d(cb), d(wc2), d(ws2), d(wcs2), d(b2), bits, 64)
+    ln = (d(lw), d(lb), 1e-6)
+    assert ops.xhat_layout(m) == 0
+    xhat = ops.linear_otf_ex(d(x), *a1, layernorm=ln, gelu=True, next_quant=(d(thr2), d(cb2)))
+    y = ops.linear_otf_ex(xhat, *a2, residual=d(x), x_is_xhat=True)
+    g = ops.linear_otf_ex(d(x), *a1, layernorm=ln, gelu=True)                     # the stored GELU output
+    want_xhat = oracle.act_quant_c(_np(g).astype(np.float32), thr2, cb2, bits, 64)["x_hat"].astype(np.float16)
+    assert xhat.dtype == torch.float16 and np.array_equal(_np(xhat).view(np.uint16), want_xhat.view(np.uint16))
+    assert torch.equal(y, ops.linear_otf_ex(g, *a2, residual=d(x)))
+
+
 def test_linear_otf_ex_fp32_and_limits(cuda, oracle):
     n, k, bits = 256, 384, 4
     pw, cb, wc, ws, wcs = _weights(oracle, n, k, bits, 41)
@@ -167,7 +193,8 @@ def test_vit_block_fusion(cuda, oracle, model, batch):
     output, captured by forward hooks, equals the oracle's value of the same fused layer on the captured input
     (LayerNorm restatement -> stage 1 -> fp64 product -> GELU / residual in fp16), and the logits stay close to the
     unfused model's (whose LayerNorm is torch's kernel: another summation order, so codes may differ at ties).  Batch 2
-    (394 rows) takes the small-M kernels: one launch per layer with everything inside, fc2 as stage 1 + split-K."""
+    (394 rows) takes the small-M kernels: one launch per layer with everything inside; the layers are hooked with fc1 and
+    fc2 called separately, and the model with fc2's stage 1 inside fc1's launch must then give the same logits bit for bit."""
     kw = dict(num_classes=100, device="cuda", half_chain=True, depth=2, shared_buffers=True, max_rows=batch * synth.TOKENS)
     fused = build_packed_vit(model, 4, fuse_elementwise=True, **kw)
     plain = build_packed_vit(model, 4, fuse_elementwise=False, **kw)
@@ -184,10 +211,16 @@ def test_vit_block_fusion(cuda, oracle, model, batch):
 
     hooks = [m.register_forward_hook(hook, with_kwargs=True) for m in fused.modules()
              if isinstance(m, A.ARCQPackedLinearOnTheFly)]
+    for blk in fused.blocks:
+        blk.chain_mlp = False
     with torch.no_grad():
         lf, lp = fused(x), plain(x)
     for h in hooks:
         h.remove()
+    for blk in fused.blocks:
+        blk.chain_mlp = True
+    with torch.no_grad():
+        assert torch.equal(fused(x), lf)
     assert bool(torch.isfinite(lf).all())
     assert len(captured) == 8
     for mod, ln, act, x2, r2, y in captured:
