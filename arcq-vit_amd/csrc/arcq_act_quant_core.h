@@ -270,4 +270,143 @@ __device__ __forceinline__ void group_codes32x2(float (&xv)[32], float mu, float
     sum_out = pair_serial_sum(xv);
 }
 
+// The same with the thresholds of the compare-chain fallback read from LDS in a rolled loop (`th_lds`, L - 1 values)
+// instead of held in registers: for callers that have no registers to keep them in (a GEMM's epilogue).  Same results.
+template <int BITS>
+__device__ __forceinline__ void group_codes32x2_lds(float (&xv)[32], float mu, float var, float s, const float *th_lds,
+                                                    const BucketScale &bq, const Bucket *table, const float *lut,
+                                                    bool table_ok, int lane, float &sum_out)
+{
+    constexpr int L = 1 << BITS;
+    const bool lane_fast = (s >= 0x1p-60f) && (s <= 0x1p60f) && !(fabsf(mu) < 0x1p-66f && var > 0.0f);
+    const bool fast = table_ok && __all(lane_fast);
+    if (fast) {
+        const float y = 1.0f / s;
+        const float ns = -s;
+        const char *lut_lane = reinterpret_cast<const char *>(lut) + lane * 4;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            const float d = xv[j];
+            float q = d * y;
+            float e = __fmaf_rn(ns, q, d);
+            q = __fmaf_rn(e, y, q);
+            e = __fmaf_rn(ns, q, d);
+            q = __fmaf_rn(e, y, q);        // == RN(d / s)
+            const Bucket bk = *reinterpret_cast<const Bucket *>(reinterpret_cast<const char *>(table) + bucket_offset_of(q, bq));
+            const uint32_t c = static_cast<uint32_t>(bk.base) + ((q > bk.thr) ? 1u : 0u);
+            xv[j] = *reinterpret_cast<const float *>(lut_lane + (c << 8));
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 32; ++j) xv[j] = xv[j] / s;
+#pragma unroll 1
+        for (int j = 0; j < 32; ++j) {
+            // (element j of a register array under a rolled loop: select it with a compare chain instead of indexing)
+            float t = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 32; ++q) t = (q == j) ? xv[q] : t;
+            uint32_t c = 0;
+            bool alive = true;
+#pragma unroll 1
+            for (int i = 0; i < L - 1; ++i) {   // while (c < L-1 && t > thr[c]) ++c
+                alive = alive && (t > th_lds[i]);
+                c += alive ? 1u : 0u;
+            }
+            const float v = lut[c * 64 + lane];
+#pragma unroll
+            for (int q = 0; q < 32; ++q) xv[q] = (q == j) ? v : xv[q];
+        }
+    }
+    sum_out = pair_serial_sum(xv);
+}
+
+// ---- stage 1 of the NEXT layer inside a GEMM's epilogue ----------------------------------------------------------
+// The block-layout GEMM kernels stage their outputs 32 rows x 64 fp16 columns at a time in a wave-private LDS tile
+// (`pitch` bytes per row) -- one quantization group per row.  When the layer's output is only ever consumed quantized
+// (fc1 -> GELU -> fc2) the wave quantizes the staged chunk right there, exactly as the consuming layer's stage 1 would
+// have done on the stored tensor (two lanes per group, same arithmetic, same bits), and writes x_hat into the
+// consumer's 32-row block layout.  The consumer's lookup tables live in LDS (built once per workgroup by
+// next_quant_setup).
+// LDS of the consumer's quantizer: [codebook per lane: L x 64 floats][buckets][per-wave flags: 64 bytes]
+// [thresholds: 16 floats][bucket geometry: scale, offset, number of buckets].
+constexpr int next_quant_lds_bytes(int bits) { return (1 << bits) * 64 * 4 + (kMaxBuckets + 64) * 8 + 64 + 64 + 16; }
+
+// All `nthreads` threads of the workgroup call this (before a barrier that precedes the first epilogue): the
+// consumer's lookup tables into `lds` (next_quant_lds_bytes(BITS) bytes, 16-byte aligned).
+template <int BITS>
+__device__ __forceinline__ void next_quant_setup(const float *__restrict__ thr, const float *__restrict__ cb,
+                                                 unsigned char *lds, int tid, int nthreads)
+{
+    constexpr int L = 1 << BITS;
+    float th[L - 1], cbv[L];
+    load_quant_params<BITS>(thr, cb, th, cbv);
+    const BucketScale bq = pick_bucket_scale<BITS>(th);
+    float *lut = reinterpret_cast<float *>(lds);
+    Bucket *table = reinterpret_cast<Bucket *>(lut + L * 64);
+    int *slots = reinterpret_cast<int *>(table + kMaxBuckets + 64);
+    build_quant_tables_by<BITS>(th, cbv, bq, lut, table, slots, tid, nthreads);
+    float *th_lds = reinterpret_cast<float *>(slots + 16);
+    if (tid == 0) {
+#pragma unroll
+        for (int i = 0; i < L - 1; ++i) th_lds[i] = th[i];
+        th_lds[16] = bq.scale;
+        th_lds[17] = bq.offset;
+        reinterpret_cast<int *>(th_lds)[18] = bq.nb;
+    }
+}
+
+// One staged chunk (32 rows x 64 fp16 values, the rows `pitch` bytes apart) -> x_hat of the consuming layer.
+// `gelu`: the exact GELU of the staged (rounded) values first, rounded to fp16 again.  dst_block = base of the chunk's
+// 32-row block in the consumer's block layout, `rows` = rows of that block (32, or fewer for a last block),
+// piece0 = index of the chunk's first 16-byte piece (column / 8).  The whole wave calls it.
+template <int BITS>
+__device__ __forceinline__ void next_quant_chunk(const unsigned char *lds, int nwaves,
+                                                 const unsigned char *stage, int pitch, int lane, bool gelu, float eps,
+                                                 __half *dst_block, int rows, int piece0)
+{
+    typedef uint32_t u32x4_nq __attribute__((ext_vector_type(4)));
+    constexpr int L = 1 << BITS;
+    const float *lut = reinterpret_cast<const float *>(lds);
+    const Bucket *table = reinterpret_cast<const Bucket *>(lut + L * 64);
+    const int *slots = reinterpret_cast<const int *>(table + kMaxBuckets + 64);
+    const float *th_lds = reinterpret_cast<const float *>(slots + 16);
+    BucketScale bq;
+    bq.scale = th_lds[16];
+    bq.offset = th_lds[17];
+    bq.nb = reinterpret_cast<const int *>(th_lds)[18];
+    const int r = lane >> 1, hf = lane & 1;
+    float v[32];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const u32x4_nq q = *reinterpret_cast<const u32x4_nq *>(stage + r * pitch + hf * 64 + i * 16);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            v[8 * i + 2 * d] = __half2float(__ushort_as_half(static_cast<unsigned short>(q[d] & 0xffffu)));
+            v[8 * i + 2 * d + 1] = __half2float(__ushort_as_half(static_cast<unsigned short>(q[d] >> 16)));
+        }
+    }
+    if (gelu) {
+#pragma unroll
+        for (int j = 0; j < 32; ++j) v[j] = __half2float(__float2half_rn(gelu_f32(v[j])));
+    }
+    bool ok = true;
+    for (int w = 0; w < nwaves; ++w) ok = ok && (slots[w] == 0);
+    float mu, var, s, sum;
+    group_stats32x2(v, eps, mu, var, s);
+    group_codes32x2_lds<BITS>(v, mu, var, s, th_lds, bq, table, lut, ok, lane, sum);
+    const float code_mean = sum * 0.015625f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t o[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const int j = 8 * i + 2 * d;
+            const __half2 h = __floats2half2_rn(fma_f32(s, v[j] - code_mean, mu), fma_f32(s, v[j + 1] - code_mean, mu));
+            o[d] = *reinterpret_cast<const uint32_t *>(&h);
+        }
+        if (r < rows)
+            store_writethrough16(dst_block + (static_cast<int64_t>(piece0 + hf * 4 + i) * rows + r) * 8, o[0], o[1], o[2], o[3]);
+    }
+}
+
 }  // namespace arcq

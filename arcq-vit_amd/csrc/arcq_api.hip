@@ -253,14 +253,26 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
                                        a->y, a->y_dtype, a->M, a->N, a->K, a->bits, 64, stream, a->residual,
                                        a->activation == ARCQ_ACT_GELU);
     }
-    if (from_xhat || next_thr)
-        return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: chaining two layers through x_hat is built for fewer than 512 rows");
     if (!arcq::otf_blocked_pays(a->M, a->N, a->K))
         return arcq::fail(ARCQ_ERR_UNSUPPORTED,
                           "arcq_linear_otf_ex: the fused options need in_features a positive multiple of 64 and a shape the "
                           "block-layout kernels run (got M=%lld K=%lld)", static_cast<long long>(a->M),
                           static_cast<long long>(a->K));
-    if (a->w_hat_ws && a->x_dtype == ARCQ_F16 &&
+    // From 512 rows on two chained layers hand x_hat over in the 32-row block layout.  The consumer runs stages 2+3 on
+    // it (the weights rebuilt into the workspace first where that pays); the producer is the block-layout GEMM on
+    // copied weights with the consumer's stage 1 in its epilogue (which needs the weight workspace).
+    if (from_xhat) {
+        if (next_thr)
+            return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: a layer that starts from x_hat cannot quantize its output "
+                              "for the next one");
+        return arcq::linear_fused_blocked(a->x, a->packed_w, a->w_codebook, a->w_center, a->w_scale, a->w_code_sum, a->bias,
+                                          a->w_hat_ws, false, a->y, a->y_dtype, a->M, a->N, a->K, a->bits, a->group_size, stream,
+                                          a->residual, a->activation == ARCQ_ACT_GELU);
+    }
+    if (next_thr && (!a->w_hat_ws || a->residual))
+        return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: from 512 rows on quantizing the output for the next layer needs "
+                          "w_hat_ws and no residual");
+    if (!next_thr && a->w_hat_ws && a->x_dtype == ARCQ_F16 &&
         arcq::otf_rows_pays(a->M, a->N, a->K, a->producer == ARCQ_PRODUCER_LAYERNORM) && a->x && a->a_thresholds &&
         a->a_codebook && a->packed_w && a->w_codebook && a->w_center && a->w_scale && a->w_code_sum && a->y &&
         (a->y_dtype == ARCQ_F16 || a->y_dtype == ARCQ_F32) && arcq::aligned(a->x, 16) && arcq::aligned(a->y, 16) &&
@@ -275,8 +287,11 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
         const int rc = arcq::launch_otf_rows(r, static_cast<hipStream_t>(stream));
         if (rc != arcq::kNotLaunched) return rc;
     }
-    const bool carry = a->w_hat_ws && arcq::blocked_uses_workspace(a->N, a->K) && a->packed_w && a->w_codebook && a->w_center &&
-                       a->w_scale && a->w_code_sum && arcq::aligned(a->w_hat_ws, 16) && arcq::aligned(a->packed_w, 16);
+    const bool carry = a->w_hat_ws && (next_thr || arcq::blocked_uses_workspace(a->N, a->K)) && a->packed_w && a->w_codebook &&
+                       a->w_center && a->w_scale && a->w_code_sum && arcq::aligned(a->w_hat_ws, 16) && arcq::aligned(a->packed_w, 16);
+    if (next_thr && !carry)
+        return arcq::fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_otf_ex: quantizing the output for the next layer needs a 16-byte aligned "
+                          "weight workspace and packed weights");
     int rc;
     if (a->producer == ARCQ_PRODUCER_LAYERNORM) {
         if (a->K > 1024)
@@ -295,7 +310,7 @@ ARCQ_API int arcq_linear_otf_ex(const arcq_linear_ex_args *a, void *stream)
     if (rc != ARCQ_OK) return rc;
     return arcq::linear_fused_blocked(a->x_hat_ws, a->packed_w, a->w_codebook, a->w_center, a->w_scale, a->w_code_sum, a->bias,
                                       a->w_hat_ws, carry, a->y, a->y_dtype, a->M, a->N, a->K, a->bits, a->group_size, stream,
-                                      a->residual, a->activation == ARCQ_ACT_GELU);
+                                      a->residual, a->activation == ARCQ_ACT_GELU, next_thr, next_cb);
 }
 
 ARCQ_API int arcq_xhat_layout(int64_t M) { return M < 512 ? 0 : 1; }

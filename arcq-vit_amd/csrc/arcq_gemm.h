@@ -20,6 +20,10 @@ struct GemmArgs {
     // keep them away from the others.
     const void *residual = nullptr;   // [M,N] of y's type, or nullptr
     bool gelu = false;
+    // Quantize-the-output mode of the block-layout kernels fed from reconstructed weights: y (fp16, N a multiple of 64)
+    // receives stage 1 of the layer that consumes this one's output (its thresholds / codebook, `bits` levels) in
+    // that layer's 32-row block layout.  No residual in this mode.
+    const float *next_thr = nullptr, *next_cb = nullptr;
 };
 
 // Large-M kernel (256-column x up-to-256-row workgroup tiles); requires K >= 64.
@@ -46,7 +50,8 @@ bool blocked_uses_workspace(int64_t N, int64_t K);
 int linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_w, const float *w_codebook,
                          const float *w_center, const float *w_scale, const float *w_code_sum, const float *bias,
                          void *w_hat_ws, bool w_hat_ready, void *y, int y_dtype, int64_t M, int64_t N, int64_t K, int bits,
-                         int group_size, void *stream, const void *residual = nullptr, bool gelu = false);
+                         int group_size, void *stream, const void *residual = nullptr, bool gelu = false,
+                         const float *next_thr = nullptr, const float *next_cb = nullptr);
 
 
 // Small-M kernel (64 x 64 tiles, K split across the waves of a workgroup); requires K >= 64.

@@ -428,7 +428,8 @@ ARCQ_API int arcq_linear_fused_blocked(const void *x_hat_blocked,
 int arcq::linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_w, const float *w_codebook,
                                const float *w_center, const float *w_scale, const float *w_code_sum, const float *bias,
                                void *w_hat_ws, bool w_hat_ready, void *y, int y_dtype, int64_t M, int64_t N, int64_t K,
-                               int bits, int group_size, void *stream, const void *residual, bool gelu)
+                               int bits, int group_size, void *stream, const void *residual, bool gelu,
+                               const float *next_thr, const float *next_cb)
 {
     if (!bits_ok(bits)) return fail(ARCQ_ERR_BITS, "arcq_linear_fused_blocked: bits must be 2, 3, or 4");
     if (group_size != 64) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_fused_blocked: group_size must be 64 (got %d)", group_size);
@@ -444,8 +445,13 @@ int arcq::linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_
         return fail(ARCQ_ERR_SHAPE, "arcq_linear_fused_blocked: M, N or K too large");
     if (!aligned(x_hat_blocked, 16) || !aligned(y, 16) || !aligned(packed_w, 16) || !aligned(w_hat_ws, 16))
         return fail(ARCQ_ERR_ALIGN, "arcq_linear_fused_blocked: x_hat_blocked, y, packed_w and w_hat_ws must be 16-byte aligned");
+    if (next_thr) {          // y receives the consuming layer's x_hat: built into the kernels that copy reconstructed weights
+        if (!next_cb || !w_hat_ws || y_dtype != ARCQ_F16 || N % 64 != 0 || residual)
+            return fail(ARCQ_ERR_UNSUPPORTED, "arcq_linear_fused_blocked: quantizing the output for the next layer needs a weight "
+                        "workspace, a float16 output, out_features a multiple of 64 and no residual");
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const bool prebuilt = w_hat_ws && (w_hat_ready || workspace_pays_blocked(N, K));
+    const bool prebuilt = w_hat_ws && (w_hat_ready || next_thr || workspace_pays_blocked(N, K));
     if (prebuilt && !w_hat_ready) {
         const int rc = arcq_weight_dequant(packed_w, w_codebook, w_center, w_scale, w_code_sum, w_hat_ws, ARCQ_F16, N, K,
                                            bits, group_size, stream);
@@ -455,6 +461,8 @@ int arcq::linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_
                static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), bits};
     g.residual = residual;
     g.gelu = gelu;
+    g.next_thr = next_thr;
+    g.next_cb = next_cb;
     launch_gemm_slab8(g, prebuilt ? w_hat_ws : nullptr, st);
     return launch_status("arcq_linear_fused_blocked");
 }

@@ -15,6 +15,7 @@
 // arrive.  Left-over blocks of a workgroup (fewer than sixteen) are dealt as pairs, single blocks and column halves.
 #include "arcq_common.h"
 #include "arcq_gemm.h"
+#include "arcq_act_quant_core.h"
 
 #include <stdlib.h>
 #include <type_traits>
@@ -52,12 +53,16 @@ template <int V> __device__ __forceinline__ void wait_vmcnt()
     asm volatile("" ::: "memory");
 }
 
-template <typename TOUT, int WAVES, int SG, bool DB>
+// NQ = 0, or the bits (2 / 3 / 4) of the activation quantizer of the layer that consumes this one's output: y then
+// receives that layer's x_hat (stage 1 of the rounded, optionally GELU'd output) in the block layout instead of the
+// output itself (arcq_act_quant_core.h, next_quant_chunk); fp16 output and N a multiple of 64 only.
+template <typename TOUT, int WAVES, int SG, bool DB, int NQ>
 __global__ void __launch_bounds__(64 * WAVES)
 gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K,
                  int row_ranges, int blocks_per_range, const __half *__restrict__ w_hat,
-                 const TOUT *__restrict__ residual, int gelu)
+                 const TOUT *__restrict__ residual, int gelu, const float *__restrict__ nx_thr, const float *__restrict__ nx_cb)
 {
+    static_assert(NQ == 0 || sizeof(TOUT) == 2, "the next layer's stage 1 works on fp16 outputs");
     constexpr int kWaves = WAVES;
     constexpr int kSliceGroups = SG;
     constexpr int kPieces = PairCfg<WAVES, SG, DB>::kPieces;
@@ -98,6 +103,9 @@ gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, 
     unsigned char *stage = smem + kAllSlabs + wave * kStageTile;
 
     if (tid < kSlabN) s_bias[tid] = (bias && n_base + tid < N) ? bias[n_base + tid] : 0.0f;
+    const unsigned char *nq_lds = smem + PairCfg<WAVES, SG, DB>::kSmem;
+    if constexpr (NQ != 0)      // (the barriers of the first slab fill publish the tables)
+        next_quant_setup<NQ>(nx_thr, nx_cb, smem + PairCfg<WAVES, SG, DB>::kSmem, tid, 64 * WAVES);
     // Direct global -> LDS loads: the slab is filled as one flat run of 16-byte pieces (piece p = row * kPieces +
     // column; the hardware writes lane l's piece at the wave-uniform LDS base + 16 l), 64 pieces per instruction
     // whatever the row length; padding pieces and the columns past a short last slice are skipped.  The caller
@@ -274,6 +282,15 @@ gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, 
                     }
                 }
                 __builtin_amdgcn_wave_barrier();
+                if constexpr (NQ != 0) {
+                    const int c0 = n_base + jb * 32 + ch * kChunkCols;          // the chunk is one group of the consumer's rows
+                    if (c0 < N)
+                        next_quant_chunk<NQ>(nq_lds, kWaves, stage, kStageRow, lane, gelu != 0, 1.0e-6f,
+                                             reinterpret_cast<__half *>(y) + static_cast<int64_t>(pblk) * 32 * N,
+                                             min(32, M - pblk * 32), c0 / 8);
+                    __builtin_amdgcn_wave_barrier();
+                    continue;
+                }
                 const int col = n_base + jb * 32 + ch * kChunkCols + (lane & 7) * kVec;
                 const int row0 = pblk * 32 + (lane >> 3);
                 TOUT *dst0 = y + static_cast<int64_t>(row0) * N + col;
@@ -459,18 +476,18 @@ gemm_pair_kernel(const __half *__restrict__ xb, const float *__restrict__ bias, 
     }
 }
 
-template <typename TOUT, int WAVES, int SG, bool DB>
+template <typename TOUT, int WAVES, int SG, bool DB, int NQ = 0>
 void launch_pair_t(const GemmArgs &g, hipStream_t stream, const void *w_hat, int ranges, int blocks_per_range)
 {
-    auto kernel = gemm_pair_kernel<TOUT, WAVES, SG, DB>;
-    constexpr int kSmem = PairCfg<WAVES, SG, DB>::kSmem;
-    allow_dynamic_lds<gemm_pair_kernel<TOUT, WAVES, SG, DB>>(kSmem);
+    auto kernel = gemm_pair_kernel<TOUT, WAVES, SG, DB, NQ>;
+    constexpr int kSmem = PairCfg<WAVES, SG, DB>::kSmem + (NQ ? next_quant_lds_bytes(NQ) : 0);
+    allow_dynamic_lds<gemm_pair_kernel<TOUT, WAVES, SG, DB, NQ>>(kSmem);
     const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
     const int tiles = n_slabs * ranges;
     hipLaunchKernelGGL(kernel, dim3(8 * ((tiles + 7) / 8)), dim3(64 * WAVES), kSmem, stream,
                        static_cast<const __half *>(g.x_hat), g.bias, static_cast<TOUT *>(g.y), g.M, g.N, g.K, ranges,
                        blocks_per_range, static_cast<const __half *>(w_hat), static_cast<const TOUT *>(g.residual),
-                       g.gelu ? 1 : 0);
+                       g.gelu ? 1 : 0, g.next_thr, g.next_cb);
 }
 
 }  // namespace
@@ -506,6 +523,12 @@ void launch_gemm_pair(const GemmArgs &g, const void *w_hat, hipStream_t stream)
     pair_ranges(g, 256, ranges, per);
     // Two slab buffers of three groups measured 0-4 % faster than one of six on every multi-slice shape (DeiT-B fc1
     // 72.3 -> 69.7 us, qkv 55.2 -> 53.7, ViT-L qkv 326 -> 324); ARCQ_PAIR=1 pins the single buffer (tuning aid).
+    if (g.next_thr) {          // quantize the output for the next layer (fp16 output; the entry point checked the rest)
+        if (g.bits == 4) launch_pair_t<__half, 8, 3, true, 4>(g, stream, w_hat, ranges, per);
+        else if (g.bits == 3) launch_pair_t<__half, 8, 3, true, 3>(g, stream, w_hat, ranges, per);
+        else launch_pair_t<__half, 8, 3, true, 2>(g, stream, w_hat, ranges, per);
+        return;
+    }
     const char *e = tuning().pair;
     const bool db = e ? e[0] != '1' : true;
     if (db) {

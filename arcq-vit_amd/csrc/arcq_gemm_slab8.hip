@@ -17,6 +17,7 @@
 // k order, so their results are bit-identical.
 #include "arcq_common.h"
 #include "arcq_gemm.h"
+#include "arcq_act_quant_core.h"
 
 #include <stdlib.h>
 #include <type_traits>
@@ -72,14 +73,18 @@ __device__ __forceinline__ uint32_t code_at(const uint32_t (&w)[BITS], int q)
 // WAVES = 8 or 12 waves per workgroup (two or three per SIMD).
 // AHEAD = 1 or 2: how many k-steps the LDS reads of the w_hat fragments run ahead of the MFMAs that use them (two
 // where the registers allow it: the LDS round trip under load is longer than one k-step of four MFMAs).
-template <int BITS, typename TOUT, bool PRE, int WAVES, int AHEAD>
+// NQ = 0, or the bits (2 / 3 / 4) of the activation quantizer of the layer that consumes this one's output: y then
+// receives that layer's x_hat in the block layout instead of the output itself (arcq_act_quant_core.h,
+// next_quant_chunk); fp16 output, N a multiple of 64, copied weights and eight waves only.
+template <int BITS, typename TOUT, bool PRE, int WAVES, int AHEAD, int NQ = 0>
 __global__ void __launch_bounds__(64 * WAVES)
 gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw, const float *__restrict__ cb,
                   const float *__restrict__ wc, const float *__restrict__ ws, const float *__restrict__ wcs,
                   const float *__restrict__ bias, TOUT *__restrict__ y, int M, int N, int K,
                   int row_ranges, int blocks_per_range, const __half *__restrict__ w_hat,
-                  const TOUT *__restrict__ residual, int gelu)
+                  const TOUT *__restrict__ residual, int gelu, const float *__restrict__ nx_thr, const float *__restrict__ nx_cb)
 {
+    static_assert(NQ == 0 || (sizeof(TOUT) == 2 && PRE), "the next layer's stage 1: fp16 outputs, copied weights");
     constexpr int L = 1 << BITS;
     constexpr int kWaves = WAVES;
     constexpr bool SPLIT = ARCQ_SPLIT_DEFAULT;                   // left-over blocks are dealt in halves
@@ -149,6 +154,9 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
         }
     }
     if (tid < kSlabN) s_bias[tid] = (bias && n_base + tid < N) ? bias[n_base + tid] : 0.0f;
+    const unsigned char *nq_lds = reinterpret_cast<const unsigned char *>(s_bias + kSlabN);
+    if constexpr (NQ != 0)      // (the barriers of the first slab fill publish the tables)
+        next_quant_setup<NQ>(nx_thr, nx_cb, reinterpret_cast<unsigned char *>(s_bias + kSlabN), tid, kThreads);
     // PRE: one direct global -> LDS load per slab row (lanes 0..47 carry the row's 48 16-byte pieces, the hardware
     // writes lane l's piece at the wave-uniform LDS base + 16 l); the caller waits for vmcnt and the barrier.
     auto copy_slice = [&](int g0, int ng) __attribute__((always_inline)) {
@@ -382,6 +390,15 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
                     }
                 }
                 __builtin_amdgcn_wave_barrier();
+                if constexpr (NQ != 0) {
+                    const int c0 = n_base + jb * 32 + ch * kChunkCols;          // the chunk is one group of the consumer's rows
+                    if (c0 < N)
+                        next_quant_chunk<NQ>(nq_lds, kWaves, stage, kStageRow, lane, gelu != 0, 1.0e-6f,
+                                             reinterpret_cast<__half *>(y) + static_cast<int64_t>(pblk) * 32 * N,
+                                             min(32, M - pblk * 32), c0 / 8);
+                    __builtin_amdgcn_wave_barrier();
+                    continue;
+                }
                 const int col = n_base + jb * 32 + ch * kChunkCols + (lane & 7) * kVec;
                 const int row0 = pblk * 32 + (lane >> 3);
                 TOUT *dst0 = y + static_cast<int64_t>(row0) * N + col;
@@ -435,13 +452,14 @@ gemm_slab8_kernel(const __half *__restrict__ xb, const uint8_t *__restrict__ pw,
     }
 }
 
-template <int BITS, typename TOUT, bool PRE, int WAVES, int AHEAD>
+template <int BITS, typename TOUT, bool PRE, int WAVES, int AHEAD, int NQ = 0>
 void launch_slab8_w(const GemmArgs &g, hipStream_t stream, const void *w_hat)
 {
     constexpr int L = 1 << BITS;
-    const size_t smem = kSlabBytes + WAVES * kStageTile + L * 64 * sizeof(float) + kSlabN * sizeof(float);
-    auto kernel = gemm_slab8_kernel<BITS, TOUT, PRE, WAVES, AHEAD>;
-    allow_dynamic_lds<gemm_slab8_kernel<BITS, TOUT, PRE, WAVES, AHEAD>>(static_cast<int>(smem));
+    const size_t smem = kSlabBytes + WAVES * kStageTile + L * 64 * sizeof(float) + kSlabN * sizeof(float) +
+                        (NQ ? next_quant_lds_bytes(NQ) : 0);
+    auto kernel = gemm_slab8_kernel<BITS, TOUT, PRE, WAVES, AHEAD, NQ>;
+    allow_dynamic_lds<gemm_slab8_kernel<BITS, TOUT, PRE, WAVES, AHEAD, NQ>>(static_cast<int>(smem));
     // One workgroup per CU where possible: split the 32-row blocks into as many ranges as CUs/slabs allow.
     const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
     const int total_blocks = (g.M + 31) / 32;
@@ -454,7 +472,8 @@ void launch_slab8_w(const GemmArgs &g, hipStream_t stream, const void *w_hat)
     hipLaunchKernelGGL(kernel, dim3(8 * ((tiles + 7) / 8)), dim3(64 * WAVES), smem, stream,
                        static_cast<const __half *>(g.x_hat), g.pw, g.cb, g.wc, g.ws, g.wcs, g.bias,
                        static_cast<TOUT *>(g.y), g.M, g.N, g.K, ranges, blocks_per_range,
-                       static_cast<const __half *>(w_hat), static_cast<const TOUT *>(g.residual), g.gelu ? 1 : 0);
+                       static_cast<const __half *>(w_hat), static_cast<const TOUT *>(g.residual), g.gelu ? 1 : 0,
+                       g.next_thr, g.next_cb);
 }
 
 // Waves per workgroup.  While one wave of a SIMD writes its block out (2-2.5 us per pass: the stores queue behind
@@ -489,6 +508,12 @@ void launch_gemm_slab8(const GemmArgs &g, const void *w_hat, hipStream_t stream)
         const char *e = tuning().pair;           // tuning aid: 0 / 1 pin the choice
         if (e ? e[0] != '0' : gemm_pair_pays(g)) {
             launch_gemm_pair(g, w_hat, stream);
+            return;
+        }
+        if (g.next_thr) {      // quantize the output for the next layer: the eight-wave variant (fp16 output)
+            if (g.bits == 4) launch_slab8_w<4, __half, true, 8, 2, 4>(g, stream, w_hat);
+            else if (g.bits == 3) launch_slab8_w<4, __half, true, 8, 2, 3>(g, stream, w_hat);
+            else launch_slab8_w<4, __half, true, 8, 2, 2>(g, stream, w_hat);
             return;
         }
         if (g.y_f16) launch_slab8<4, __half, true>(g, stream, w_hat);

@@ -143,11 +143,23 @@ class ARCQPackedLinearOnTheFly(nn.Module):
 
     def can_quantize_for(self, consumer: nn.Module, rows: int) -> bool:
         """Whether ``forward(..., quantize_for=consumer)`` is available: this layer's launch then ends with the
-        consumer's stage 1 (the consumer is called with ``input_is_xhat=True``).  Built for fewer than 512 rows."""
-        return (isinstance(consumer, ARCQPackedLinearOnTheFly) and not self.fp8_operands and not consumer.fp8_operands
-                and 0 < rows < 512 and self.group_size == 64 and consumer.group_size == 64 and self.bits == consumer.bits
+        consumer's stage 1 (the consumer is called with ``input_is_xhat=True``).  From 512 rows on it needs the shared
+        weight buffer (``_weight_buffer``)."""
+        if not (isinstance(consumer, ARCQPackedLinearOnTheFly) and not self.fp8_operands and not consumer.fp8_operands
+                and rows > 0 and self.group_size == 64 and consumer.group_size == 64 and self.bits == consumer.bits
                 and consumer.in_features == self.out_features and self.out_features % 64 == 0
-                and self.in_features % 64 == 0 and self.in_features <= 1536 and self.out_dtype == torch.float16)
+                and self.in_features % 64 == 0 and self.out_dtype == torch.float16):
+            return False
+        if rows < 512:                       # the small-M kernel's epilogue
+            return self.in_features <= 1536
+        # The block-layout GEMM kernels' epilogue: needs the weight workspace.  Not taken where this layer would run as
+        # one launch with stage 1 inside (short rows: DeiT-S at batch 64): the consumer's stage 1 is then already hidden
+        # under its own product and the chained pair measured slower (DeiT-S forward 1.86 -> 2.08 ms; DeiT-B 4.88 ->
+        # 4.76, ViT-L 49.7 -> 48.5).
+        if getattr(self, "_weight_buffer", None) is None or rows * self.in_features * 2 >= 2 ** 32:
+            return False
+        kernel = _lib.load().arcq_linear_otf_ws_kernel(rows, self.out_features, self.in_features, 1)
+        return not kernel.startswith(b"otf_rows")
 
     def forward(self, x: torch.Tensor, layernorm: Optional[nn.LayerNorm] = None, activation: Optional[str] = None,
                 residual: Optional[torch.Tensor] = None, quantize_for: Optional[nn.Module] = None,

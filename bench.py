@@ -444,9 +444,7 @@ def chained_step(model, bits, batch, steps, warmup, dev):
             cur = nxt
 
     out = {}
-    variants = [("plain", False), ("fused", True)]
-    if lib.arcq_xhat_layout(m) == 0:          # (chaining fc1 -> fc2 through x_hat is built for fewer than 512 rows)
-        variants.append(("fused_mlp_chained_through_x_hat", "xhat"))
+    variants = [("plain", False), ("fused", True), ("fused_mlp_chained_through_x_hat", "xhat")]
     for name, fused in variants:
         run(fused, torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()

@@ -130,7 +130,12 @@ def test_linear_otf_ex_equals_the_unfused_sequence(cuda, oracle, m, n, k, bits, 
 
 
 @pytest.mark.parametrize("m,k,h,bits", [(197, 384, 1536, 4), (100, 384, 1536, 3), (197, 192, 768, 4), (33, 768, 3072, 4),
-                                        (1, 64, 64, 2)])
+                                        (1, 64, 64, 2),
+                                        # from 512 rows on: the block-layout GEMM kernels, x_hat handed over in the block layout
+                                        (1000, 384, 1536, 4),        # eight-wave kernel, ragged last block
+                                        (3000, 192, 768, 3), (520, 64, 128, 2),
+                                        (12608, 768, 3072, 4),       # DeiT-B: two row blocks per wave
+                                        (8200, 1024, 4096, 3)])      # ViT-L widths
 def test_two_layers_chained_through_x_hat(cuda, oracle, m, k, h, bits):
     """fc1 -> GELU -> fc2 with fc2's stage 1 inside fc1's launch (next_quant / x_is_xhat): the x_hat handed over equals
     the oracle's stage 1 of the stored GELU output bit for bit, and fc2's result equals the unfused sequence's."""
@@ -146,13 +151,19 @@ def test_two_layers_chained_through_x_hat(cuda, oracle, m, k, h, bits):
     a1 = (d(thr), d(cb), d(pw1), d(cb), d(wc1), d(ws1), d(wcs1), d(b1), bits, 64)
     a2 = (d(thr2), d(cb2), d(pw2), d(cb), d(wc2), d(ws2), d(wcs2), d(b2), bits, 64)
     ln = (d(lw), d(lb), 1e-6)
-    assert ops.xhat_layout(m) == 0
-    xhat = ops.linear_otf_ex(d(x), *a1, layernorm=ln, gelu=True, next_quant=(d(thr2), d(cb2)))
-    y = ops.linear_otf_ex(xhat, *a2, residual=d(x), x_is_xhat=True)
-    g = ops.linear_otf_ex(d(x), *a1, layernorm=ln, gelu=True)                     # the stored GELU output
-    want_xhat = oracle.act_quant_c(_np(g).astype(np.float32), thr2, cb2, bits, 64)["x_hat"].astype(np.float16)
-    assert xhat.dtype == torch.float16 and np.array_equal(_np(xhat).view(np.uint16), want_xhat.view(np.uint16))
-    assert torch.equal(y, ops.linear_otf_ex(g, *a2, residual=d(x)))
+    blocked = ops.xhat_layout(m) == 1
+    assert blocked == (m >= 512)
+    w1 = torch.empty(h * k, dtype=torch.float16, device=cuda)        # weight workspaces (the block-layout path needs one)
+    xhat = ops.linear_otf_ex(d(x), *a1, layernorm=ln, gelu=True, next_quant=(d(thr2), d(cb2)), w_hat_ws=w1)
+    y = ops.linear_otf_ex(xhat, *a2, residual=d(x), x_is_xhat=True, w_hat_ws=w1)
+    g = ops.linear_otf_ex(d(x), *a1, layernorm=ln, gelu=True, w_hat_ws=w1)       # the stored GELU output
+    want_xhat = torch.from_numpy(oracle.act_quant_c(_np(g).astype(np.float32), thr2, cb2, bits, 64)["x_hat"].astype(np.float16))
+    if blocked:
+        want_xhat = _to_blocked(want_xhat)
+    assert xhat.dtype == torch.float16
+    assert np.array_equal(_np(xhat).reshape(-1).view(np.uint16), want_xhat.numpy().reshape(-1).view(np.uint16))
+    assert torch.equal(y, ops.linear_otf_ex(g, *a2, residual=d(x), w_hat_ws=w1))
+    assert torch.equal(y, ops.linear_otf_ex(xhat, *a2, residual=d(x), x_is_xhat=True))     # consumer without a workspace
 
 
 def test_linear_otf_ex_fp32_and_limits(cuda, oracle):
