@@ -78,7 +78,8 @@ _SIGNATURES = {
     "arcq_linear_forward_u8": [_c_ptr] * 11 + [_c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
 }
 EXPORTED_SYMBOLS = ("arcq_version", "arcq_last_error", "arcq_reload_tuning", "arcq_linear_fused_kernel",
-                    "arcq_linear_fused_ws_kernel", "arcq_linear_otf_ws_kernel") + tuple(_SIGNATURES)
+                    "arcq_linear_fused_ws_kernel", "arcq_linear_otf_ws_kernel", "arcq_rows_wait_timeouts",
+                    "arcq_rows_counter_slot") + tuple(_SIGNATURES)
 
 _lib = None
 _lock = threading.Lock()
@@ -112,6 +113,10 @@ def load() -> ctypes.CDLL:
             lib.arcq_linear_fused_ws_kernel.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
             lib.arcq_linear_otf_ws_kernel.restype = ctypes.c_char_p
             lib.arcq_linear_otf_ws_kernel.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
+            lib.arcq_rows_wait_timeouts.restype = ctypes.c_longlong
+            lib.arcq_rows_wait_timeouts.argtypes = []
+            lib.arcq_rows_counter_slot.restype = _c_int
+            lib.arcq_rows_counter_slot.argtypes = [ctypes.POINTER(ctypes.c_void_p), _c_int, _c_ptr]
             for name, argtypes in _SIGNATURES.items():
                 fn = getattr(lib, name)
                 fn.restype = _c_int

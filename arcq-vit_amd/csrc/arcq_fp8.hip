@@ -22,12 +22,12 @@ namespace {
 constexpr float kFp8Max = 448.0f;
 constexpr int kFp8Waves = 4;
 
-// Eight floats -> eight FP8 (E4M3, round to nearest even, saturating) in two dwords.
+// Eight floats -> eight FP8 (E4M3, round to nearest even, finite values saturating at +-448, NaN kept) in two dwords.
 __device__ __forceinline__ void to_fp8x8(const float (&v)[8], uint32_t &lo, uint32_t &hi)
 {
     float c[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) c[i] = fminf(fmaxf(v[i], -kFp8Max), kFp8Max);
+    for (int i = 0; i < 8; ++i) c[i] = v[i] != v[i] ? v[i] : fminf(fmaxf(v[i], -kFp8Max), kFp8Max);      // (NaN stays NaN)
     int a = 0, b = 0;
     a = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], a, false);
     a = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], a, true);

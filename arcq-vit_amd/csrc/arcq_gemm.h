@@ -54,6 +54,10 @@ int linear_fused_blocked(const void *x_hat_blocked, const uint8_t *packed_w, con
                          const float *next_thr = nullptr, const float *next_cb = nullptr);
 
 
+// Compute units of the current device (256 when there is none to ask: the host-side predicates also run without a
+// GPU); what the weight-stationary kernels size their row ranges by (one workgroup per compute unit).
+int device_cus();
+
 // Small-M kernel (64 x 64 tiles, K split across the waves of a workgroup); requires K >= 64.
 void launch_gemm_splitk(const GemmArgs &g, hipStream_t stream);
 // arcq_linear_fused with GELU / a residual ([M,N] of y's type) on the rounded outputs; with either set it needs the
@@ -114,6 +118,9 @@ bool otf_rows_pays(int64_t M, int64_t N, int64_t K, bool layernorm = false);
 // Returns kNotLaunched (having launched nothing and recorded no error) when the stream cannot be given a counter or
 // the device would not hold all the launch's workgroups at once: the caller takes the two-launch path.
 constexpr int kNotLaunched = -1000;
+// Slot of `key` in a table of `slots` keys (nullptr = free): its own if it has one, else the first free one on its
+// probe sequence, which it then owns; -1 when the table is full.  (The per-workspace counters of launch_otf_rows.)
+int rows_counter_slot(const void **table, int slots, const void *key);
 int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream);
 
 }  // namespace arcq

@@ -474,10 +474,10 @@ void launch_fp8_t(const void *x8, const void *w8, const float *bias, float inv_m
     auto kernel = gemm_fp8_kernel<TOUT, WAVES, SG, DB>;
     constexpr int kSmem = Fp8Cfg<WAVES, SG, DB>::kSmem;
     allow_dynamic_lds<gemm_fp8_kernel<TOUT, WAVES, SG, DB>>(kSmem);
-    // Row ranges: one workgroup per compute unit (tiles = slabs x ranges ~ 256).
+    // Row ranges: one workgroup per compute unit (tiles = slabs x ranges ~ the number of compute units).
     const int n_slabs = (N + kSlabN - 1) / kSlabN;
     const int total_blocks = (M + 31) / 32;
-    int ranges = 256 / n_slabs;
+    int ranges = device_cus() / n_slabs;
     if (ranges < 1) ranges = 1;
     if (ranges > total_blocks) ranges = total_blocks;
     const int blocks_per_range = (total_blocks + ranges - 1) / ranges;

@@ -512,7 +512,7 @@ static void pair_ranges(const GemmArgs &g, int slots, int &ranges, int &blocks_p
 bool gemm_pair_pays(const GemmArgs &g)
 {
     int ranges, per;
-    pair_ranges(g, 256, ranges, per);
+    pair_ranges(g, device_cus(), ranges, per);
     return g.K > 6 * 64 && per >= 8;
 }
 
@@ -520,7 +520,7 @@ bool gemm_pair_pays(const GemmArgs &g)
 void launch_gemm_pair(const GemmArgs &g, const void *w_hat, hipStream_t stream)
 {
     int ranges, per;
-    pair_ranges(g, 256, ranges, per);
+    pair_ranges(g, device_cus(), ranges, per);
     // Two slab buffers of three groups measured 0-4 % faster than one of six on every multi-slice shape (DeiT-B fc1
     // 72.3 -> 69.7 us, qkv 55.2 -> 53.7, ViT-L qkv 326 -> 324); ARCQ_PAIR=1 pins the single buffer (tuning aid).
     if (g.next_thr) {          // quantize the output for the next layer (fp16 output; the entry point checked the rest)

@@ -463,7 +463,7 @@ void launch_slab8_w(const GemmArgs &g, hipStream_t stream, const void *w_hat)
     // One workgroup per CU where possible: split the 32-row blocks into as many ranges as CUs/slabs allow.
     const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
     const int total_blocks = (g.M + 31) / 32;
-    int ranges = 256 / n_slabs;
+    int ranges = device_cus() / n_slabs;
     if (ranges < 1) ranges = 1;
     if (ranges > total_blocks) ranges = total_blocks;
     const int blocks_per_range = (total_blocks + ranges - 1) / ranges;
@@ -488,7 +488,7 @@ void launch_slab8(const GemmArgs &g, hipStream_t stream, const void *w_hat)
     if constexpr (PRE) {
         const int n_slabs = (g.N + kSlabN - 1) / kSlabN;
         const int total_blocks = (g.M + 31) / 32;
-        const int ranges = max(1, min(256 / n_slabs, total_blocks));
+        const int ranges = max(1, min(device_cus() / n_slabs, total_blocks));
         const int64_t units = static_cast<int64_t>((total_blocks + ranges - 1) / ranges) * (g.K / 64);
         if (units >= 256) {
             launch_slab8_w<BITS, TOUT, PRE, 12, 1>(g, stream, w_hat);

@@ -33,6 +33,7 @@
 #include "arcq_act_quant_core.h"
 
 #include <mutex>
+#include <vector>
 
 namespace arcq {
 namespace {
@@ -58,6 +59,7 @@ struct RowsParams {
     __half *w_blk;                   // weight workspace, block layout
     unsigned long long *counter;     // nullptr: w_blk is complete already
     long long wait_ticks;            // bound of the wait for the other workgroups' shares, ticks of the 100 MHz clock
+    unsigned long long *timeouts;    // counts the workgroups whose wait ran out (a diagnostic: arcq_rows_wait_timeouts)
     const float *bias;               // [N] or nullptr
     void *y;
     const void *residual;
@@ -282,15 +284,16 @@ otf_rows_kernel(const RowsParams p)
 
     // ---- every share of w_hat written? ----
     if (p.counter && tid == 0) {
-        int ok = 1;
+        int ok = p.wait_ticks > 0;      // (a bound of zero: give up without looking -- how the tests reach the rebuild)
         const long long t0 = wall_clock64();
-        while (__hip_atomic_load(p.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        while (ok && __hip_atomic_load(p.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
             if (wall_clock64() - t0 > p.wait_ticks) {
                 ok = 0;
                 break;
             }
             __builtin_amdgcn_s_sleep(4);
         }
+        if (!ok) __hip_atomic_fetch_add(p.timeouts, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_flag = ok;
     }
     // One wave drops whatever this CU's L1 and this XCD's L2 may hold of the workspace (nothing, unless a line was
@@ -610,15 +613,16 @@ otf_rows_phased_kernel(const RowsParams p)
         if (ph == -1) {
             // ---- every share of w_hat written? ----
             if (p.counter && tid == 0) {
-                int ok = 1;
+                int ok = p.wait_ticks > 0;      // (a bound of zero: give up without looking -- how the tests reach the rebuild)
                 const long long t0 = wall_clock64();
-                while (__hip_atomic_load(p.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+                while (ok && __hip_atomic_load(p.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
                     if (wall_clock64() - t0 > p.wait_ticks) {
                         ok = 0;
                         break;
                     }
                     __builtin_amdgcn_s_sleep(4);
                 }
+                if (!ok) __hip_atomic_fetch_add(p.timeouts, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 s_flag = ok;
             }
             if (p.counter && wave == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -688,36 +692,68 @@ otf_rows_phased_kernel(const RowsParams p)
     }
 }
 
-// One counter per stream (calls on one stream run one after another; calls on different streams may overlap and must
-// not count into the same word).  The counters live in device memory that is zero when the code object is loaded.
-constexpr int kCounterSlots = 256;
+// One counter per weight workspace.  Launches that share a counter word must never overlap (a workgroup derives its
+// target from the value it finds); launches that share a weight workspace must never overlap either -- they would
+// overwrite each other's w_hat -- so the workspace's address is the key: whatever the caller does with streams and
+// graphs (two graphs captured on one stream and replayed on two, a destroyed stream whose handle is reused, the null
+// stream's two flavours), overlapping launches count into different words as long as the caller keeps the rule it has
+// to keep anyway.  The words live in device memory that is zero when the code object is loaded; the key -> word table
+// is per device, open addressing from a hash of the address, never recycled (a word whose key left could still be
+// counted into by a launch in flight): after 4096 distinct workspace addresses on a device further ones take the
+// two-launch path (a model shares one workspace between its layers; the table is sized for processes that allocate
+// and free workspaces all the time, such as a test suite).
+constexpr int kCounterSlots = 4096;
 __device__ unsigned long long g_rows_counters[kCounterSlots];
+__device__ unsigned long long g_rows_timeouts;          // workgroups whose bounded wait ran out, ever
 
 constexpr int kMaxDevices = 64;
 std::mutex g_rows_mutex;
 unsigned long long *g_counters_ptr[kMaxDevices];
-void *g_slot_stream[kMaxDevices][kCounterSlots];
-int g_slots_used[kMaxDevices];
+unsigned long long *g_timeouts_ptr[kMaxDevices];
+std::vector<const void *> g_slot_key[kMaxDevices];          // kCounterSlots keys per device, allocated on first use
 
-// Device address of the counter of `stream` on the current device; nullptr if it cannot be had.
-unsigned long long *counter_for(hipStream_t stream)
+}  // namespace
+
+// Slot of `key` in a table of `slots` keys (nullptr = free): the key's own slot if it has one, else the first free
+// one on its probe sequence (which it then owns), else -1.  Host logic only.
+int rows_counter_slot(const void **table, int slots, const void *key)
+{
+    if (!key || slots <= 0) return -1;
+    uint64_t h = reinterpret_cast<uintptr_t>(key) >> 8;          // (workspaces are at least 128-byte aligned)
+    h ^= h >> 17;
+    h *= 0x9E3779B97F4A7C15ull;
+    h ^= h >> 29;
+    const int start = static_cast<int>(h % static_cast<uint64_t>(slots));
+    for (int i = 0; i < slots; ++i) {
+        const int s = (start + i) % slots;
+        if (table[s] == key) return s;
+        if (table[s] == nullptr) {
+            table[s] = key;
+            return s;
+        }
+    }
+    return -1;
+}
+
+namespace {
+
+// Device address of the counter that belongs to weight workspace `key` on the current device; nullptr if none is left.
+unsigned long long *counter_for(const void *key, unsigned long long **timeouts)
 {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
     std::lock_guard<std::mutex> lock(g_rows_mutex);
     if (!g_counters_ptr[dev]) {
-        void *ptr = nullptr;
+        void *ptr = nullptr, *tptr = nullptr;
         if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_rows_counters)) != hipSuccess || !ptr) return nullptr;
+        if (hipGetSymbolAddress(&tptr, HIP_SYMBOL(g_rows_timeouts)) != hipSuccess || !tptr) return nullptr;
         g_counters_ptr[dev] = static_cast<unsigned long long *>(ptr);
+        g_timeouts_ptr[dev] = static_cast<unsigned long long *>(tptr);
     }
-    int slot = -1;
-    for (int i = 0; i < g_slots_used[dev]; ++i)
-        if (g_slot_stream[dev][i] == static_cast<void *>(stream)) slot = i;
-    if (slot < 0) {
-        if (g_slots_used[dev] == kCounterSlots) return nullptr;      // more streams than counters: the caller falls back
-        slot = g_slots_used[dev]++;
-        g_slot_stream[dev][slot] = static_cast<void *>(stream);
-    }
+    if (g_slot_key[dev].empty()) g_slot_key[dev].assign(kCounterSlots, nullptr);
+    const int slot = rows_counter_slot(g_slot_key[dev].data(), kCounterSlots, key);
+    if (slot < 0) return nullptr;            // more workspaces than counters: the caller falls back
+    *timeouts = g_timeouts_ptr[dev];
     return g_counters_ptr[dev] + slot;
 }
 
@@ -744,6 +780,8 @@ int resident_workgroups(int threads, size_t smem)
     return per_cu * cus;
 }
 
+}  // namespace
+
 // Compute units of the current device (256 when there is none to ask: the host-side predicates also run without a GPU).
 int device_cus()
 {
@@ -755,6 +793,8 @@ int device_cus()
     known[dev].store(cus, std::memory_order_relaxed);
     return cus;
 }
+
+namespace {
 
 size_t rows_lds_bytes(int N, int K)
 {
@@ -864,8 +904,8 @@ int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream)
     p.gamma = a.ln_weight, p.beta = a.ln_bias, p.ln_eps = a.ln_eps;
     p.pw = a.pw, p.cb_w = a.w_cb, p.wc = a.wc, p.ws = a.ws, p.wcs = a.wcs;
     p.w_blk = static_cast<__half *>(a.w_hat_ws);
-    p.counter = counter_for(stream);
-    if (!p.counter) return kNotLaunched;     // more streams than counters: the caller takes the two-launch path
+    p.counter = counter_for(a.w_hat_ws, &p.timeouts);
+    if (!p.counter) return kNotLaunched;     // more workspaces than counters: the caller takes the two-launch path
     p.wait_ticks = tuning().rows_wait_ticks;
     p.bias = a.bias, p.y = a.y, p.residual = a.residual, p.gelu = a.gelu ? 1 : 0;
     p.M = a.M, p.N = a.N, p.G = a.K / 64;
@@ -894,3 +934,24 @@ int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream)
 }
 
 }  // namespace arcq
+
+// Host-side slot logic of the per-workspace counters, exposed so that it can be tested without a GPU: `table` is a
+// caller-owned array of `slots` pointers, all NULL at first.
+ARCQ_API int arcq_rows_counter_slot(const void **table, int slots, const void *key)
+{
+    return arcq::rows_counter_slot(table, slots, key);
+}
+
+// Diagnostic: how many workgroups of the one-launch layer kernels have, on the current device and since the library was
+// loaded, given up waiting for the other workgroups' weight shares and rebuilt all of w_hat themselves (correct
+// results, but each such launch is many times slower: the sign of a device shared with other work).  Synchronizes
+// with the device (a blocking copy); -1 if the count cannot be read.
+ARCQ_API long long arcq_rows_wait_timeouts(void)
+{
+    unsigned long long v = 0;
+    if (hipMemcpyFromSymbol(&v, HIP_SYMBOL(arcq::g_rows_timeouts), sizeof(v), 0, hipMemcpyDeviceToHost) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    return static_cast<long long>(v);
+}

@@ -101,15 +101,24 @@ class ARCQPackedLinearOnTheFly(nn.Module):
 
     def _prepare(self):
         """Validated, fp32-contiguous views of the buffers and their raw pointers, built once and reused by every
-        forward until the buffers move (``_apply``, ``load_state_dict``) or are replaced."""
+        forward until a buffer moves (``_apply``, ``load_state_dict``), is replaced or is written in place."""
         a = [ops._f32c(self.activation_thresholds), ops._f32c(self.activation_codebook)]
         w = [self.packed_weight_codes.contiguous(), ops._f32c(self.weight_codebook), ops._f32c(self.weight_center),
              ops._f32c(self.weight_scale), ops._f32c(self.weight_code_sum)]
         bias = ops._f32c(self.bias_tensor) if self.bias_tensor.numel() > 0 else None
         keep = a + w + [bias]
-        self._prep = (keep, tuple(0 if t is None else t.data_ptr() for t in keep), self.packed_weight_codes.data_ptr(),
+        self._prep = (keep, tuple(0 if t is None else t.data_ptr() for t in keep), self._buffers_key(),
                       self.packed_weight_codes.device)
         return self._prep
+
+    _PREP_BUFFERS = ("activation_thresholds", "activation_codebook", "packed_weight_codes", "weight_codebook",
+                     "weight_center", "weight_scale", "weight_code_sum", "bias_tensor")
+
+    def _buffers_key(self):
+        """Identity and version of every buffer the cached pointers were made from: replacing a buffer or writing into
+        one in place changes it, and the next forward prepares again."""
+        b = self._buffers
+        return tuple((b[n].data_ptr(), b[n]._version) for n in self._PREP_BUFFERS)
 
     def _load_from_state_dict(self, *args, **kwargs):
         self._prep = None
@@ -205,7 +214,7 @@ class ARCQPackedLinearOnTheFly(nn.Module):
                 y = y + residual.reshape(-1, self.out_features)
             return y.reshape(*original_shape[:-1], self.out_features)
         prep = self._prep
-        if prep is None or prep[2] != self.packed_weight_codes.data_ptr():
+        if prep is None or prep[2] != self._buffers_key():
             prep = self._prepare()
             self._fp8_mult = None
         if prep[3] != x2.device:
@@ -258,7 +267,7 @@ class ARCQPackedLinearOnTheFly(nn.Module):
                     a.producer = _lib.ARCQ_PRODUCER_XHAT
                 if quantize_for is not None:
                     nprep = quantize_for._prep
-                    if nprep is None or nprep[2] != quantize_for.packed_weight_codes.data_ptr():
+                    if nprep is None or nprep[2] != quantize_for._buffers_key():
                         nprep = quantize_for._prepare()
                         quantize_for._fp8_mult = None
                     a.next_a_thresholds, a.next_a_codebook = nprep[1][0], nprep[1][1]

@@ -153,10 +153,11 @@ int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const
  * cooperatively, in 32-column blocks [N/32][K/8][32][8]).  The upper limit on M keeps every workgroup of the launch
  * resident at once: each waits, for at most 0.5 ms, until all the others have written their share of w_hat; if the
  * device is shared with other kernels at that moment the wait can run out, after which a workgroup rebuilds all of
- * w_hat itself (same result, late).  That launch counts in a word of the library's static device memory chosen by `stream`: calls
- * on one stream run one after another as always; a HIP graph captured from a stream must not be replayed
- * concurrently with other calls made on that same stream; the first 256 streams a process uses for such calls on a
- * device get a word each, calls on further streams take the two-launch path.  ARCQ_ROWS=0 in the environment keeps
+ * w_hat itself (same result, late; arcq_rows_wait_timeouts counts these).  That launch counts in a word of the
+ * library's static device memory chosen by the address of w_hat_ws: calls that may overlap in time (different
+ * streams, graphs replayed side by side) must use different weight workspaces -- which they must anyway, since each
+ * call overwrites its workspace -- and then never share a word; the first 4096 workspace addresses a process uses on a
+ * device get a word each, calls with further ones take the two-launch path.  ARCQ_ROWS=0 in the environment keeps
  * the two-launch path everywhere. */
 int arcq_linear_fused_ws(const void *x_hat,
                          const uint8_t *packed_w, const float *w_codebook,
@@ -282,7 +283,8 @@ int arcq_linear_otf_static(const void *x, int x_dtype, const float *a_thresholds
                            const float *bias, void *y, int y_dtype,
                            int64_t M, int64_t N, int64_t K, int bits, int group_size, void *stream);
 
-/* The two operands of the layer rounded to FP8 (OCP E4M3, round to nearest even, clamped to +-448) instead of fp16, for
+/* The two operands of the layer rounded to FP8 (OCP E4M3, round to nearest even; finite values beyond +-448 saturate --
+ * activations carry no multiplier, so |x_hat| > 448 is clipped and |x_hat| < 2^-6 loses precision -- NaN stays NaN) instead of fp16, for
  * a product on FP8 matrix units: the low-precision formulation that EXT/arcq_linear_kernel.cu:22-202 points at.  They
  * have no counterpart in the reference and do NOT reproduce its numbers (3 mantissa bits per operand where fp16 has
  * 10); codes, mu, s and the fp32 reconstruction are those of arcq_act_quant / arcq_weight_dequant.
@@ -320,6 +322,16 @@ int arcq_linear_otf_fp8(const void *x, int x_dtype, const float *a_thresholds, c
                         const uint8_t *packed_w, const float *w_codebook, const float *w_center, const float *w_scale,
                         const float *w_code_sum, const float *bias, float w_mult, void *x8_ws, void *w8_ws, void *y,
                         int y_dtype, int64_t M, int64_t N, int64_t K, int bits, void *stream);
+
+/* Diagnostics of the one-launch layer kernels; no counterpart in the reference.
+ * arcq_rows_wait_timeouts: number of workgroups that, on the current device since the library was loaded, gave up
+ * their bounded wait for the other workgroups' weight shares and rebuilt all of w_hat themselves (results stay
+ * correct; such a launch is many times slower -- the sign of a device shared with other work, or of a launch larger
+ * than the device holds).  Blocks until the device has finished (a synchronous copy); -1 if it cannot be read.
+ * arcq_rows_counter_slot: the host-side logic that assigns a weight workspace its counter word (`table`: `slots`
+ * pointers, NULL = free; returns the slot of `key`, claiming a free one on its probe sequence, or -1 when full). */
+long long arcq_rows_wait_timeouts(void);
+int arcq_rows_counter_slot(const void **table, int slots, const void *key);
 
 /* Kernels arcq_linear_otf_ws runs after stage 1 for these sizes: "gemm_slab8_kernel", or, with the weights rebuilt
  * in the stage-1 launch and copied by the GEMM, "gemm_slab8_kernel<copy>" or "gemm_pair_kernel" (two row blocks per

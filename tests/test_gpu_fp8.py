@@ -36,10 +36,16 @@ def test_stage1_fp8_is_the_oracle_reconstruction_rounded(cuda, oracle, m, k, bit
     thr = synth.midpoint_thresholds(cb)
     x = synth.make_activation(m, k, 7, "ln").to(dtype)
     x[0, :64] = 1000.0 * torch.linspace(-1, 1, 64).to(dtype)            # a group whose values leave FP8's range: clamped
+    if m > 1:
+        x[1, 5] = float("nan")                                          # a NaN poisons its group and stays a NaN in FP8
     x8 = ops.quantize_activation_fp8(x.to(cuda), thr.to(cuda), cb.to(cuda), bits)
-    want = oracle.fp8_e4m3_np(oracle.act_quant_c(x.float().numpy(), thr, cb, bits, 64)["x_hat"])
-    assert np.abs(want).max() == 448.0
-    assert np.array_equal(_np(x8.view(torch.uint8)), _fp8_bytes(want))
+    with np.errstate(invalid="ignore"):
+        want = oracle.fp8_e4m3_np(oracle.act_quant_c(x.float().numpy(), thr, cb, bits, 64)["x_hat"])
+    nan = np.isnan(want)
+    assert np.nanmax(np.abs(want)) == 448.0 and (m == 1 or (nan[1, :64].all() and nan.sum() == 64))
+    got = _np(x8.view(torch.uint8))
+    assert np.array_equal((got & 0x7f) == 0x7f, nan)                     # E4M3: S.1111.111 is the only NaN
+    assert np.array_equal(got[~nan], _fp8_bytes(np.where(nan, 0.0, want))[~nan])
 
 
 @pytest.mark.parametrize("n,k,bits", [(384, 1536, 4), (96, 192, 3), (1024, 1024, 2)])

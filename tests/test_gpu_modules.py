@@ -354,3 +354,21 @@ def test_fullsize_gemm_shapes(cuda, oracle, m, n, k, bits):
     assert torch.equal(ops.linear_fused_blocked(xb, m, k, pw, cb, wc, ws, wcs, bias, bits, out_dtype=torch.float32), y)
     assert torch.equal(ops.linear_fused_blocked(xb, m, k, pw, cb, wc, ws, wcs, bias, bits, out_dtype=torch.float32,
                                                 w_hat_ws=w16.reshape(-1), w_hat_ready=True), y)
+
+
+def test_on_the_fly_layer_sees_replaced_and_updated_buffers(cuda):
+    """The layer caches raw pointers of its buffers; swapping a buffer for another tensor, or writing into one in place,
+    must show in the next forward."""
+    from arcq_vit_amd.vit import build_packed_vit
+    vit = build_packed_vit("deit_tiny", 4, depth=1)
+    layer = vit.blocks[0].attn.proj
+    x = synth.make_activation(197, layer.in_features, 3).to(cuda).half()
+    with torch.no_grad():
+        y0 = layer(x).clone()
+        layer.bias_tensor = layer.bias_tensor * 64.0                     # replaced (a power of two: undone exactly below)
+        y1 = layer(x).clone()
+        assert not torch.equal(y1, y0)
+        layer.bias_tensor.mul_(1.0 / 64.0)                               # in place
+        assert torch.equal(layer(x), y0)
+        layer.activation_thresholds = layer.activation_thresholds * 0.5  # another buffer than the packed codes
+        assert not torch.equal(layer(x), y0)

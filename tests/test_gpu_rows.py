@@ -145,7 +145,7 @@ def test_phased_kernel_with_gelu_and_residual(cuda, oracle, monkeypatch, n, k, b
 
 
 def test_rows_kernel_counter_protocol(cuda, oracle):
-    """The cooperative weight reconstruction counts per stream and never resets: many calls in a row, layers of
+    """The cooperative weight reconstruction counts per weight workspace and never resets: many calls in a row, layers of
     different sizes sharing one weight workspace (every call must find the other layer's weights replaced), two
     streams at once, and HIP graph replays with eager calls in between all give the first call's bits."""
     shapes = [(12608, 1152, 384), (12608, 384, 384), (2000, 576, 192), (12608, 384, 1536)]
@@ -211,12 +211,20 @@ def test_rows_kernels_when_nobody_waits(cuda, oracle, monkeypatch, m, n, k, bits
     w_ws = torch.zeros(n * k, dtype=torch.float16, device=cuda)
     want = ops.linear_otf(x, *args, out_dtype=torch.float16, w_hat_ws=w_ws)
     w_want = w_ws.clone()
+    torch.cuda.synchronize()
+    timeouts0 = _lib.load().arcq_rows_wait_timeouts()
+    assert timeouts0 >= 0
     monkeypatch.setenv("ARCQ_ROWS_WAIT_TICKS", "0")
     for _ in range(3):
         w_ws.zero_()
         assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float16, w_hat_ws=w_ws), want)
         assert torch.equal(w_ws, w_want)
+    # the diagnostic counter saw the workgroups that gave up (nearly all of them: one that finds the shares complete
+    # at its first look does not count), and stands still again under the normal bound
+    timeouts1 = _lib.load().arcq_rows_wait_timeouts()
+    assert timeouts1 > timeouts0
     monkeypatch.delenv("ARCQ_ROWS_WAIT_TICKS")
     w_ws.zero_()
     assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float16, w_hat_ws=w_ws), want)
     assert torch.equal(w_ws, w_want)
+    assert _lib.load().arcq_rows_wait_timeouts() == timeouts1

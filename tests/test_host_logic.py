@@ -462,3 +462,25 @@ def test_bench_host_side_contract():
             traffic = bench.profiled_traffic(model, bits, batch, kernel)
             assert traffic is not None and traffic > 1e6, (model, kernel)
     assert bench.profiled_traffic("deit_small", 4, 64, "no_such_kernel") is None
+
+
+def test_rows_counter_slot_logic():
+    """The table that gives every weight workspace its own counter word: a key keeps its slot, distinct keys never
+    share one, a full table refuses further keys, and a collision moves on along the probe sequence."""
+    import ctypes
+    from arcq_vit_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built")
+    lib = _lib.load()
+    slots = 64
+    table = (ctypes.c_void_p * slots)()
+    keys = [0x7f0000000000 + 256 * i * 4099 for i in range(slots)]
+    got = [lib.arcq_rows_counter_slot(table, slots, k) for k in keys]
+    assert sorted(got) == list(range(slots))                      # all distinct, table now full
+    assert [lib.arcq_rows_counter_slot(table, slots, k) for k in keys] == got      # stable
+    assert lib.arcq_rows_counter_slot(table, slots, 0x7e0000000100) == -1           # full: the caller falls back
+    assert lib.arcq_rows_counter_slot(table, slots, None) == -1
+    small = (ctypes.c_void_p * 2)()
+    a = lib.arcq_rows_counter_slot(small, 2, 0x1000)
+    b = lib.arcq_rows_counter_slot(small, 2, 0x2000)
+    assert {a, b} == {0, 1} and lib.arcq_rows_counter_slot(small, 2, 0x3000) == -1
