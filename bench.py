@@ -4,19 +4,23 @@
 Workload (the headline configuration): the 48 packed linears of DeiT-Small (12 blocks x qkv 384->1152,
 proj 384->384, fc1 384->1536, fc2 1536->384), W4A4, group size 64, fp16 activations in and out,
 batch 64 (M = 64*197 = 12608 tokens).  One step = one pass over all 48 layers through
-arcq_linear_otf_ws: stage 1 (activation group-residual quantize + reconstruct, with the layer's fp16
-weights reconstructed by extra workgroups of the same launch) and an fp16 MFMA GEMM + bias on them.
-Inputs (one synthetic activation tensor per layer shape, packed weights of 48 distinct random layers)
-are resident in HBM before the timed region starts.
+arcq_linear_otf_ws with both scratch workspaces lent; at this batch every DeiT-S layer runs as ONE launch
+(otf_rows_kernel / otf_rows_phased_kernel: stage 1 into LDS, the fp16 weights reconstructed cooperatively into
+the workspace, fp16 MFMA GEMM + bias), the wider models as two (stage 1 into the block layout with the weight
+reconstruction carried along, then a weight-stationary GEMM).  Inputs (one synthetic activation tensor per layer
+shape, packed weights of 48 distinct random layers) are resident in HBM before the timed region starts.
 
-Prints ONE JSON line.  ``value`` is images/s of that step (packed linears only: no attention,
-LayerNorm or GELU; ``model_forward`` times the whole skeleton model next to it).  ``roofline`` is for
-the dominant kernel, the GEMM: algorithmic flops (2*M*N*K) of its launches divided by their time
-alone, measured here with HIP events on the launch stream in a GEMM-only loop; ``roofline.layer`` is
-the whole step against the same peaks; ``roofline.weights_rebuilt_inside_gemm`` the variant that
-dequantizes inside the GEMM.  ``cpu_baseline`` times the oracle's restatement of the reference's
-fake-quant CPU path (quantize + reconstruct activation and weight, fp32 matmul) on a bounded sample
-on this host.
+Prints ONE JSON line.  ``value`` is images/s of that step (packed linears only, on fixed inputs: no attention,
+LayerNorm or GELU; ``model_forward`` times the whole skeleton model next to it and ``bs1.chained`` /
+``detail.chained`` the linears as a dependency chain).  ``roofline`` is for the dominant kernel of the step --
+the one with the largest share of its time; for DeiT-S that is a whole-layer kernel, so its duration includes
+stage 1 and the weight reconstruction: algorithmic flops (2*M*N*K) of its launches divided by their time alone,
+measured here with HIP events on the launch stream in a graph of only these launches; ``roofline.layer`` is the
+whole step against the same peaks; ``roofline.weights_rebuilt_inside_gemm`` the variant that dequantizes inside
+the GEMM.  ``other_configs`` times the other BASELINE configurations (DeiT-B W4A4 batch 64, ViT-L W3A3 batch
+256) briefly in the same run, each with its own whole-step roofline.  ``cpu_baseline`` times the oracle's
+restatement of the reference's fake-quant CPU path (quantize + reconstruct activation and weight, fp32 matmul)
+on a bounded sample on this host.
 """
 from __future__ import annotations
 
@@ -55,6 +59,34 @@ def profiled_traffic(model, bits, batch, kernel):
     return float(m.group(1)) if m else None
 
 
+def traffic_source(model, bits, batch):
+    """Where `roofline.traffic` comes from: the committed profile's file name and the digest of the kernel sources it
+    was taken with (the summary records `kernel_sources_sha16 = ...`); `stale` says that the sources have changed
+    since, i.e. that the figure describes an older build of the kernel."""
+    import re
+    name = PROFILE_NAMES.get((model, bits, batch))
+    if not name:
+        return None
+    try:
+        text = open(os.path.join(ROOT, "profiles", name)).read()
+    except OSError:
+        return None
+    m = re.search(r"kernel_sources_sha16\s*=\s*([0-9a-f]+)", text)
+    now = kernel_sources_sha16()
+    return {"file": "profiles/" + name, "measured_live": False, "kernel_sources_sha16_of_profile": m.group(1) if m else None,
+            "kernel_sources_sha16_now": now, "stale": (m.group(1) != now) if m else None}
+
+
+def kernel_sources_sha16():
+    """First 16 hex digits of the SHA-256 over the library's kernel sources (csrc/*.hip, csrc/*.h, in name order)."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    for f in sorted(glob.glob(os.path.join(ROOT, "arcq-vit_amd", "csrc", "*.hip")) + glob.glob(os.path.join(ROOT, "arcq-vit_amd", "csrc", "*.h"))):
+        h.update(open(f, "rb").read())
+    return h.hexdigest()[:16]
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -66,6 +98,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bs1", action="store_true")
     ap.add_argument("--no-model", action="store_true", help="skip the model_forward block (whole ViT forward)")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the short runs of the other BASELINE configurations (default run only)")
     ap.add_argument("--fp8", action="store_true",
                     help="also time the same step with FP8 operands (ops.linear_otf_fp8: not the reference's numerics; "
                          "reported in a block of its own, never as `value`)")
@@ -665,6 +699,7 @@ def main():
         "roofline": {"bound": "mfma", "kernel": dom, "kernel_does": kernel_note(dom), "achieved": dk["tflops"],
                      "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": dk["tflops"] / PEAK_FP16_TFLOPS,
                      "traffic": profiled_traffic(args.model, args.bits, args.batch, dom),
+                     "traffic_source": traffic_source(args.model, args.bits, args.batch),
                      "algorithmic_flops_per_launch": dk["flops_per_launch"],
                      "algorithmic_bytes_per_launch": dk["bytes_per_launch"],
                      "avg_launch_us": dk["us_per_launch"], "launches_per_step": dk["launches_per_step"],
@@ -693,6 +728,23 @@ def main():
                       "hip_graph": True}
         out["bs1"]["cold_cache"] = cold_cache_bs1(args.model, args.bits, max(args.steps, 50), max(args.warmup, 10), dev)
         out["bs1"]["chained"] = chained_step(args.model, args.bits, 1, max(args.steps, 50), max(args.warmup, 10), dev)
+    if not args.no_other_configs and (args.model, args.bits, args.batch) == ("deit_small", 4, 64):
+        # the other BASELINE configurations, a short timed run each (their own whole-step roofline; same kernels as
+        # `bench.py --model ... --bits ... --batch ...` times at length)
+        out["other_configs"] = {}
+        for name, (mo, bi, ba, st) in {"deit_small_w3a3_bs64": ("deit_small", 3, 64, 20), "deit_base_w4a4_bs64": ("deit_base", 4, 64, 10),
+                                       "vit_large_w3a3_bs256": ("vit_large", 3, 256, 4)}.items():
+            ro, _, _ = run_config(mo, bi, ba, st, 2, dev, use_graph=not args.eager)
+            domo = max(ro["gemm_kernels"], key=lambda k: ro["gemm_kernels"][k]["ms_per_step"])
+            out["other_configs"][name] = {
+                "ms_per_step": ro["ms_per_step"], "images_per_s": ro["images_per_s"], "steps": st, "layers": ro["layers"], "M": ro["M"],
+                "dominant_kernel": domo, "dominant_kernel_us_per_launch": ro["gemm_kernels"][domo]["us_per_launch"],
+                "dominant_kernel_tflops": ro["gemm_kernels"][domo]["tflops"],
+                "dominant_kernel_frac_mfma": ro["gemm_kernels"][domo]["tflops"] / PEAK_FP16_TFLOPS,
+                "stage1_us_per_launch": ro["act_us_per_launch"], "stage1_launches_per_step": ro["act_launches_per_step"],
+                "layer": layer_roofline(ro, bi)}
+            del ro
+            torch.cuda.empty_cache()
     if not args.no_model:
         out["model_forward"] = model_forward(args.model, args.bits, sorted({1, args.batch}), args.steps, args.warmup, dev)
     if args.fp8:
