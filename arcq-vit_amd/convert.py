@@ -94,15 +94,13 @@ def load_training_checkpoint(model: nn.Module, source: Union[str, Path, Dict]) -
     """Load a training checkpoint (path, wrapper dict or state dict) into a fake-quant model
     (scripts/benchmark_arcq_packed_inference.py:101-113)."""
     state = read_checkpoint_state(source) if isinstance(source, (str, Path)) else unwrap_checkpoint(source)
-    current = model.state_dict()
-    compatible = {}
-    skipped_shape = 0
-    for key, value in state.items():
-        if key in current and tuple(current[key].shape) == tuple(value.shape):
-            compatible[key] = value
-        elif key in current:
-            skipped_shape += 1
-    missing, unexpected = model.load_state_dict(compatible, strict=False)
+    # Entries whose name the model knows are split by whether the shapes agree; only those go through
+    # load_state_dict, the rest (the quantizers' dynamically sized tensors among them) is handled below.
+    own_shapes = {name: tuple(t.shape) for name, t in model.state_dict().items()}
+    known = [name for name in state if name in own_shapes]
+    fitting = {name: state[name] for name in known if tuple(state[name].shape) == own_shapes[name]}
+    skipped_shape = len(known) - len(fitting)
+    missing, unexpected = model.load_state_dict(fitting, strict=False)
     restored = restore_dynamic_state_tensors(model, state)
     return LoadReport(len(missing), len(unexpected), skipped_shape, restored)
 

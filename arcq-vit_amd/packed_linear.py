@@ -230,7 +230,16 @@ class ARCQPackedLinear(nn.Module):
                                 out_dtype=torch.float32)
             return y2.reshape(*original_shape[:-1], self.out_features)
         x2 = x.reshape(-1, self.in_features).to(device=dev, dtype=torch.float32).contiguous()
-        if fmt == "dequant_gemm":
+        if fmt == "dequant_gemm" and self.group_size == 64 and x2.shape[0] > 0:
+            # Stage 1 -> fp16 x_hat (the fp32 reconstruction rounded once, as `.half()` of the reference's fp32 x_hat),
+            # then this library's MFMA GEMM on the cached dense weight (no vendor GEMM); the bias is added in fp32
+            # before the one output rounding (the reference rounds it to fp16 first, FQ/arcq_packed_linear.py:175).
+            xb = ops.quantize_activation_blocked(x2, self.activation_thresholds, self.activation_codebook, self.bits)
+            y2 = ops.linear_fused_blocked(xb, x2.shape[0], self.in_features, self.packed_weight_codes, self.weight_codebook,
+                                          self.weight_center, self.weight_scale, self.weight_code_sum, bias, self.bits,
+                                          out_dtype=torch.float32, w_hat_ws=self.weight_dequant.reshape(-1),
+                                          w_hat_ready=True)
+        elif fmt == "dequant_gemm":          # other group sizes: the generic stage-1 kernel and a library GEMM
             x_hat = ops.quantize_activation_dequant(x2, self.activation_thresholds, self.activation_codebook,
                                                     self.bits, self.group_size)
             gemm_bias = self.bias.to(torch.float16) if bias is not None else None

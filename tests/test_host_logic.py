@@ -484,3 +484,30 @@ def test_rows_counter_slot_logic():
     a = lib.arcq_rows_counter_slot(small, 2, 0x1000)
     b = lib.arcq_rows_counter_slot(small, 2, 0x2000)
     assert {a, b} == {0, 1} and lib.arcq_rows_counter_slot(small, 2, 0x3000) == -1
+
+
+def test_linear_ex_args_mirror_the_header():
+    """``_lib.LinearExArgs`` must list the fields of ``arcq_linear_ex_args`` (include/arcq_hip.h) in the header's order
+    with the header's types: all the 32-bit fields are the same size, so a swapped pair would not show anywhere else."""
+    import ctypes
+    import re
+    from arcq_vit_amd import _lib
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "include", "arcq_hip.h")).read()
+    body = re.search(r"typedef struct arcq_linear_ex_args \{(.*?)\} arcq_linear_ex_args;", text, re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    want = []
+    for decl in body.split(";"):
+        decl = " ".join(decl.split())
+        if not decl:
+            continue
+        m = re.match(r"(const )?(uint32_t|int32_t|int64_t|float|void|uint8_t) (.*)", decl)
+        assert m, decl
+        base = m.group(2)
+        for name in m.group(3).split(","):
+            name = name.strip()
+            pointer = name.startswith("*")
+            ctype = ctypes.c_void_p if pointer else {"uint32_t": ctypes.c_uint32, "int32_t": ctypes.c_int32,
+                                                     "int64_t": ctypes.c_int64, "float": ctypes.c_float}[base]
+            want.append((name.lstrip("*"), ctype))
+    assert [(n, t) for n, t in _lib.LinearExArgs._fields_] == want
