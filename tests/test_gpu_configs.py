@@ -44,7 +44,9 @@ def test_model_forward_layerwise_fullbatch(cuda, oracle, model, bits, batch, dep
     widths, through the module path with the shared weight scratch buffer the reference's benchmark sets up.
     Forward hooks take 48 sampled rows of every packed linear's input and output (the method of
     scripts/debug_arcq_packed_correctness.py:198-225); the output rows must equal the oracle's on those input rows
-    within the fp32-accumulation bound plus one fp16 rounding."""
+    within the fp32-accumulation bound plus one fp16 rounding.  Two blocks stand for the models' 12 / 24: every block
+    has the same four layer shapes, so depth changes how often the kernels run, not which ones (the full-depth
+    forwards that bench.py times check nothing and are not a substitute for this test)."""
     vit = build_packed_vit(model, bits, num_classes=100, device="cuda", half_chain=True, depth=depth,
                            shared_buffers=True, max_rows=batch * synth.TOKENS)
     gen = torch.Generator().manual_seed(7)
