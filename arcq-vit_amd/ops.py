@@ -378,6 +378,27 @@ def quantize_activation_blocked_ln(x: torch.Tensor, ln_weight: torch.Tensor, ln_
     return out
 
 
+def attention_fwd(qkv: torch.Tensor, heads: int, scale: Optional[float] = None,
+                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Softmax attention on the qkv layer's output ``[B, n, 3 C]`` fp16 (q, k, v of head h at columns
+    ``(0|1|2) C + 64 h``) -> ``[B, n, C]`` fp16, the proj layer's input, in one launch with no reshaping copies
+    (``arcq_attention_fwd``: head dimension 64, at most 256 tokens).  ``scale`` defaults to ``1 / sqrt(64)``."""
+    _check(qkv.is_cuda and qkv.dtype == torch.float16 and qkv.dim() == 3, "qkv must be a CUDA fp16 tensor [B, n, 3 C]")
+    _check(qkv.is_contiguous(), "qkv must be contiguous")
+    b, n, c3 = qkv.shape
+    _check(c3 % 3 == 0 and (c3 // 3) == heads * 64, f"head dimension must be 64 (C={c3 // 3}, heads={heads})")
+    c = c3 // 3
+    if out is None:
+        out = torch.empty((b, n, c), dtype=torch.float16, device=qkv.device)
+    else:
+        _check(out.is_cuda and out.dtype == torch.float16 and out.is_contiguous() and out.numel() == b * n * c,
+               "out must be a contiguous CUDA fp16 tensor of B * n * C elements")
+    with torch.cuda.device(qkv.device):
+        _lib.check(_lib.load().arcq_attention_fwd(_ptr(qkv), _ptr(out), b, n, heads, 64,
+                                                  0.125 if scale is None else float(scale), _stream()))
+    return out.view(b, n, c)
+
+
 def xhat_layout(m: int) -> int:
     """Layout of an ``x_hat`` passed between two chained layers (``linear_otf_ex`` with ``next_quant`` / ``x_is_xhat``):
     0 = row-major, 1 = the 32-row block layout."""

@@ -39,11 +39,18 @@ class Attention(nn.Module):
         self.num_heads = heads
         self.qkv = linear(dim, dim * 3, True)
         self.proj = linear(dim, dim, True)
+        # True: the library's own attention kernel where it serves the shape (fp16 on the GPU, head dimension 64, at
+        # most 256 tokens): one launch that reads qkv's output and writes proj's input as they lie.
+        self.own_kernel = False
 
     def mix(self, qkv: torch.Tensor) -> torch.Tensor:
         """Softmax attention on the output of ``qkv`` ``[B, tokens, 3 C]`` -> ``[B, tokens, C]`` (input of ``proj``)."""
         b, n, c3 = qkv.shape
         c = c3 // 3
+        if (self.own_kernel and qkv.is_cuda and qkv.dtype == torch.float16 and c == 64 * self.num_heads and n <= 256
+                and qkv.is_contiguous()):
+            from . import ops
+            return ops.attention_fwd(qkv, self.num_heads)
         q, k, v = qkv.reshape(b, n, 3, self.num_heads, c // self.num_heads).permute(2, 0, 3, 1, 4).unbind(0)
         return F.scaled_dot_product_attention(q, k, v).transpose(1, 2).reshape(b, n, c)
 
@@ -162,12 +169,14 @@ def build_fakequant_vit(model: str, bits: int, group_size: int = 64, seed: int =
 def build_packed_vit(model: str, bits: int, group_size: int = 64, seed: int = SEED, num_classes: int = 1000,
                      device: str = "cuda", half_chain: bool = True, depth: Optional[int] = None,
                      shared_buffers: bool = False, max_rows: int = 0, fuse_elementwise: bool = False,
-                     quantize_patch_embed: bool = False, head_quant: str = "fp32") -> VisionTransformer:
+                     quantize_patch_embed: bool = False, head_quant: str = "fp32",
+                     own_attention: bool = False) -> VisionTransformer:
     """Fake-quant ViT -> packed (``convert_arcq_linear_to_packed``) -> on-the-fly layers -> device,
     the sequence of scripts/benchmark_arcq_on_the_fly.py:88-199.  ``half_chain`` casts the
     floating-point rest of the model to fp16 (packed metadata stays fp32).  ``shared_buffers`` gives all
     layers one weight scratch buffer (:182-191 there) and, with ``max_rows`` tokens, one x_hat buffer.
     ``fuse_elementwise``: LayerNorm, GELU and the skip connections run inside the packed layers' launches.
+    ``own_attention``: softmax attention on the library's kernel instead of torch's.
     ``quantize_patch_embed``: the patch embedding is an ``ARCQPackedPatchConv``; ``head_quant="w8a8"``: LSQ head."""
     vit = build_fakequant_vit(model, bits, group_size, seed, num_classes, depth, quantize_patch_embed, head_quant)
     convert_arcq_linear_to_packed(vit, runtime_code_format="packed")
@@ -180,4 +189,5 @@ def build_packed_vit(model: str, bits: int, group_size: int = 64, seed: int = SE
         share_buffers(vit, max_rows)
     for blk in vit.blocks:
         blk.fuse_elementwise = bool(fuse_elementwise)
+        blk.attn.own_kernel = bool(own_attention)
     return vit.eval()

@@ -323,6 +323,18 @@ int arcq_linear_otf_fp8(const void *x, int x_dtype, const float *a_thresholds, c
                         const float *w_code_sum, const float *bias, float w_mult, void *x8_ws, void *w8_ws, void *y,
                         int y_dtype, int64_t M, int64_t N, int64_t K, int bits, void *stream);
 
+/* ---- softmax attention between the packed qkv and proj layers ---------------
+ * No counterpart in the reference's packed path: its models leave attention to timm / torch
+ * (scripts/benchmark_arcq_on_the_fly.py:202-243 times the model with it).  Here so that a ViT block is the four packed
+ * layers plus one more launch, with no reshaping copies: it reads the qkv layer's output as it lies and writes the
+ * proj layer's input as it lies.
+ *   qkv [B, n, 3, H, 64] fp16 (= [B*n, 3*H*64] row-major), out [B, n, H*64] fp16:
+ *   out[b, i, h*64 + j] = sum_k softmax_k(scale * q_i . k_k) v_k[j], fp32 scores / softmax / accumulation, the
+ *   probabilities rounded to fp16 before the second product.
+ * head_dim must be 64 and n <= 256 (ARCQ_ERR_UNSUPPORTED otherwise); qkv 16-byte, out 8-byte aligned. */
+int arcq_attention_fwd(const void *qkv, void *out, int64_t B, int64_t n, int64_t H, int64_t head_dim, float scale,
+                       void *stream);
+
 /* Diagnostics of the one-launch layer kernels; no counterpart in the reference.
  * arcq_rows_wait_timeouts: number of workgroups that, on the current device since the library was loaded, gave up
  * their bounded wait for the other workgroups' weight shares and rebuilt all of w_hat themselves (results stay
