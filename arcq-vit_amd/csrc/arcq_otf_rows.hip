@@ -137,11 +137,12 @@ otf_rows_kernel(const RowsParams p)
     const int rb2 = wave / G, g = wave - rb2 * G;
     uint4 raw[4];
     {
-        const int64_t r0 = row_base + rb2 * 32 + (lane >> 1);
+        // Rows past the tensor's end re-read its last row (their outputs are never stored).  Unconditional loads on
+        // purpose: with a per-lane condition around them the compiler waits for the first load before it issues the next.
+        const int64_t r0 = min(row_base + rb2 * 32 + (lane >> 1), static_cast<int64_t>(p.M) - 1);
         const __half *src = p.x + r0 * K + g * 64 + (lane & 1) * 32;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)          // rows past the tensor's end read as zeros
-            raw[i] = r0 < p.M ? *reinterpret_cast<const uint4 *>(src + i * 8) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < 4; ++i) raw[i] = *reinterpret_cast<const uint4 *>(src + i * 8);
     }
 
     // ---- this workgroup's share of w_hat: the inputs of this thread's first piece are requested here, the piece is
@@ -474,12 +475,11 @@ otf_rows_phased_kernel(const RowsParams p)
     const int rb2 = wave / G, g = wave - rb2 * G;
     const int row = lane >> 1, half = lane & 1;
     uint4 raw[4];
-    auto load_slice = [&](int ph) {                              // rows past the tensor's end read as zeros
-        const int64_t my_row = row_base + rb2 * 32 + row;
+    auto load_slice = [&](int ph) {          // rows past the tensor's end re-read its last row (outputs never stored)
+        const int64_t my_row = min(row_base + rb2 * 32 + row, static_cast<int64_t>(p.M) - 1);
         const __half *src = p.x + my_row * K + ph * KS + g * 64 + half * 32;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            raw[i] = my_row < p.M ? *reinterpret_cast<const uint4 *>(src + i * 8) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < 4; ++i) raw[i] = *reinterpret_cast<const uint4 *>(src + i * 8);
     };
     load_slice(0);
 
