@@ -378,6 +378,32 @@ def quantize_activation_blocked_ln(x: torch.Tensor, ln_weight: torch.Tensor, ln_
     return out
 
 
+def patch_embed_fwd(img: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], cls_token: torch.Tensor,
+                    pos_embed: torch.Tensor) -> torch.Tensor:
+    """Front end of a ViT in one launch (``arcq_patch_embed_fwd``): 16 x 16 stride-16 patch convolution of ``img``
+    ``[B, 3, H, W]`` with ``weight`` ``[N, 3, 16, 16]`` and ``bias``, the class token in front, ``pos_embed`` added ->
+    ``[B, 1 + patches, N]``; everything fp16, fp32 accumulation, rounded as the separate torch operations round."""
+    _check(img.is_cuda and img.dtype == torch.float16 and img.dim() == 4 and img.shape[1] == 3,
+           "img must be a CUDA fp16 tensor [B, 3, H, W]")
+    _check(weight.dtype == torch.float16 and weight.dim() == 4 and tuple(weight.shape[1:]) == (3, 16, 16),
+           "weight must be fp16 [N, 3, 16, 16]")
+    b, _, h, w_ = img.shape
+    n = weight.shape[0]
+    tokens = 1 + (h // 16) * (w_ // 16)
+    _check(h % 16 == 0 and w_ % 16 == 0, "image sides must be multiples of 16")
+    _check(cls_token.numel() == n and pos_embed.numel() == tokens * n, "cls_token / pos_embed do not match the patch grid")
+    for t in (cls_token, pos_embed, bias):
+        _check(t is None or (t.is_cuda and t.dtype == torch.float16), "bias, cls_token and pos_embed must be CUDA fp16 tensors")
+    img, weight = img.contiguous(), weight.contiguous()
+    cls_c, pos_c = cls_token.contiguous(), pos_embed.contiguous()
+    bias_c = None if bias is None else bias.contiguous()
+    out = torch.empty((b, tokens, n), dtype=torch.float16, device=img.device)
+    with torch.cuda.device(img.device):
+        _lib.check(_lib.load().arcq_patch_embed_fwd(_ptr(img), _ptr(weight), _ptr(bias_c), _ptr(cls_c), _ptr(pos_c), _ptr(out),
+                                                    b, h, w_, 16, n, _stream()))
+    return out
+
+
 def attention_fwd(qkv: torch.Tensor, heads: int, scale: Optional[float] = None,
                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Softmax attention on the qkv layer's output ``[B, n, 3 C]`` fp16 (q, k, v of head h at columns

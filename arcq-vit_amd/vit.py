@@ -111,10 +111,20 @@ class VisionTransformer(nn.Module):
         self.blocks = nn.Sequential(*[Block(dim, heads, mlp, linear) for _ in range(depth)])
         self.norm = nn.LayerNorm(dim, eps=1e-6)
         self.head = nn.Linear(dim, num_classes)
+        # True: the library's one-launch fp16 patch embedding where it serves the model (see forward_features)
+        self.own_patch_embed = False
 
     def forward_features(self, x: torch.Tensor) -> torch.Tensor:
-        x = self.patch_embed(x)
-        x = torch.cat([self.cls_token.expand(x.shape[0], -1, -1).to(x.dtype), x], dim=1) + self.pos_embed.to(x.dtype)
+        conv = self.patch_embed.proj
+        if (self.own_patch_embed and type(conv) is nn.Conv2d and x.is_cuda and x.dtype == torch.float16
+                and conv.weight.dtype == torch.float16 and conv.kernel_size == (16, 16) and conv.stride == (16, 16)
+                and conv.padding == (0, 0) and conv.in_channels == 3 and conv.out_channels % 32 == 0
+                and x.shape[-1] % 16 == 0 and x.shape[-2] % 16 == 0):
+            from . import ops       # convolution, class token and position embedding in one launch
+            x = ops.patch_embed_fwd(x, conv.weight, conv.bias, self.cls_token, self.pos_embed)
+        else:
+            x = self.patch_embed(x)
+            x = torch.cat([self.cls_token.expand(x.shape[0], -1, -1).to(x.dtype), x], dim=1) + self.pos_embed.to(x.dtype)
         return self.norm(self.blocks(x))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -170,13 +180,14 @@ def build_packed_vit(model: str, bits: int, group_size: int = 64, seed: int = SE
                      device: str = "cuda", half_chain: bool = True, depth: Optional[int] = None,
                      shared_buffers: bool = False, max_rows: int = 0, fuse_elementwise: bool = False,
                      quantize_patch_embed: bool = False, head_quant: str = "fp32",
-                     own_attention: bool = False) -> VisionTransformer:
+                     own_attention: bool = False, own_patch_embed: bool = False) -> VisionTransformer:
     """Fake-quant ViT -> packed (``convert_arcq_linear_to_packed``) -> on-the-fly layers -> device,
     the sequence of scripts/benchmark_arcq_on_the_fly.py:88-199.  ``half_chain`` casts the
     floating-point rest of the model to fp16 (packed metadata stays fp32).  ``shared_buffers`` gives all
     layers one weight scratch buffer (:182-191 there) and, with ``max_rows`` tokens, one x_hat buffer.
     ``fuse_elementwise``: LayerNorm, GELU and the skip connections run inside the packed layers' launches.
-    ``own_attention``: softmax attention on the library's kernel instead of torch's.
+    ``own_attention``: softmax attention on the library's kernel instead of torch's; ``own_patch_embed``: the fp16 patch
+    convolution, class token and position embedding in one launch of the library's instead of four torch kernels.
     ``quantize_patch_embed``: the patch embedding is an ``ARCQPackedPatchConv``; ``head_quant="w8a8"``: LSQ head."""
     vit = build_fakequant_vit(model, bits, group_size, seed, num_classes, depth, quantize_patch_embed, head_quant)
     convert_arcq_linear_to_packed(vit, runtime_code_format="packed")
@@ -190,4 +201,5 @@ def build_packed_vit(model: str, bits: int, group_size: int = 64, seed: int = SE
     for blk in vit.blocks:
         blk.fuse_elementwise = bool(fuse_elementwise)
         blk.attn.own_kernel = bool(own_attention)
+    vit.own_patch_embed = bool(own_patch_embed)
     return vit.eval()

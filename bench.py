@@ -547,16 +547,17 @@ def model_forward(model, bits, batches, steps, warmup, dev):
     images: the protocol of scripts/benchmark_arcq_on_the_fly.py:202-243 (HIP graph at batch 1, eager otherwise; both
     figures are given for every batch).  Two models: the block's LayerNorms, GELU and skip connections
     as separate torch kernels (`unfused`, the reference's structure), inside the packed layers' launches
-    (`fused_elementwise`), and that with the softmax attention on the library's own kernel instead of torch's
-    (`fused_elementwise_own_attention`: a block is then five launches)."""
+    (`fused_elementwise`), and that with the softmax attention and the fp16 patch embedding on the library's own kernels
+    instead of torch's (`fused_elementwise_own_attention_patch_embed`: a block is then five launches, the front end one)."""
     import torch
     from arcq_vit_amd import synth
     from arcq_vit_amd.vit import build_packed_vit
     out = {"model": model, "bits": bits, "trunk": "fp16 (patch embed, LayerNorm, attention, GELU, head)"}
     for name, fuse, own in (("unfused", False, False), ("fused_elementwise", True, False),
-                            ("fused_elementwise_own_attention", True, True)):
+                            ("fused_elementwise_own_attention_patch_embed", True, True)):
         vit = build_packed_vit(model, bits, device="cuda", half_chain=True, shared_buffers=True,
-                               max_rows=max(batches) * synth.TOKENS, fuse_elementwise=fuse, own_attention=own)
+                               max_rows=max(batches) * synth.TOKENS, fuse_elementwise=fuse, own_attention=own,
+                               own_patch_embed=own)
         out["blocks"] = len(vit.blocks)
         part = {}
         with torch.no_grad():

@@ -335,6 +335,18 @@ int arcq_linear_otf_fp8(const void *x, int x_dtype, const float *a_thresholds, c
 int arcq_attention_fwd(const void *qkv, void *out, int64_t B, int64_t n, int64_t H, int64_t head_dim, float scale,
                        void *stream);
 
+/* ---- fp16 patch embedding of a ViT in one launch ----------------------------
+ * No counterpart in the reference's packed path: the fp16 patch embedding of its models is a torch convolution
+ * followed by the class-token concatenation and the position-embedding addition (timm's VisionTransformer, which
+ * scripts/benchmark_arcq_on_the_fly.py:202-243 times as part of the model).  The quantized patch convolution
+ * (QuantConv2dPCARCQ, FQ/timm_quant_models.py) does not go through this entry point.
+ *   img [B, 3, H, W] fp16; w [N, 768] fp16 (the Conv2d weight [N, 3, 16, 16] as it lies); bias [N] fp16 or NULL;
+ *   cls [N], pos [1 + (H/16)(W/16), N], out [B, 1 + (H/16)(W/16), N] fp16:
+ *   out[b, 0] = cls + pos[0];  out[b, 1 + p] = fp16(fp16(patch(b, p) . w^T + bias) + pos[1 + p]), fp32 accumulation.
+ * patch must be 16, H and W multiples of 16, N a multiple of 32; img and w 16-byte, the others 8-byte aligned. */
+int arcq_patch_embed_fwd(const void *img, const void *w, const void *bias, const void *cls, const void *pos, void *out,
+                         int64_t B, int64_t H, int64_t W, int64_t patch, int64_t N, void *stream);
+
 /* Diagnostics of the one-launch layer kernels; no counterpart in the reference.
  * arcq_rows_wait_timeouts: number of workgroups that, on the current device since the library was loaded, gave up
  * their bounded wait for the other workgroups' weight shares and rebuilt all of w_hat themselves (results stay
