@@ -14,9 +14,8 @@
 //
 // A k-step of 16 covers half of one 16-pixel image row of a patch: the eight values a lane needs of it are 16
 // contiguous bytes of the image, so the fragments are plain 16-byte loads from the image (and from w, whose row is the
-// patch in the same order).  Wave tile = (32 TM) patches x (32 TN) channels, TM = TN = 1 while that gives at most 1024
-// wave tiles, else 2 x 2 (each fragment feeds two MFMAs); up to 256 tiles of 32 x 32 a workgroup per tile with the
-// k-steps split over its four waves (patch_embed_small_kernel).
+// patch in the same order).  Two kernels: patch_embed_kernel (workgroup = 256 patches x 32 channels, weight rows in LDS)
+// and, up to 256 tiles of 32 x 32, patch_embed_small_kernel (a workgroup per tile, the k-steps split over its waves).
 #include "arcq_common.h"
 
 namespace arcq {
@@ -29,21 +28,26 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kPatch = 16, kChannels = 3, kK = kChannels * kPatch * kPatch, kSteps = kK / 16;      // 768, 48
 
-template <int TM, int TN>
+// Workgroup = 256 patches (four waves of 64) x 32 channels.  The 32 weight rows (48 KB) are copied into LDS once, with
+// coalesced loads, and every wave reads its weight fragments from there: straight from global memory a weight
+// fragment touches 32 different cache lines per instruction (one row each), which costs the vector memory path a clock
+// per line and bounded the launch; an image fragment is 1 KB in two or three contiguous runs and stays a global load.
+constexpr int kTM = 2;                                  // 32-patch blocks per wave
+constexpr int kWPitch = kK * 2 + 16;                    // bytes per weight row in LDS (odd number of 16-byte pieces)
+
 __global__ void __launch_bounds__(256)
 patch_embed_kernel(const __half *__restrict__ img, const __half *__restrict__ w, const __half *__restrict__ bias,
                    const __half *__restrict__ cls, const __half *__restrict__ pos, __half *__restrict__ out, int B, int H,
-                   int W, int N, int row_tiles, int col_tiles)
+                   int W, int N, int row_groups, int col_tiles)
 {
+    __shared__ __attribute__((aligned(16))) unsigned char ws[32 * kWPitch];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lh = lane >> 5;
     const int pw = W / kPatch, np = (H / kPatch) * pw;
     const int M = B * np;
-    const int tile = blockIdx.x * 4 + wave;
-    const int tiles = row_tiles * col_tiles;
-    if (tile >= tiles) {
-        // the class-token rows, by the waves past the last tile: element e = b * N + n
-        const int64_t e0 = (static_cast<int64_t>(tile - tiles) * 64 + lane) * 8;
+    const int tiles = row_groups * col_tiles;
+    if (static_cast<int>(blockIdx.x) >= tiles) {        // the class-token rows: element e = b * N + n
+        const int64_t e0 = (static_cast<int64_t>(blockIdx.x - tiles) * 256 + tid) * 8;
         if (e0 < static_cast<int64_t>(B) * N) {
             const int b = static_cast<int>(e0 / N), n = static_cast<int>(e0 - static_cast<int64_t>(b) * N);
             __half *dst = out + static_cast<int64_t>(b) * (np + 1) * N + n;
@@ -52,85 +56,89 @@ patch_embed_kernel(const __half *__restrict__ img, const __half *__restrict__ w,
         }
         return;
     }
-    const int rt = tile / col_tiles, ct = tile - rt * col_tiles;
-    // per row block: this lane's patch, its first image row (channel 0, i = 0) at column 8 lh, its output row
-    const __half *a_base[TM];
-    int64_t out_row[TM];
-    bool valid[TM];
+    const int rg = blockIdx.x / col_tiles, ct = blockIdx.x - rg * col_tiles;      // neighbours share the patches
+    const int n0 = ct * 32;
+    // ---- the weight rows n0 .. n0 + 31 into LDS: 3072 pieces of 16 bytes, twelve per thread, all in flight ----
+    {
+        constexpr int kPiecesPerRow = kK / 8;           // 96
+        u32x4_t t[12];
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm) {
-        const int m = (rt * TM + tm) * 32 + lr;
+        for (int j = 0; j < 12; ++j) {
+            const int p = tid + 256 * j, row = p / kPiecesPerRow, col = p - row * kPiecesPerRow;
+            t[j] = *reinterpret_cast<const u32x4_t *>(w + static_cast<int64_t>(n0 + row) * kK + col * 8);
+        }
+#pragma unroll
+        for (int j = 0; j < 12; ++j) {
+            const int p = tid + 256 * j, row = p / kPiecesPerRow, col = p - row * kPiecesPerRow;
+            *reinterpret_cast<u32x4_t *>(ws + row * kWPitch + col * 16) = t[j];
+        }
+    }
+    // per row block: this lane's patch, its first image row (channel 0, i = 0) at column 8 lh, its output row
+    const __half *a_base[kTM];
+    int64_t out_row[kTM];
+    int pos_row[kTM];
+    bool valid[kTM];
+#pragma unroll
+    for (int tm = 0; tm < kTM; ++tm) {
+        const int m = ((rg * 4 + wave) * kTM + tm) * 32 + lr;
         const int mc = min(m, M - 1);
         const int b = mc / np, p = mc - b * np, py = p / pw, px = p - py * pw;
         a_base[tm] = img + (static_cast<int64_t>(b) * kChannels * H + py * kPatch) * W + px * kPatch + 8 * lh;
         out_row[tm] = static_cast<int64_t>(b) * (np + 1) + 1 + p;
+        pos_row[tm] = 1 + p;
         valid[tm] = m < M;
     }
-    const __half *w_base[TN];
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn) w_base[tn] = w + static_cast<int64_t>(min((ct * TN + tn) * 32 + lr, N - 1)) * kK + 8 * lh;
     const int64_t plane = static_cast<int64_t>(H) * W;
-
-    auto load_step = [&](int s, u32x4_t (&af)[TM], u32x4_t (&bf)[TN]) {
+    auto load_step = [&](int s, u32x4_t (&af)[kTM]) {
         const int c = s >> 4, i = s & 15;
         const int64_t a_off = c * plane + static_cast<int64_t>(i) * W;
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm) af[tm] = *reinterpret_cast<const u32x4_t *>(a_base[tm] + a_off);
-#pragma unroll
-        for (int tn = 0; tn < TN; ++tn) bf[tn] = *reinterpret_cast<const u32x4_t *>(w_base[tn] + s * 16);
+        for (int tm = 0; tm < kTM; ++tm) af[tm] = *reinterpret_cast<const u32x4_t *>(a_base[tm] + a_off);
     };
-    float16_t acc[TM][TN];
+    float16_t acc[kTM];
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm)
+    for (int tm = 0; tm < kTM; ++tm)
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn)
+        for (int v = 0; v < 16; ++v) acc[tm][v] = 0.0f;
+    constexpr int kAhead = 8;                  // k-steps of image fragments in flight
+    u32x4_t af[kAhead][kTM];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[tm][tn][v] = 0.0f;
-    constexpr int kAhead = 4;                  // k-steps in flight
-    u32x4_t af[kAhead][TM], bf[kAhead][TN];
-#pragma unroll
-    for (int s = 0; s < kAhead - 1; ++s) load_step(s, af[s], bf[s]);
+    for (int s = 0; s < kAhead - 1; ++s) load_step(s, af[s]);
+    __syncthreads();                           // the weight rows are in LDS
+    const unsigned char *w_lane = ws + lr * kWPitch + lh * 16;
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
-        if (s + kAhead - 1 < kSteps) load_step(s + kAhead - 1, af[(s + kAhead - 1) % kAhead], bf[(s + kAhead - 1) % kAhead]);
+        if (s + kAhead - 1 < kSteps) load_step(s + kAhead - 1, af[(s + kAhead - 1) % kAhead]);
+        const half8_t wb = *reinterpret_cast<const half8_t *>(w_lane + s * 32);
+        __builtin_amdgcn_sched_barrier(0);     // (left alone, the compiler sinks the loads towards their use)
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm) {
+        for (int tm = 0; tm < kTM; ++tm) {
             half8_t xa;
             __builtin_memcpy(&xa, &af[s % kAhead][tm], 16);
-#pragma unroll
-            for (int tn = 0; tn < TN; ++tn) {
-                half8_t wb;
-                __builtin_memcpy(&wb, &bf[s % kAhead][tn], 16);
-                acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wb, xa, acc[tm][tn], 0, 0, 0);
-            }
+            acc[tm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wb, xa, acc[tm], 0, 0, 0);
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
-    // acc[tm][tn][v]: patch lr of row block tm, channel 8 (v / 4) + 4 lh + v % 4 of column block tn
+    // acc[tm][v]: patch lr of row block tm, channel n0 + 8 (v / 4) + 4 lh + v % 4
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm) {
+    for (int tm = 0; tm < kTM; ++tm) {
         if (!valid[tm]) continue;
-        const int64_t prow = out_row[tm] % (np + 1);            // row of pos
         __half *dst = out + out_row[tm] * N;
-        const __half *ps = pos + prow * N;
+        const __half *ps = pos + static_cast<int64_t>(pos_row[tm]) * N;
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn) {
-            const int n0 = (ct * TN + tn) * 32;
-            if (n0 >= N) continue;
+        for (int q = 0; q < 4; ++q) {
+            const int n = n0 + 8 * q + 4 * lh;
+            const u32x2_t pv = *reinterpret_cast<const u32x2_t *>(ps + n);
+            u32x2_t bv = {0u, 0u};
+            if (bias) bv = *reinterpret_cast<const u32x2_t *>(bias + n);
+            const __half *ph = reinterpret_cast<const __half *>(&pv), *bh = reinterpret_cast<const __half *>(&bv);
+            __half o[4];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int n = n0 + 8 * q + 4 * lh;
-                const u32x2_t pv = *reinterpret_cast<const u32x2_t *>(ps + n);
-                u32x2_t bv = {0u, 0u};
-                if (bias) bv = *reinterpret_cast<const u32x2_t *>(bias + n);
-                const __half *ph = reinterpret_cast<const __half *>(&pv), *bh = reinterpret_cast<const __half *>(&bv);
-                __half o[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const __half y = __float2half_rn(acc[tm][tn][4 * q + e] + __half2float(bh[e]));
-                    o[e] = __float2half_rn(__half2float(y) + __half2float(ph[e]));
-                }
-                *reinterpret_cast<u32x2_t *>(dst + n) = *reinterpret_cast<const u32x2_t *>(o);
+            for (int e = 0; e < 4; ++e) {
+                const __half y = __float2half_rn(acc[tm][4 * q + e] + __half2float(bh[e]));
+                o[e] = __float2half_rn(__half2float(y) + __half2float(ph[e]));
             }
+            *reinterpret_cast<u32x2_t *>(dst + n) = *reinterpret_cast<const u32x2_t *>(o);
         }
     }
 }
@@ -213,20 +221,6 @@ patch_embed_small_kernel(const __half *__restrict__ img, const __half *__restric
     }
 }
 
-template <int TM, int TN>
-void launch_patch_embed(const void *img, const void *w, const void *bias, const void *cls, const void *pos, void *out, int B, int H,
-                        int W, int N, hipStream_t stream)
-{
-    const int M = B * (H / kPatch) * (W / kPatch);
-    const int row_tiles = (M + 32 * TM - 1) / (32 * TM), col_tiles = (N + 32 * TN - 1) / (32 * TN);
-    const int64_t cls_waves = (static_cast<int64_t>(B) * N / 8 + 63) / 64;
-    const int64_t waves = static_cast<int64_t>(row_tiles) * col_tiles + cls_waves;
-    hipLaunchKernelGGL((patch_embed_kernel<TM, TN>), dim3(static_cast<unsigned>((waves + 3) / 4)), dim3(256), 0, stream,
-                       static_cast<const __half *>(img), static_cast<const __half *>(w), static_cast<const __half *>(bias),
-                       static_cast<const __half *>(cls), static_cast<const __half *>(pos), static_cast<__half *>(out), B, H, W, N,
-                       row_tiles, col_tiles);
-}
-
 }  // namespace
 }  // namespace arcq
 
@@ -249,16 +243,19 @@ ARCQ_API int arcq_patch_embed_fwd(const void *img, const void *w, const void *bi
         return fail(ARCQ_ERR_SHAPE, "arcq_patch_embed_fwd: tensor too large");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int b = static_cast<int>(B), h = static_cast<int>(H), wd = static_cast<int>(W), n = static_cast<int>(N);
-    if (((M + 31) / 32) * (N / 32) <= 256) {
-        const int row_tiles = static_cast<int>((M + 31) / 32), col_tiles = n / 32;
-        const int cls_wgs = static_cast<int>((B * N / 8 + 255) / 256);
-        hipLaunchKernelGGL(patch_embed_small_kernel, dim3(row_tiles * col_tiles + cls_wgs), dim3(256), 0, st,
-                           static_cast<const __half *>(img), static_cast<const __half *>(w), static_cast<const __half *>(bias),
-                           static_cast<const __half *>(cls), static_cast<const __half *>(pos), static_cast<__half *>(out), b, h, wd, n,
-                           row_tiles, col_tiles);
-    } else if (((M + 31) / 32) * (N / 32) <= 1024)
-        launch_patch_embed<1, 1>(img, w, bias, cls, pos, out, b, h, wd, n, st);
-    else
-        launch_patch_embed<2, 2>(img, w, bias, cls, pos, out, b, h, wd, n, st);
+    const auto *pi = static_cast<const __half *>(img), *pwt = static_cast<const __half *>(w), *pb = static_cast<const __half *>(bias);
+    const auto *pc = static_cast<const __half *>(cls), *pp = static_cast<const __half *>(pos);
+    auto *po = static_cast<__half *>(out);
+    const int cls_wgs = static_cast<int>((B * N / 8 + 255) / 256);
+    const int col_tiles = n / 32;
+    if (((M + 31) / 32) * col_tiles <= 256) {
+        const int row_tiles = static_cast<int>((M + 31) / 32);
+        hipLaunchKernelGGL(patch_embed_small_kernel, dim3(row_tiles * col_tiles + cls_wgs), dim3(256), 0, st, pi, pwt, pb, pc, pp, po,
+                           b, h, wd, n, row_tiles, col_tiles);
+    } else {
+        const int row_groups = static_cast<int>((M + 128 * kTM - 1) / (128 * kTM));      // four waves of 32 kTM patches
+        hipLaunchKernelGGL(patch_embed_kernel, dim3(row_groups * col_tiles + cls_wgs), dim3(256), 0, st, pi, pwt, pb, pc, pp, po, b, h, wd,
+                           n, row_groups, col_tiles);
+    }
     return launch_status("arcq_patch_embed_fwd");
 }

@@ -125,7 +125,11 @@ class VisionTransformer(nn.Module):
         else:
             x = self.patch_embed(x)
             x = torch.cat([self.cls_token.expand(x.shape[0], -1, -1).to(x.dtype), x], dim=1) + self.pos_embed.to(x.dtype)
-        return self.norm(self.blocks(x))
+        x = self.blocks(x)
+        # LayerNorm works token by token and the head reads the class token only: with own_patch_embed (the trimmed
+        # trunk) only that row is normalised -- the same logits as normalising all tokens first, which is what timm's
+        # forward_features does and what happens otherwise
+        return self.norm(x[:, :1] if self.own_patch_embed else x)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.head(self.forward_features(x)[:, 0])
