@@ -92,6 +92,7 @@ attention_kernel(const __half *__restrict__ qkv, __half *__restrict__ out, int n
     // Keys in chunks of CH blocks with a running maximum and sum (the scores of one chunk are live at a time, which
     // keeps the wave at half the registers and two workgroups on a CU); one chunk is the plain two-pass softmax.
     const float ninf = -__builtin_inff();
+    const float c2 = scale * 1.44269504088896341f;      // exp(scale x) = exp2(c2 x)
     float m = ninf, l = 0.0f;
     float16_t oacc[2];      // oacc[jb][v]: dim jb*32 + 8 (v / 4) + 4 lh + v % 4 of this lane's query
 #pragma unroll
@@ -119,18 +120,21 @@ attention_kernel(const __half *__restrict__ qkv, __half *__restrict__ out, int n
                 __builtin_memcpy(&qv, &qf[kk], 16);
                 acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qv, acc[i], 0, 0, 0);
             }
+            // (raw scores: the scale is positive, so it commutes with the maximum and is applied inside the exponential;
+            // only the last key block can hold keys past n)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int key = kb * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-                const float sv = key < n ? acc[i][v] * scale : ninf;
-                acc[i][v] = sv;
-                cm = fmaxf(cm, sv);
+                if (kb == NKB - 1) {
+                    const int key = kb * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+                    acc[i][v] = key < n ? acc[i][v] : ninf;
+                }
+                cm = fmaxf(cm, acc[i][v]);
             }
         }
         cm = fmaxf(cm, __shfl_xor(cm, 32));
         const float m_new = fmaxf(m, cm);       // finite: every chunk holds at least one key < n
         if (ch > 0) {                           // rescale what the earlier chunks left (exp(-inf) never occurs here)
-            const float alpha = __expf(m - m_new);
+            const float alpha = __builtin_amdgcn_exp2f((m - m_new) * c2);
             l *= alpha;
 #pragma unroll
             for (int jb = 0; jb < 2; ++jb)
@@ -138,6 +142,7 @@ attention_kernel(const __half *__restrict__ qkv, __half *__restrict__ out, int n
                 for (int v = 0; v < 16; ++v) oacc[jb][v] *= alpha;
         }
         m = m_new;
+        const float mc = -m * c2;
         // ---- probabilities (this lane's share of the row sum; the two halves are added at the end) and O^T += V^T P^T ----
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
@@ -145,7 +150,7 @@ attention_kernel(const __half *__restrict__ qkv, __half *__restrict__ out, int n
             const int kb = ch * CH + i;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const float p = __expf(acc[i][v] - m);
+                const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[i][v], c2, mc));      // exp(scale (s - m))
                 acc[i][v] = p;
                 l += p;
             }
@@ -202,6 +207,7 @@ ARCQ_API int arcq_attention_fwd(const void *qkv, void *out, int64_t B, int64_t n
                                 void *stream)
 {
     if (B < 0 || n < 0 || H < 0) return fail(ARCQ_ERR_SHAPE, "arcq_attention_fwd: negative size");
+    if (!(scale > 0.0f)) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_attention_fwd: scale must be positive");
     if (head_dim != kHeadDim) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_attention_fwd: head_dim must be 64 (got %lld)", static_cast<long long>(head_dim));
     if (n > 256) return fail(ARCQ_ERR_UNSUPPORTED, "arcq_attention_fwd: at most 256 tokens (got %lld)", static_cast<long long>(n));
     if (B * n * H == 0) return ARCQ_OK;

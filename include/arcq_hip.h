@@ -331,7 +331,7 @@ int arcq_linear_otf_fp8(const void *x, int x_dtype, const float *a_thresholds, c
  *   qkv [B, n, 3, H, 64] fp16 (= [B*n, 3*H*64] row-major), out [B, n, H*64] fp16:
  *   out[b, i, h*64 + j] = sum_k softmax_k(scale * q_i . k_k) v_k[j], fp32 scores / softmax / accumulation, the
  *   probabilities rounded to fp16 before the second product.
- * head_dim must be 64 and n <= 256 (ARCQ_ERR_UNSUPPORTED otherwise); qkv 16-byte, out 8-byte aligned. */
+ * head_dim must be 64, n <= 256 and scale > 0 (ARCQ_ERR_UNSUPPORTED otherwise); qkv 16-byte, out 8-byte aligned. */
 int arcq_attention_fwd(const void *qkv, void *out, int64_t B, int64_t n, int64_t H, int64_t head_dim, float scale,
                        void *stream);
 
