@@ -385,8 +385,9 @@ def patch_embed_fwd(img: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
     ``[B, 1 + patches, N]``; everything fp16, fp32 accumulation, rounded as the separate torch operations round."""
     _check(img.is_cuda and img.dtype == torch.float16 and img.dim() == 4 and img.shape[1] == 3,
            "img must be a CUDA fp16 tensor [B, 3, H, W]")
-    _check(weight.dtype == torch.float16 and weight.dim() == 4 and tuple(weight.shape[1:]) == (3, 16, 16),
-           "weight must be fp16 [N, 3, 16, 16]")
+    _check(weight.is_cuda and weight.dtype == torch.float16 and weight.dim() == 4 and tuple(weight.shape[1:]) == (3, 16, 16),
+           "weight must be a CUDA fp16 tensor [N, 3, 16, 16]")
+    _check(weight.shape[0] % 32 == 0, "the embedding width must be a multiple of 32")
     b, _, h, w_ = img.shape
     n = weight.shape[0]
     tokens = 1 + (h // 16) * (w_ // 16)
