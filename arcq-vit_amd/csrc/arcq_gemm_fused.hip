@@ -387,7 +387,7 @@ bool arcq::otf_blocked_pays(int64_t M, int64_t N, int64_t K)
 
 ARCQ_API const char *arcq_linear_otf_ws_kernel(int64_t M, int64_t N, int64_t K, int have_workspace)
 {
-    if (have_workspace && otf_rows_pays(M, N, K)) return K > 384 ? "otf_rows_phased_kernel" : "otf_rows_kernel";      // (for fp16 input)
+    if (have_workspace && otf_rows_pays(M, N, K)) return otf_rows_is_phased(N, K) ? "otf_rows_phased_kernel" : "otf_rows_kernel";      // (for fp16 input)
     if (otf_blocked_pays(M, N, K)) {
         if (!(have_workspace && blocked_uses_workspace(N, K))) return "gemm_slab8_kernel";
         GemmArgs g{};

@@ -1,8 +1,9 @@
 // Whole on-the-fly layer in ONE launch for many rows of moderate length: a workgroup owns 64 rows of x, quantizes
 // them into LDS (stage 1, optionally with the LayerNorm in front of it) and multiplies them with every column of
 // w_hat, which streams through the registers from a 32-column block layout in the weight workspace.  Two kernels:
-// otf_rows_kernel (K = 192 / 256 / 384: the whole row at once) and otf_rows_phased_kernel (K = 768 / 1536, at most
-// 384 output columns: the row in slices of 384 values, stage 1 of a slice under the MFMAs of the one before).
+// otf_rows_kernel (K = 192 / 256 / 384: the whole row at once; also K = 768 with fp16 outputs, twelve waves that
+// quantize two tiles each and a 97 KB x_hat tile) and otf_rows_phased_kernel (K = 768 / 1536, at most 384 output
+// columns: the row in slices of 384 values, stage 1 of a slice under the MFMAs of the one before).
 //
 //   y[M,N] = post( stage1( [LayerNorm] x )[M,K] * w_hat[N,K]^T + bias )
 //
@@ -44,6 +45,9 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kWaveLds = 4608;               // bytes of LDS per wave: the output staging tile (32 rows of 128 + 16 bytes)
+// otf_rows_kernel's staging tile: kWaveLds, or, where a wave quantizes two tiles (K = 768: LDS is short), just the
+// 32 rows of 32 outputs + 16 bytes that the epilogue uses.
+constexpr int rows_stage_bytes(int rounds, size_t out_size) { return rounds == 1 ? kWaveLds : 32 * (32 * static_cast<int>(out_size) + 16); }
 constexpr unsigned long long kEpoch = 1ull << 20;     // what one launch adds to its counter, whatever its grid
 
 constexpr int gcd_of(int a, int b) { return b == 0 ? a : gcd_of(b, a % b); }
@@ -109,40 +113,47 @@ __device__ __forceinline__ void finish_piece(const RowsParams &p, int64_t idx, c
 // G = K / 64 groups per row (the workgroup has 2 G waves); RING = groups of w_hat fragments a wave holds (the one
 // being multiplied and RING - 1 on their way from L2); AHEAD = k-steps by which the LDS reads of the x_hat fragments
 // run ahead of the MFMAs that use them.
-template <int BITS, typename TOUT, int G, int RING, int AHEAD>
-__global__ void __launch_bounds__(128 * G)
+// WV = waves per workgroup: 2 G (every wave one stage-1 tile) or, for K = 768, G (two tiles per wave, one after the
+// other: sixteen waves are the most a workgroup can have).
+template <int BITS, typename TOUT, int G, int RING, int AHEAD, int WV = 2 * G>
+__global__ void __launch_bounds__(64 * WV)
 otf_rows_kernel(const RowsParams p)
 {
     constexpr int L = 1 << BITS;
-    constexpr int MAXW = 2 * G;
+    constexpr int MAXW = WV;
+    constexpr int ROUNDS = 2 * G / WV;                              // stage-1 tiles per wave
+    static_assert(ROUNDS * WV == 2 * G, "waves must divide the 2 G stage-1 tiles");
+    constexpr int kStage = rows_stage_bytes(ROUNDS, sizeof(TOUT));  // bytes of a wave's output staging tile
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ float lut[L * 64];
     __shared__ Bucket table[kMaxBuckets + 1];
     __shared__ int slow_slots[MAXW];
     __shared__ int s_flag;
 
-    constexpr int K = 64 * G, W = 2 * G;
+    constexpr int K = 64 * G, W = WV;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     constexpr int nthreads = 64 * W;
     constexpr int pitch = K * 2 + 16;                               // bytes per x_hat row in LDS (conflict-free 16-byte reads)
     unsigned char *xs = smem;                                   // [64][pitch]
-    unsigned char *wave_lds = smem + 64 * pitch + wave * kWaveLds;
-    float *part = reinterpret_cast<float *>(smem + 64 * pitch + W * kWaveLds);      // [64][2 G + 1]
+    unsigned char *wave_lds = smem + 64 * pitch + wave * kStage;
+    float *part = reinterpret_cast<float *>(smem + 64 * pitch + W * kStage);        // [64][2 G + 1]
     float *s_bias = part + 64 * (2 * G + 1);                    // [N]
     const int64_t row_base = static_cast<int64_t>(blockIdx.x) * 64;
     const int64_t pieces = static_cast<int64_t>(p.N) * (K / 8);
 
     // The wave's stage-1 inputs (wave = (row block rb2, group g): 32 rows x 64 values; a lane pair holds one row's 64,
     // each lane 64 contiguous bytes) are requested first, so that they travel while the weights are rebuilt.
-    const int rb2 = wave / G, g = wave - rb2 * G;
-    uint4 raw[4];
-    {
+    // (tile t = wave + round * W: row block t / G, group t % G)
+    uint4 raws[ROUNDS][4];
+#pragma unroll
+    for (int rnd = 0; rnd < ROUNDS; ++rnd) {
         // Rows past the tensor's end re-read its last row (their outputs are never stored).  Unconditional loads on
         // purpose: with a per-lane condition around them the compiler waits for the first load before it issues the next.
+        const int t = wave + rnd * W, rb2 = t / G, g = t - rb2 * G;
         const int64_t r0 = min(row_base + rb2 * 32 + (lane >> 1), static_cast<int64_t>(p.M) - 1);
         const __half *src = p.x + r0 * K + g * 64 + (lane & 1) * 32;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) raw[i] = *reinterpret_cast<const uint4 *>(src + i * 8);
+        for (int i = 0; i < 4; ++i) raws[rnd][i] = *reinterpret_cast<const uint4 *>(src + i * 8);
     }
 
     // ---- this workgroup's share of w_hat: the inputs of this thread's first piece are requested here, the piece is
@@ -211,6 +222,10 @@ otf_rows_kernel(const RowsParams p)
             const unsigned long long old = __hip_atomic_fetch_add(p.counter, inc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             target = (old & ~(kEpoch - 1)) + kEpoch;            // every launch adds kEpoch in total
         }
+#pragma unroll
+      for (int rnd = 0; rnd < ROUNDS; ++rnd) {
+        const int tile = wave + rnd * W, rb2 = tile / G, g = tile - rb2 * G;
+        const uint4 (&raw)[4] = raws[rnd];
         float xv[32];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -281,6 +296,7 @@ otf_rows_kernel(const RowsParams p)
             }
             *reinterpret_cast<u32x4_t *>(dst + q4 * 16) = o;
         }
+      }
     }
 
     // ---- every share of w_hat written? ----
@@ -796,11 +812,14 @@ int device_cus()
 
 namespace {
 
-size_t rows_lds_bytes(int N, int K)
+// Waves of otf_rows_kernel's workgroup: one per stage-1 tile (2 K / 64), for K = 768 half as many.
+constexpr int rows_waves(int G) { return G == 12 ? 12 : 2 * G; }
+
+size_t rows_lds_bytes(int N, int K, size_t out_size = 2)
 {
-    const int G = K / 64;
-    return static_cast<size_t>(64) * (K * 2 + 16) + static_cast<size_t>(2 * G) * kWaveLds + 64 * (2 * G + 1) * sizeof(float) +
-           static_cast<size_t>(N) * sizeof(float);
+    const int G = K / 64, W = rows_waves(G);
+    return static_cast<size_t>(64) * (K * 2 + 16) + static_cast<size_t>(W) * rows_stage_bytes(2 * G / W, out_size) +
+           64 * (2 * G + 1) * sizeof(float) + static_cast<size_t>(N) * sizeof(float);
 }
 
 // Workgroups to add to a launch of `tiles` row workgroups for the reconstruction of w_hat alone, given `spare` free
@@ -819,12 +838,13 @@ int helper_workgroups(const RowsParams &p, int tiles, int spare, int threads)
 template <int BITS, typename TOUT, int G, int RING, int AHEAD>
 bool launch_rows_g(const RowsParams &p, size_t smem, hipStream_t stream)
 {
-    allow_dynamic_lds<otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>>(160 * 1024 - 10 * 1024);
+    constexpr int W = rows_waves(G);
+    allow_dynamic_lds<otf_rows_kernel<BITS, TOUT, G, RING, AHEAD, W>>(160 * 1024 - 10 * 1024);
     const int tiles = (p.M + 63) / 64;
-    const int cap = resident_workgroups<otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>>(128 * G, smem);
+    const int cap = resident_workgroups<otf_rows_kernel<BITS, TOUT, G, RING, AHEAD, W>>(64 * W, smem);
     if (cap < tiles) return false;
-    hipLaunchKernelGGL((otf_rows_kernel<BITS, TOUT, G, RING, AHEAD>), dim3(tiles + helper_workgroups(p, tiles, cap - tiles, 128 * G)),
-                       dim3(128 * G), smem, stream, p);
+    hipLaunchKernelGGL((otf_rows_kernel<BITS, TOUT, G, RING, AHEAD, W>), dim3(tiles + helper_workgroups(p, tiles, cap - tiles, 64 * W)),
+                       dim3(64 * W), smem, stream, p);
     return true;
 }
 
@@ -837,6 +857,10 @@ bool launch_rows(const RowsParams &p, size_t smem, hipStream_t stream)
 {
     if (p.G == 3) return launch_rows_g<BITS, TOUT, 3, 2, 1>(p, smem, stream);
     if (p.G == 4) return launch_rows_g<BITS, TOUT, 4, 2, 1>(p, smem, stream);
+    if (p.G == 12) {
+        if constexpr (sizeof(TOUT) == 2) return launch_rows_g<BITS, TOUT, 12, 2, 1>(p, smem, stream);
+        else return false;      // (fp32 outputs: the staging tiles do not fit beside a 64 x 768 x_hat tile)
+    }
     return launch_rows_g<BITS, TOUT, 6, 2, 1>(p, smem, stream);
 }
 
@@ -865,6 +889,8 @@ bool phased_shape(int64_t N, int64_t K) { return (K == 768 || K == 1536) && N <=
 
 }  // namespace
 
+bool otf_rows_is_phased(int64_t N, int64_t K) { return phased_shape(N, K); }
+
 bool otf_rows_supported(int64_t M, int64_t N, int64_t K, bool layernorm)
 {
     if (M < 512 || N < 32 || N % 32 != 0 || N > 16384) return false;
@@ -873,6 +899,7 @@ bool otf_rows_supported(int64_t M, int64_t N, int64_t K, bool layernorm)
     const int64_t tiles = (M + 63) / 64;
     if (tiles > static_cast<int64_t>(device_cus()) * (K == 192 ? 2 : 1)) return false;
     if (phased_shape(N, K)) return !layernorm;
+    if (K == 768) return rows_lds_bytes(static_cast<int>(N), 768) <= 160 * 1024 - 10 * 1024;      // (fp16 outputs only: launch_rows)
     if (K != 192 && K != 256 && K != 384) return false;
     return rows_lds_bytes(static_cast<int>(N), static_cast<int>(K)) <= 160 * 1024 - 10 * 1024;
 }
@@ -920,7 +947,7 @@ int launch_otf_rows(const OtfRowsArgs &a, hipStream_t stream)
                        : a.bits == 3 ? launch_phased<3, float>(p, a.K, stream)
                                      : launch_phased<2, float>(p, a.K, stream);
     } else {
-        const size_t smem = rows_lds_bytes(a.N, a.K);
+        const size_t smem = rows_lds_bytes(a.N, a.K, a.y_f16 ? 2 : 4);
         if (a.y_f16)
             launched = a.bits == 4   ? launch_rows<4, __half>(p, smem, stream)
                        : a.bits == 3 ? launch_rows<3, __half>(p, smem, stream)

@@ -34,7 +34,9 @@ def _w_blocked(w16):
                                             (1001, 96, 192, 2, torch.float32), (5000, 1024, 256, 3, torch.float16),
                                             (577, 32, 384, 4, torch.float32),
                                             (12608, 384, 1536, 4, torch.float16), (12608, 192, 768, 3, torch.float32),
-                                            (9000, 96, 1536, 2, torch.float16), (6001, 384, 768, 4, torch.float32)])
+                                            (9000, 96, 1536, 2, torch.float16), (6001, 384, 768, 4, torch.float32),
+                                            (12608, 2304, 768, 4, torch.float16), (12608, 768, 768, 3, torch.float16),
+                                            (9001, 3072, 768, 2, torch.float16)])
 def test_rows_kernel_against_oracle_and_two_launch_path(cuda, oracle, monkeypatch, m, n, k, bits, out):
     """The kernel's y against the fp64 oracle on sampled rows (fp32-accumulation bound plus the output rounding),
     the weight workspace against the oracle's w_hat bit for bit (block layout), and y bit for bit against the
@@ -43,7 +45,8 @@ def test_rows_kernel_against_oracle_and_two_launch_path(cuda, oracle, monkeypatc
     x = synth.make_activation(m, k, 33, "ln").to(torch.float16)
     d = lambda t: t.to(cuda)
     args = (d(thr), d(cb), d(pw), d(cb), d(wc), d(ws), d(wcs), d(bias), bits, 64)
-    kernel = b"otf_rows_kernel" if k <= 384 else b"otf_rows_phased_kernel"
+    # (K = 768 with more than 384 outputs: the whole-row kernel with two stage-1 tiles per wave, fp16 outputs only)
+    kernel = b"otf_rows_kernel" if k <= 384 or n > 384 else b"otf_rows_phased_kernel"
     assert _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1) == kernel
     w_ws = torch.zeros(n * k, dtype=torch.float16, device=cuda)
     y = ops.linear_otf(d(x), *args, out_dtype=out, w_hat_ws=w_ws)
@@ -86,12 +89,12 @@ def test_more_row_tiles_than_the_device_holds_take_the_two_launch_path(cuda, ora
     assert torch.equal(y, ops.linear_otf(x, *args, out_dtype=torch.float16, w_hat_ws=w_ws))
 
 
-@pytest.mark.parametrize("bits,out", [(4, torch.float16), (3, torch.float32)])
-def test_rows_kernel_with_layernorm_gelu_residual(cuda, oracle, monkeypatch, bits, out):
+@pytest.mark.parametrize("m,n,k,bits,out", [(6016, 768, 384, 4, torch.float16), (6016, 768, 384, 3, torch.float32),
+                                            (12608, 2304, 768, 4, torch.float16), (9000, 1536, 768, 3, torch.float16)])
+def test_rows_kernel_with_layernorm_gelu_residual(cuda, oracle, monkeypatch, m, n, k, bits, out):
     """arcq_linear_otf_ex through the one-launch kernel: LayerNorm in front, GELU and the skip connection behind,
     bit for bit what the two-launch path gives (whose parts are checked against the oracle elsewhere) and what the
     separate torch operations give around the plain layer."""
-    m, n, k = 6016, 768, 384
     assert _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1) == b"otf_rows_kernel"
     cb, thr, pw, wc, ws, wcs, bias = _layer(oracle, n, k, bits, 41)
     g = torch.Generator().manual_seed(9)
@@ -198,7 +201,8 @@ def test_rows_kernel_counter_protocol(cuda, oracle):
         torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("m,n,k,bits", [(12608, 1152, 384, 4), (3000, 576, 192, 3), (12608, 384, 1536, 4)])
+@pytest.mark.parametrize("m,n,k,bits", [(12608, 1152, 384, 4), (3000, 576, 192, 3), (12608, 384, 1536, 4),
+                                        (12608, 768, 768, 4)])
 def test_rows_kernels_when_nobody_waits(cuda, oracle, monkeypatch, m, n, k, bits):
     """The wait for the other workgroups' weight shares is bounded; with the bound set to zero every workgroup gives
     up at once and reconstructs all the weights itself (what happens, later, when part of a launch is not resident).
@@ -228,3 +232,23 @@ def test_rows_kernels_when_nobody_waits(cuda, oracle, monkeypatch, m, n, k, bits
     assert torch.equal(ops.linear_otf(x, *args, out_dtype=torch.float16, w_hat_ws=w_ws), want)
     assert torch.equal(w_ws, w_want)
     assert _lib.load().arcq_rows_wait_timeouts() == timeouts1
+
+
+def test_k768_fp32_output_takes_the_two_launch_path(cuda, oracle, monkeypatch):
+    """The whole-row kernel for K = 768 has LDS for fp16 staging tiles only: with fp32 outputs the call runs as two
+    launches (the weight workspace then holds w_hat row-major) and gives the bits of the call with the one-launch
+    kernels switched off."""
+    m, n, k, bits = 12608, 1536, 768, 4
+    cb, thr, pw, wc, ws, wcs, bias = _layer(oracle, n, k, bits, 51)
+    x = synth.make_activation(m, k, 53, "ln").to(torch.float16).to(cuda)
+    d = lambda t: t.to(cuda)
+    args = (d(thr), d(cb), d(pw), d(cb), d(wc), d(ws), d(wcs), d(bias), bits, 64)
+    w_ws = torch.zeros(n * k, dtype=torch.float16, device=cuda)
+    y = ops.linear_otf(x, *args, out_dtype=torch.float32, w_hat_ws=w_ws)
+    w16 = oracle.weight_dequant_c(pw.numpy(), cb, wc, ws, wcs, bits, 64, fma=True).astype(np.float16)
+    assert np.array_equal(_np(w_ws).view(np.uint16), w16.reshape(-1).view(np.uint16))
+    y16 = ops.linear_otf(x, *args, out_dtype=torch.float16, w_hat_ws=w_ws)
+    assert np.array_equal(_np(w_ws).view(np.uint16), _w_blocked(w16).view(np.uint16))      # (one launch: block layout)
+    assert torch.equal(y.to(torch.float16), y16)
+    monkeypatch.setenv("ARCQ_ROWS", "0")
+    assert torch.equal(y, ops.linear_otf(x, *args, out_dtype=torch.float32, w_hat_ws=torch.zeros_like(w_ws)))
