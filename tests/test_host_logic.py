@@ -364,7 +364,7 @@ def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
     # The whole-layer entry point with scratch workspaces: whole 32-row blocks from 512 rows on take the block layout.
     monkeypatch.delenv("ARCQ_GEMM_KERNEL")
     both8 = b"gemm_slab8_kernel<copy>"
-    rows = b"otf_rows_kernel"         # short rows (K = 192 / 256 / 384) and both workspaces: the whole layer in one launch
+    rows = b"otf_rows_kernel"         # rows that fit LDS whole (K = 192 / 256 / 384 / 768) and both workspaces: one launch
     assert lib.arcq_linear_otf_ws_kernel(12608, 1152, 384, 1) == rows
     assert lib.arcq_linear_otf_ws_kernel(12608, 576, 192, 1) == rows
     assert lib.arcq_linear_otf_ws_kernel(512, 576, 192, 1) == rows                          # few weights: from 512 rows on
@@ -400,14 +400,22 @@ def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 1) == both8
     monkeypatch.delenv("ARCQ_ROWS")
     assert lib.arcq_linear_otf_ws_kernel(12608, 384, 1536, 0) == b"gemm_slab8_kernel"
+    # K = 768 with more than 384 outputs (the DeiT-B widths): the whole-row kernel, two stage-1 tiles per wave
+    assert lib.arcq_linear_otf_ws_kernel(12608, 768, 768, 1) == rows
+    assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 1) == rows
+    assert lib.arcq_linear_otf_ws_kernel(12608, 3072, 768, 1) == rows
+    assert lib.arcq_linear_otf_ws_kernel(16448, 2304, 768, 1) != rows                      # (not resident at once)
+    assert lib.arcq_linear_otf_ws_kernel(4096, 2304, 768, 1) != rows                       # (few rows: two launches are faster)
     pair = b"gemm_pair_kernel"        # several slices and at least eight row blocks per workgroup: two blocks per wave
-    assert lib.arcq_linear_otf_ws_kernel(12608, 768, 768, 1) == pair                       # two slices, six slabs
+    assert lib.arcq_linear_otf_ws_kernel(12608, 768, 3072, 1) == pair                      # sixteen slices, six slabs
     assert lib.arcq_linear_otf_ws_kernel(50432, 4096, 1024, 1) == pair                     # three slices
+    monkeypatch.setenv("ARCQ_ROWS", "0")
     assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 1) == pair
     assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 0) == b"gemm_slab8_kernel"      # (needs the weights ready)
     monkeypatch.setenv("ARCQ_PAIR", "0")
     assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 1) == both8
     monkeypatch.delenv("ARCQ_PAIR")
+    monkeypatch.delenv("ARCQ_ROWS")
     assert lib.arcq_linear_otf_ws_kernel(1576, 384, 1536, 1) == both8                      # a ragged last block is fine
     assert lib.arcq_linear_otf_ws_kernel(197, 1152, 384, 1) == b"gemm_splitk_kernel"
     monkeypatch.setenv("ARCQ_GEMM_KERNEL", "stream")
