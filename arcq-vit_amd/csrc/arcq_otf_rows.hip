@@ -361,6 +361,11 @@ otf_rows_kernel(const RowsParams p)
 
     constexpr int kSlots = 2 * AHEAD;
     constexpr int kStageRow = 32 * static_cast<int>(sizeof(TOUT)) + 16;      // bytes per staged output row
+    // fp16 outputs with the full-size staging tile: two column blocks per write-out, rows of 128 + 16 bytes
+    constexpr bool kPairOut = sizeof(TOUT) == 2 && kStage >= 32 * 144 && G > 3;      // (K = 192 needs its registers for two workgroups per CU)
+    constexpr int kOutRow = kPairOut ? 144 : kStageRow;
+    float16_t held[2];
+    bool have_held = false;
     constexpr int kVec = 16 / static_cast<int>(sizeof(TOUT));
     constexpr int kPiecesPerRow = 32 / kVec;                                  // 4 (fp16) / 8 (fp32)
     constexpr int kRowsPerInstr = 64 / kPiecesPerRow;                         // 16 / 8
@@ -410,47 +415,80 @@ otf_rows_kernel(const RowsParams p)
             }
         }
 
-        // ---- epilogue: bias, rounding, optional GELU / residual; 32 x 32 outputs at a time through the wave's
-        // staging tile so that every lane stores 16 contiguous bytes ----
+        // ---- epilogue: bias, rounding, optional GELU / residual, through the wave's staging tile so that every lane
+        // stores 16 contiguous bytes.  fp16 outputs leave two column blocks at a time where the wave has two in a row
+        // (the first one's accumulators wait in `held`): a row's segment is then a whole 128-byte line instead of two
+        // halves written at different times, which do not always meet again before they reach memory. ----
+        if constexpr (kPairOut) {
+            if (!have_held && cbk + 1 < cb_last) {
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb) held[rb] = acc[rb];
+                have_held = true;
+                continue;
+            }
+        }
+        const int nblk = have_held ? 2 : 1;          // column blocks in this write-out
+        const int cb_out = have_held ? cbk - 1 : cbk;
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
-            float4 bv[4];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) bv[q] = *reinterpret_cast<const float4 *>(s_bias + cbk * 32 + 8 * q + 4 * lh);
+            for (int hb = 0; hb < (kPairOut ? 2 : 1); ++hb) {
+                if (hb >= nblk) continue;
+                const float16_t &src = (kPairOut && nblk == 2 && hb == 0) ? held[rb] : acc[rb];
+                float4 bv[4];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int cl = 8 * q + 4 * lh;
-                const float o0 = acc[rb][4 * q] + bv[q].x, o1 = acc[rb][4 * q + 1] + bv[q].y;
-                const float o2 = acc[rb][4 * q + 2] + bv[q].z, o3 = acc[rb][4 * q + 3] + bv[q].w;
-                unsigned char *dst = wave_lds + lr * kStageRow + cl * static_cast<int>(sizeof(TOUT));
-                if constexpr (sizeof(TOUT) == 2) {
-                    const __half2 lo = __floats2half2_rn(o0, o1), hi = __floats2half2_rn(o2, o3);
-                    u32x2_t pk;
-                    pk[0] = *reinterpret_cast<const uint32_t *>(&lo);
-                    pk[1] = *reinterpret_cast<const uint32_t *>(&hi);
-                    *reinterpret_cast<u32x2_t *>(dst) = pk;
-                } else {
-                    u32x4_t pk;
-                    pk[0] = __float_as_uint(o0); pk[1] = __float_as_uint(o1);
-                    pk[2] = __float_as_uint(o2); pk[3] = __float_as_uint(o3);
-                    *reinterpret_cast<u32x4_t *>(dst) = pk;
+                for (int q = 0; q < 4; ++q) bv[q] = *reinterpret_cast<const float4 *>(s_bias + (cb_out + hb) * 32 + 8 * q + 4 * lh);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int cl = hb * 32 + 8 * q + 4 * lh;
+                    const float o0 = src[4 * q] + bv[q].x, o1 = src[4 * q + 1] + bv[q].y;
+                    const float o2 = src[4 * q + 2] + bv[q].z, o3 = src[4 * q + 3] + bv[q].w;
+                    unsigned char *dst = wave_lds + lr * kOutRow + cl * static_cast<int>(sizeof(TOUT));
+                    if constexpr (sizeof(TOUT) == 2) {
+                        const __half2 lo = __floats2half2_rn(o0, o1), hi = __floats2half2_rn(o2, o3);
+                        u32x2_t pk;
+                        pk[0] = *reinterpret_cast<const uint32_t *>(&lo);
+                        pk[1] = *reinterpret_cast<const uint32_t *>(&hi);
+                        *reinterpret_cast<u32x2_t *>(dst) = pk;
+                    } else {
+                        u32x4_t pk;
+                        pk[0] = __float_as_uint(o0); pk[1] = __float_as_uint(o1);
+                        pk[2] = __float_as_uint(o2); pk[3] = __float_as_uint(o3);
+                        *reinterpret_cast<u32x4_t *>(dst) = pk;
+                    }
                 }
             }
             __builtin_amdgcn_wave_barrier();
-            const int col = cbk * 32 + (lane % kPiecesPerRow) * kVec;
+            if (kPairOut && nblk == 2) {              // 8 lanes per row of 128 bytes, 8 rows per instruction
+                const int col = cb_out * 32 + (lane & 7) * kVec;
 #pragma unroll
-            for (int i = 0; i < 32 / kRowsPerInstr; ++i) {
-                const int r = i * kRowsPerInstr + lane / kPiecesPerRow;
-                u32x4_store_t v = *reinterpret_cast<const u32x4_store_t *>(wave_lds + r * kStageRow + (lane % kPiecesPerRow) * 16);
-                const int64_t grow = row_base + rb * 32 + r;
-                if (grow < p.M) {
-                    if (residual || p.gelu)
-                        post_ops16<TOUT>(v, residual ? residual + grow * p.N + col : nullptr, p.gelu != 0, kVec);
-                    store_streaming16(y + grow * p.N + col, v[0], v[1], v[2], v[3]);
+                for (int i = 0; i < 4; ++i) {
+                    const int r = i * 8 + (lane >> 3);
+                    u32x4_store_t v = *reinterpret_cast<const u32x4_store_t *>(wave_lds + r * kOutRow + (lane & 7) * 16);
+                    const int64_t grow = row_base + rb * 32 + r;
+                    if (grow < p.M) {
+                        if (residual || p.gelu)
+                            post_ops16<TOUT>(v, residual ? residual + grow * p.N + col : nullptr, p.gelu != 0, kVec);
+                        store_streaming16(y + grow * p.N + col, v[0], v[1], v[2], v[3]);
+                    }
+                }
+            } else {
+                const int col = cb_out * 32 + (lane % kPiecesPerRow) * kVec;
+#pragma unroll
+                for (int i = 0; i < 32 / kRowsPerInstr; ++i) {
+                    const int r = i * kRowsPerInstr + lane / kPiecesPerRow;
+                    u32x4_store_t v = *reinterpret_cast<const u32x4_store_t *>(wave_lds + r * kOutRow + (lane % kPiecesPerRow) * 16);
+                    const int64_t grow = row_base + rb * 32 + r;
+                    if (grow < p.M) {
+                        if (residual || p.gelu)
+                            post_ops16<TOUT>(v, residual ? residual + grow * p.N + col : nullptr, p.gelu != 0, kVec);
+                        store_streaming16(y + grow * p.N + col, v[0], v[1], v[2], v[3]);
+                    }
                 }
             }
             __builtin_amdgcn_wave_barrier();
         }
+        have_held = false;
       }
     }
 }
