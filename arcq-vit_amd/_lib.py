@@ -74,6 +74,8 @@ _SIGNATURES = {
                                             _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr],
     "arcq_linear_fused_blocked": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int,
                                   _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr],
+    "arcq_act_quant_patches": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_f32,
+                               _c_int, _c_ptr],
     "arcq_patch_embed_fwd": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr],
     "arcq_attention_fwd": [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_f32, _c_ptr],
     "arcq_linear_forward_packed": [_c_ptr] * 11 + [_c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_ptr],

@@ -378,6 +378,26 @@ def quantize_activation_blocked_ln(x: torch.Tensor, ln_weight: torch.Tensor, ln_
     return out
 
 
+def quantize_patches(img: torch.Tensor, thresholds: torch.Tensor, codebook: torch.Tensor, bits: int,
+                     blocked: bool = False) -> torch.Tensor:
+    """Stage 1 of a quantized 16 x 16 patch convolution on three channels (``arcq_act_quant_patches``): every pixel's
+    channels are one group; returns the reconstructed patch rows ``[B * patches, 768]`` fp16 (column order ``(c, i, j)``
+    of ``conv.weight.reshape``), or with ``blocked`` the flat 32-row block layout ``linear_fused_blocked`` reads."""
+    _check(img.is_cuda and img.dim() == 4 and img.shape[1] == 3 and img.dtype in (torch.float16, torch.float32),
+           "img must be a CUDA fp16 or fp32 tensor [B, 3, H, W]")
+    _check_bits(bits)
+    b, _, h, w = img.shape
+    _check(h % 16 == 0 and w % 16 == 0, "image sides must be multiples of 16")
+    img = img.contiguous()
+    m = b * (h // 16) * (w // 16)
+    out = torch.empty(m * 768 if blocked else (m, 768), dtype=torch.float16, device=img.device)
+    with torch.cuda.device(img.device):
+        _lib.check(_lib.load().arcq_act_quant_patches(_ptr(img), _dtype_code(img, "img"), _ptr(_f32c(thresholds)),
+                                                      _ptr(_f32c(codebook)), _ptr(out), b, 3, h, w, 16, bits, 1.0e-6,
+                                                      int(bool(blocked)), _stream()))
+    return out
+
+
 def patch_embed_fwd(img: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], cls_token: torch.Tensor,
                     pos_embed: torch.Tensor) -> torch.Tensor:
     """Front end of a ViT in one launch (``arcq_patch_embed_fwd``): 16 x 16 stride-16 patch convolution of ``img``

@@ -163,12 +163,22 @@ class ARCQPackedPatchConv(nn.Module):
         x = x.to(dev)
         if x.dtype not in (torch.float16, torch.float32):
             x = x.float()
-        pixels = x.permute(0, 2, 3, 1).contiguous().reshape(-1, c)
-        x_hat = ops.dequant_activation_hip(pixels, self.activation_thresholds, self.activation_codebook,
-                                           self.act_group_size)
-        rows = self.patch_rows(x_hat.reshape(b, h, w, c)).to(torch.float16)
         bias = self.bias if self.bias.numel() > 0 else None
-        y = ops.linear_fused(rows, self.packed_weight_codes, self.weight_codebook, self.weight_center,
-                             self.weight_scale, self.weight_code_sum, bias, self.bits, self.group_size,
-                             out_dtype=x.dtype)
+        weights = (self.packed_weight_codes, self.weight_codebook, self.weight_center, self.weight_scale, self.weight_code_sum)
+        m = b * (h // kh) * (w // kw)
+        if (kh, kw) == (16, 16) and c == 3 and self.act_group_size == 3 and self.group_size == 64:
+            # one launch for stage 1: the pixels' groups quantized and written as patch rows (same values, bit for bit,
+            # as the general route below); from 512 patches on in the block layout of the weight-stationary GEMMs
+            blocked = m >= 512
+            rows = ops.quantize_patches(x, self.activation_thresholds, self.activation_codebook, self.bits, blocked=blocked)
+            if blocked:
+                y = ops.linear_fused_blocked(rows, m, c * kh * kw, *weights, bias, self.bits, out_dtype=x.dtype)
+            else:
+                y = ops.linear_fused(rows, *weights, bias, self.bits, self.group_size, out_dtype=x.dtype)
+        else:
+            pixels = x.permute(0, 2, 3, 1).contiguous().reshape(-1, c)
+            x_hat = ops.dequant_activation_hip(pixels, self.activation_thresholds, self.activation_codebook,
+                                               self.act_group_size)
+            rows = self.patch_rows(x_hat.reshape(b, h, w, c)).to(torch.float16)
+            y = ops.linear_fused(rows, *weights, bias, self.bits, self.group_size, out_dtype=x.dtype)
         return y.reshape(b, h // kh, w // kw, self.out_channels).permute(0, 3, 1, 2)

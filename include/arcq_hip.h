@@ -335,6 +335,19 @@ int arcq_linear_otf_fp8(const void *x, int x_dtype, const float *a_thresholds, c
 int arcq_attention_fwd(const void *qkv, void *out, int64_t B, int64_t n, int64_t H, int64_t head_dim, float scale,
                        void *stream);
 
+/* ---- stage 1 of a quantized patch-embedding convolution ---------------------
+ * QuantConv2dPCARCQ (FQ/quant_backends.py:329-384; the activation quantizer groups min(64, in_channels) = 3 channels
+ * of one pixel, :351) for kernel == stride == 16 on three channels: the pixels' groups are quantized with the
+ * arithmetic of arcq_act_quant (group_size 3) and the reconstructions written as the rows of the patch matrix,
+ * row = (b, py, px), column = c * 256 + i * 16 + j, fp16 -- the values arcq_act_quant gives for the NHWC pixels, bit for
+ * bit, without the NHWC copy and the gather of the rows.
+ *   img [B, 3, H, W] ARCQ_F16 or ARCQ_F32; x_hat: blocked == 0: [B * (H/16) * (W/16), 768] row-major (the input of
+ *   arcq_linear_fused), blocked != 0: the 32-row block layout of arcq_linear_fused_blocked.  img and x_hat 16-byte
+ *   aligned.  Other channel counts or patch sizes: ARCQ_ERR_UNSUPPORTED (compose arcq_act_quant on NHWC pixels). */
+int arcq_act_quant_patches(const void *img, int img_dtype, const float *thresholds, const float *codebook, void *x_hat,
+                           int64_t B, int64_t C, int64_t H, int64_t W, int64_t patch, int bits, float eps, int blocked,
+                           void *stream);
+
 /* ---- fp16 patch embedding of a ViT in one launch ----------------------------
  * No counterpart in the reference's packed path: the fp16 patch embedding of its models is a torch convolution
  * followed by the class-token concatenation and the position-embedding addition (timm's VisionTransformer, which

@@ -34,6 +34,51 @@ def test_stage1_groups_of_three_channels(cuda, oracle, bits, dtype):
                           want.view(np.uint16 if dtype == torch.float16 else np.uint32))
 
 
+def _blocked(rows16: np.ndarray) -> np.ndarray:
+    """[M, K] -> the 32-row block layout: whole blocks [M/32][K/8][32][8], a last block of r rows as [K/8][r][8]."""
+    m, k = rows16.shape
+    full = m // 32 * 32
+    parts = [rows16[:full].reshape(full // 32, 32, k // 8, 8).transpose(0, 2, 1, 3).reshape(-1)]
+    if m > full:
+        parts.append(rows16[full:].reshape(m - full, k // 8, 8).transpose(1, 0, 2).reshape(-1))
+    return np.concatenate(parts)
+
+
+@pytest.mark.parametrize("bits,dtype,b,h,w", [(4, torch.float16, 2, 224, 224), (3, torch.float32, 3, 224, 224),
+                                              (2, torch.float16, 1, 32, 48), (4, torch.float32, 5, 64, 16),
+                                              (4, torch.float16, 64, 224, 224)])
+def test_patch_rows_in_one_launch_equal_the_oracle(cuda, oracle, bits, dtype, b, h, w):
+    """ops.quantize_patches (pixels quantized in groups of three channels and written as patch rows, one launch)
+    against the oracle's stage 1 on the NHWC pixels, gathered into patch rows on the host: bit for bit, row-major and
+    in the block layout (whole blocks and a ragged last one), grey and black pixels included."""
+    cb = synth.quantile_codebook(bits)
+    thr = synth.midpoint_thresholds(cb)
+    g = torch.Generator().manual_seed(7 * b + h)
+    img = (torch.rand(b, 3, h, w, generator=g) - 0.45) / 0.23
+    img[0, :, :3, :5] = img[0, :1, :3, :5]                               # grey pixels: all residuals zero
+    img[0, :, 4, :4] = 0.0
+    img = img.to(dtype)
+    pix = img.permute(0, 2, 3, 1).reshape(-1, 3).contiguous()
+    xh = oracle.act_quant_c(pix.float().numpy(), thr, cb, bits, 3)["x_hat"].astype(np.float16)
+    rows = xh.reshape(b, h // 16, 16, w // 16, 16, 3).transpose(0, 1, 3, 5, 2, 4).reshape(b * (h // 16) * (w // 16), 768)
+    got = ops.quantize_patches(img.to(cuda), thr.to(cuda), cb.to(cuda), bits)
+    assert got.shape == rows.shape and np.array_equal(_np(got).view(np.uint16), rows.view(np.uint16))
+    gotb = ops.quantize_patches(img.to(cuda), thr.to(cuda), cb.to(cuda), bits, blocked=True)
+    assert np.array_equal(_np(gotb).view(np.uint16), _blocked(rows).view(np.uint16))
+
+
+def test_quantize_patches_argument_errors(cuda):
+    lib = A._lib.load()
+    img = torch.zeros(1, 3, 32, 32, dtype=torch.float16, device=cuda)
+    t = torch.zeros(16, dtype=torch.float32, device=cuda)
+    out = torch.zeros(4 * 768, dtype=torch.float16, device=cuda)
+    call = lambda **k: lib.arcq_act_quant_patches(k.get("img", img.data_ptr()), k.get("dt", 1), t.data_ptr(), t.data_ptr(), out.data_ptr(),
+                                                  1, k.get("c", 3), k.get("h", 32), 32, k.get("patch", 16), k.get("bits", 4), 1e-6, 0, None)
+    assert call() == 0
+    assert call(bits=5) == -1 and call(c=4) == -6 and call(patch=8) == -6 and call(h=40) == -4 and call(dt=7) == -5
+    assert call(img=None) == -3 and call(img=img.data_ptr() + 2) == -7
+
+
 @pytest.mark.parametrize("model,bits,batch,dtype", [("deit_small", 4, 8, torch.float16), ("deit_base", 3, 3, torch.float32),
                                                     ("deit_tiny", 2, 5, torch.float16)])
 def test_packed_patch_conv_against_oracle(cuda, oracle, model, bits, batch, dtype):
