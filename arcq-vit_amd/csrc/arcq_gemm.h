@@ -112,7 +112,7 @@ struct OtfRowsArgs {
 // Shapes the kernels can run: M >= 512 and few enough rows that one workgroup per 64 of them is resident at once
 // (M <= 64 x compute units, twice that for K = 192), N a multiple of 32 and either K = 192 / 256 / 384 / 768 with
 // everything within LDS (otf_rows_kernel; K = 768: fp16 outputs only, which launch_otf_rows checks) or K = 768 / 1536
-// with N <= 384 and no LayerNorm in front (otf_rows_phased_kernel).
+// with N <= 384 or K = 3072 with N <= 768, no LayerNorm in front (otf_rows_phased_kernel).
 bool otf_rows_supported(int64_t M, int64_t N, int64_t K, bool layernorm = false);
 bool otf_rows_is_phased(int64_t N, int64_t K);      // which of the two one-launch kernels serves the shape
 // Whether the whole-layer entry points take it for this shape (fp16 input, both workspaces given).

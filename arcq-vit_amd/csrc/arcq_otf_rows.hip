@@ -2,8 +2,9 @@
 // them into LDS (stage 1, optionally with the LayerNorm in front of it) and multiplies them with every column of
 // w_hat, which streams through the registers from a 32-column block layout in the weight workspace.  Two kernels:
 // otf_rows_kernel (K = 192 / 256 / 384: the whole row at once; also K = 768 with fp16 outputs, twelve waves that
-// quantize two tiles each and a 97 KB x_hat tile) and otf_rows_phased_kernel (K = 768 / 1536, at most 384 output
-// columns: the row in slices of 384 values, stage 1 of a slice under the MFMAs of the one before).
+// quantize two tiles each and a 97 KB x_hat tile) and otf_rows_phased_kernel (K = 768 / 1536 with at most 384 output
+// columns, K = 3072 with at most 768: the row in slices of 384 or 256 values, stage 1 of a slice under the MFMAs of the
+// one before).
 //
 //   y[M,N] = post( stage1( [LayerNorm] x )[M,K] * w_hat[N,K]^T + bias )
 //
@@ -501,7 +502,9 @@ otf_rows_kernel(const RowsParams p)
 // 32-column block for the whole launch, so the accumulators stay in registers across the slices; k order per output
 // is ascending as everywhere else.  A lane pair reads its 64 inputs of the next slice straight from global memory
 // (two whole 64-byte halves of a 128-byte line) as soon as the registers of the current one are converted.
-template <int BITS, typename TOUT, int G, int PHASES>
+// NB = column blocks per wave (block nb of wave w is w + nb * 2 G): with eight waves (G = 4) and three blocks each the
+// kernel serves K = 3072 with up to 768 outputs (fc2 of DeiT-B) inside the 256 registers two waves per SIMD have.
+template <int BITS, typename TOUT, int G, int PHASES, int NB = 1>
 __global__ void __launch_bounds__(128 * G)
 otf_rows_phased_kernel(const RowsParams p)
 {
@@ -519,7 +522,7 @@ otf_rows_phased_kernel(const RowsParams p)
     constexpr int pitch = KS * 2 + 16;                           // bytes per x_hat row of a slice
     constexpr int kBuf = 64 * pitch;
     unsigned char *xs = smem;                                    // [2][64][pitch]
-    float *s_bias = reinterpret_cast<float *>(smem + 2 * kBuf);  // [32 W]
+    float *s_bias = reinterpret_cast<float *>(smem + 2 * kBuf);  // [32 W NB]
     unsigned char *wave_lds = smem + wave * kWaveLds;            // output staging: reuses the slice buffers at the end
     static_assert(W * kWaveLds <= 2 * kBuf, "output staging must fit into the slice buffers");
     const int64_t pieces = static_cast<int64_t>(p.N) * (K / 8);
@@ -529,11 +532,12 @@ otf_rows_phased_kernel(const RowsParams p)
     const int rb2 = wave / G, g = wave - rb2 * G;
     const int row = lane >> 1, half = lane & 1;
     uint4 raw[4];
-    auto load_slice = [&](int ph) {          // rows past the tensor's end re-read its last row (outputs never stored)
-        const int64_t my_row = min(row_base + rb2 * 32 + row, static_cast<int64_t>(p.M) - 1);
+    auto load_slice = [&](int ph) {                              // rows past the tensor's end read as zeros
+        const int64_t my_row = row_base + rb2 * 32 + row;
         const __half *src = p.x + my_row * K + ph * KS + g * 64 + half * 32;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) raw[i] = *reinterpret_cast<const uint4 *>(src + i * 8);
+        for (int i = 0; i < 4; ++i)
+            raw[i] = my_row < p.M ? *reinterpret_cast<const uint4 *>(src + i * 8) : make_uint4(0, 0, 0, 0);
     };
     load_slice(0);
 
@@ -551,7 +555,7 @@ otf_rows_phased_kernel(const RowsParams p)
         share_hi = share_lo + per < pieces ? share_lo + per : pieces;
         if (ptid >= 0 && share_lo + ptid < share_hi) fetch_piece<BITS, GT>(p, share_lo + ptid, pc);
     }
-    for (int i = tid; i < 32 * W; i += nthreads) s_bias[i] = (p.bias && i < p.N) ? p.bias[i] : 0.0f;
+    for (int i = tid; i < 32 * W * NB; i += nthreads) s_bias[i] = (p.bias && i < p.N) ? p.bias[i] : 0.0f;
     float th[L - 1], cbv[L];
     load_quant_params<BITS>(p.thr, p.cb_a, th, cbv);
     const BucketScale bq = pick_bucket_scale<BITS>(th);
@@ -574,21 +578,29 @@ otf_rows_phased_kernel(const RowsParams p)
     bool table_ok = true;
     for (int w = 0; w < kBuilders; ++w) table_ok = table_ok && (slow_slots[w] == 0);
 
-    // ---- product role: wave = 32-column block `wave` (idle in the product if the layer has fewer blocks) ----
+    // ---- product role: wave = the 32-column blocks wave, wave + W, ... (idle in the product if it has none) ----
     const int lr = lane & 31, lh = lane >> 5;
     const int ncb = p.N / 32;
-    const bool has_block = wave < ncb;
+    const int nv = wave < ncb ? min(NB, (ncb - wave + W - 1) / W) : 0;      // this wave's blocks: nb < nv
+    const bool has_block = nv > 0;
     const char *w_col = reinterpret_cast<const char *>(p.w_blk) + lh * 2048 + lr * 16 +
                         static_cast<int64_t>(has_block ? wave : 0) * (static_cast<int64_t>(K) * 64);
-    int ld_g = 0;
-    auto load_unit = [&](u32x4_t (&r)[4]) {      // the four fragments of the next group; past the last it re-reads the last
-        const char *q = w_col + (ld_g < GT ? ld_g : GT - 1) * 4096;
+    constexpr int64_t kBlockStride = static_cast<int64_t>(W) * K * 64;      // bytes from a wave's block to its next one
+    // The fragment groups are consumed slice by slice, within a slice block by block, within a block group by group;
+    // load_unit walks the same order (ld_s = G * (slice * nv + block) + group) and re-reads the last group past the end.
+    int ld_ph = 0, ld_nb = 0, ld_g = 0;
+    auto load_unit = [&](u32x4_t (&r)[4]) {
+        const char *q = w_col + ld_nb * kBlockStride + (ld_ph * G + ld_g) * 4096;
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) r[kk] = *reinterpret_cast<const u32x4_t *>(q + kk * 512);
-        ++ld_g;
+        const bool last = ld_ph == PHASES - 1 && ld_nb == nv - 1 && ld_g == G - 1;      // (the last group: stay)
+        const bool wrap_g = ld_g == G - 1, wrap_nb = wrap_g && ld_nb >= nv - 1;
+        ld_g = last ? ld_g : (wrap_g ? 0 : ld_g + 1);
+        ld_nb = last ? ld_nb : (wrap_nb ? 0 : (wrap_g ? ld_nb + 1 : ld_nb));
+        ld_ph = last ? ld_ph : (wrap_nb ? ld_ph + 1 : ld_ph);
     };
     u32x4_t ring[2][4];
-    float16_t acc[2];
+    float16_t acc[NB][2];
 
     auto stage1 = [&](int ph) {                  // slice ph: registers -> xs[ph & 1]; then requests slice ph + 1
         float xv[32];
@@ -622,6 +634,9 @@ otf_rows_phased_kernel(const RowsParams p)
 
     auto product = [&](int ph) {                 // acc += x_hat slice ph * w_hat slice ph^T
         const unsigned char *xb = xs + (ph & 1) * kBuf + lr * pitch + lh * 64;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        if (nb >= nv) break;
         half8_t xf[2][2];
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) xf[0][rb] = *reinterpret_cast<const half8_t *>(xb + rb * 32 * pitch);
@@ -642,7 +657,7 @@ otf_rows_phased_kernel(const RowsParams p)
                 __builtin_memcpy(&wf, &cur_set[kk], 16);
 #pragma unroll
                 for (int rb = 0; rb < 2; ++rb)
-                    acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf, xf[kk % 2][rb], acc[rb], 0, 0, 0);
+                    acc[nb][rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf, xf[kk % 2][rb], acc[nb][rb], 0, 0, 0);
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // 1 MFMA
@@ -651,12 +666,15 @@ otf_rows_phased_kernel(const RowsParams p)
                 }
             }
         }
+      }
     };
 
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[rb][v] = 0.0f;
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[nb][rb][v] = 0.0f;
 
     // ---- the phases: iteration ph multiplies slice ph and quantizes slice ph + 1; iteration -1 only quantizes ----
     const bool multiply_first = ((wave >> 2) & 1) != 0;
@@ -695,15 +713,17 @@ otf_rows_phased_kernel(const RowsParams p)
         }
     }
 
-    // ---- epilogue: as in otf_rows_kernel, one column block per wave ----
-    if (has_block) {
+    // ---- epilogue: as in otf_rows_kernel, one column block at a time ----
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+    if (nb >= nv) break;
     constexpr int kStageRow = 32 * static_cast<int>(sizeof(TOUT)) + 16;
     constexpr int kVec = 16 / static_cast<int>(sizeof(TOUT));
     constexpr int kPiecesPerRow = 32 / kVec;
     constexpr int kRowsPerInstr = 64 / kPiecesPerRow;
     TOUT *y = static_cast<TOUT *>(p.y);
     const TOUT *residual = static_cast<const TOUT *>(p.residual);
-    const int cbk = wave;
+    const int cbk = wave + nb * W;
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
         float4 bv[4];
@@ -712,8 +732,8 @@ otf_rows_phased_kernel(const RowsParams p)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int cl = 8 * q + 4 * lh;
-            const float o0 = acc[rb][4 * q] + bv[q].x, o1 = acc[rb][4 * q + 1] + bv[q].y;
-            const float o2 = acc[rb][4 * q + 2] + bv[q].z, o3 = acc[rb][4 * q + 3] + bv[q].w;
+            const float o0 = acc[nb][rb][4 * q] + bv[q].x, o1 = acc[nb][rb][4 * q + 1] + bv[q].y;
+            const float o2 = acc[nb][rb][4 * q + 2] + bv[q].z, o3 = acc[nb][rb][4 * q + 3] + bv[q].w;
             unsigned char *dst = wave_lds + lr * kStageRow + cl * static_cast<int>(sizeof(TOUT));
             if constexpr (sizeof(TOUT) == 2) {
                 const __half2 lo = __floats2half2_rn(o0, o1), hi = __floats2half2_rn(o2, o3);
@@ -902,28 +922,35 @@ bool launch_rows(const RowsParams &p, size_t smem, hipStream_t stream)
     return launch_rows_g<BITS, TOUT, 6, 2, 1>(p, smem, stream);
 }
 
-constexpr int kPhasedG = 6;                  // groups per slice of the phased kernel (twelve waves)
-constexpr size_t kPhasedLds = 2 * 64 * (64 * kPhasedG * 2 + 16) + 32 * 2 * kPhasedG * sizeof(float);
+// The phased kernel's configurations: slices of G groups on 2 G waves, NB column blocks per wave.
+//   K = 768 / 1536, N <= 384:  G = 6 (twelve waves), one block per wave
+//   K = 3072,       N <= 768:  G = 4 (eight waves),  three blocks per wave
+constexpr int kPhasedG = 6;
+constexpr size_t phased_lds(int G, int NB) { return 2 * 64 * (64 * G * 2 + 16) + 32 * 2 * G * NB * sizeof(float); }
 
-template <int BITS, typename TOUT, int PHASES>
+template <int BITS, typename TOUT, int G, int PHASES, int NB>
 bool launch_phased_p(const RowsParams &p, hipStream_t stream)
 {
-    allow_dynamic_lds<otf_rows_phased_kernel<BITS, TOUT, kPhasedG, PHASES>>(160 * 1024 - 10 * 1024);
+    constexpr size_t lds = phased_lds(G, NB);
+    allow_dynamic_lds<otf_rows_phased_kernel<BITS, TOUT, G, PHASES, NB>>(160 * 1024 - 10 * 1024);
     const int tiles = (p.M + 63) / 64;
-    if (resident_workgroups<otf_rows_phased_kernel<BITS, TOUT, kPhasedG, PHASES>>(128 * kPhasedG, kPhasedLds) < tiles) return false;
-    hipLaunchKernelGGL((otf_rows_phased_kernel<BITS, TOUT, kPhasedG, PHASES>), dim3(tiles), dim3(128 * kPhasedG), kPhasedLds,
-                       stream, p);
+    if (resident_workgroups<otf_rows_phased_kernel<BITS, TOUT, G, PHASES, NB>>(128 * G, lds) < tiles) return false;
+    hipLaunchKernelGGL((otf_rows_phased_kernel<BITS, TOUT, G, PHASES, NB>), dim3(tiles), dim3(128 * G), lds, stream, p);
     return true;
 }
 
 template <int BITS, typename TOUT>
 bool launch_phased(const RowsParams &p, int K, hipStream_t stream)
 {
-    if (K == 768) return launch_phased_p<BITS, TOUT, 2>(p, stream);
-    return launch_phased_p<BITS, TOUT, 4>(p, stream);
+    if (K == 768) return launch_phased_p<BITS, TOUT, kPhasedG, 2, 1>(p, stream);
+    if (K == 3072) return launch_phased_p<BITS, TOUT, 4, 12, 3>(p, stream);
+    return launch_phased_p<BITS, TOUT, kPhasedG, 4, 1>(p, stream);
 }
 
-bool phased_shape(int64_t N, int64_t K) { return (K == 768 || K == 1536) && N <= 32 * 2 * kPhasedG; }
+bool phased_shape(int64_t N, int64_t K)
+{
+    return ((K == 768 || K == 1536) && N <= 32 * 2 * kPhasedG) || (K == 3072 && N <= 32 * 8 * 3);
+}
 
 }  // namespace
 
@@ -952,7 +979,7 @@ bool otf_rows_pays(int64_t M, int64_t N, int64_t K, bool layernorm)
         // of a whole row on one CU); the two launches it replaces spread stage 1 over all CUs and win while the grid
         // is small.  Crossover measured at 128 row tiles for K = 1536 and at 90 for K = 768 (256 CUs).
         const int64_t tiles = (M + 63) / 64;
-        return tiles * (K == 1536 ? 2 : 3) >= device_cus();
+        return tiles * (K == 768 ? 3 : 2) >= device_cus();
     }
     // otf_rows_kernel takes about 8 us + 23 ps per weight whatever the number of rows (every workgroup streams all of
     // w_hat); the two launches take about 12 us + 2.6 fs per multiply-add.  Fitted on N = 384 .. 1536, K = 192 .. 384,

@@ -149,7 +149,8 @@ int arcq_linear_otf(const void *x, int x_dtype, const float *a_thresholds, const
  * With fp16 x, N a multiple of 32, w_hat_ws given (128-byte aligned) and 512 <= M <= 64 x the device's compute units
  * (twice that for K = 192), arcq_linear_otf_ws runs the whole layer as ONE launch for K = 192 / 256 / 384 and, with
  * fp16 outputs, K = 768 with more than 384 outputs (from M >= 8800 - 1.15e9 / (N K) rows on: below that the two
- * launches are faster), and for K = 768 / 1536 with N <= 384 from 86 / 128 blocks of 64 rows on (x_hat stays on chip; w_hat_ws is filled
+ * launches are faster), and for K = 768 / 1536 with N <= 384 or K = 3072 with N <= 768 from 86 / 128 / 128 blocks of
+ * 64 rows on (x_hat stays on chip; w_hat_ws is filled
  * cooperatively, in 32-column blocks [N/32][K/8][32][8]).  The upper limit on M keeps every workgroup of the launch
  * resident at once: each waits, for at most 0.5 ms, until all the others have written their share of w_hat; if the
  * device is shared with other kernels at that moment the wait can run out, after which a workgroup rebuilds all of

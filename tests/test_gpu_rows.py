@@ -36,7 +36,8 @@ def _w_blocked(w16):
                                             (12608, 384, 1536, 4, torch.float16), (12608, 192, 768, 3, torch.float32),
                                             (9000, 96, 1536, 2, torch.float16), (6001, 384, 768, 4, torch.float32),
                                             (12608, 2304, 768, 4, torch.float16), (12608, 768, 768, 3, torch.float16),
-                                            (9001, 3072, 768, 2, torch.float16)])
+                                            (9001, 3072, 768, 2, torch.float16),
+                                            (12608, 768, 3072, 4, torch.float16), (8200, 416, 3072, 3, torch.float32)])
 def test_rows_kernel_against_oracle_and_two_launch_path(cuda, oracle, monkeypatch, m, n, k, bits, out):
     """The kernel's y against the fp64 oracle on sampled rows (fp32-accumulation bound plus the output rounding),
     the weight workspace against the oracle's w_hat bit for bit (block layout), and y bit for bit against the
@@ -45,8 +46,9 @@ def test_rows_kernel_against_oracle_and_two_launch_path(cuda, oracle, monkeypatc
     x = synth.make_activation(m, k, 33, "ln").to(torch.float16)
     d = lambda t: t.to(cuda)
     args = (d(thr), d(cb), d(pw), d(cb), d(wc), d(ws), d(wcs), d(bias), bits, 64)
-    # (K = 768 with more than 384 outputs: the whole-row kernel with two stage-1 tiles per wave, fp16 outputs only)
-    kernel = b"otf_rows_kernel" if k <= 384 or n > 384 else b"otf_rows_phased_kernel"
+    # (K = 768 with more than 384 outputs: the whole-row kernel with two stage-1 tiles per wave, fp16 outputs only;
+    # K = 3072 with up to 768 outputs: the phased kernel with three column blocks per wave)
+    kernel = b"otf_rows_kernel" if k <= 384 or (k == 768 and n > 384) else b"otf_rows_phased_kernel"
     assert _lib.load().arcq_linear_otf_ws_kernel(m, n, k, 1) == kernel
     w_ws = torch.zeros(n * k, dtype=torch.float16, device=cuda)
     y = ops.linear_otf(d(x), *args, out_dtype=out, w_hat_ws=w_ws)
@@ -118,7 +120,8 @@ def test_rows_kernel_with_layernorm_gelu_residual(cuda, oracle, monkeypatch, m, 
     assert float(close.float().mean()) > 0.999        # torch's LayerNorm may round a value differently: rare code flips
 
 
-@pytest.mark.parametrize("n,k,bits,out", [(384, 1536, 4, torch.float16), (192, 768, 3, torch.float32)])
+@pytest.mark.parametrize("n,k,bits,out", [(384, 1536, 4, torch.float16), (192, 768, 3, torch.float32),
+                                          (768, 3072, 4, torch.float16)])
 def test_phased_kernel_with_gelu_and_residual(cuda, oracle, monkeypatch, n, k, bits, out):
     """arcq_linear_otf_ex on the fc2 shapes: GELU and the skip connection in the one-launch kernel's epilogue give the
     bits of the two-launch path and of the separate torch operations behind the plain layer; a LayerNorm in front is
@@ -202,7 +205,7 @@ def test_rows_kernel_counter_protocol(cuda, oracle):
 
 
 @pytest.mark.parametrize("m,n,k,bits", [(12608, 1152, 384, 4), (3000, 576, 192, 3), (12608, 384, 1536, 4),
-                                        (12608, 768, 768, 4)])
+                                        (12608, 768, 768, 4), (12608, 768, 3072, 3)])
 def test_rows_kernels_when_nobody_waits(cuda, oracle, monkeypatch, m, n, k, bits):
     """The wait for the other workgroups' weight shares is bounded; with the bound set to zero every workgroup gives
     up at once and reconstructs all the weights itself (what happens, later, when part of a launch is not resident).

@@ -406,8 +406,12 @@ def test_fused_kernel_choice_is_reported_without_a_gpu(monkeypatch):
     assert lib.arcq_linear_otf_ws_kernel(12608, 3072, 768, 1) == rows
     assert lib.arcq_linear_otf_ws_kernel(16448, 2304, 768, 1) != rows                      # (not resident at once)
     assert lib.arcq_linear_otf_ws_kernel(4096, 2304, 768, 1) != rows                       # (few rows: two launches are faster)
+    assert lib.arcq_linear_otf_ws_kernel(12608, 768, 3072, 1) == phased                    # K = 3072: up to 768 outputs
+    assert lib.arcq_linear_otf_ws_kernel(8192, 768, 3072, 1) == phased                     # 128 row tiles
+    assert lib.arcq_linear_otf_ws_kernel(8128, 768, 3072, 1) != phased
+    assert lib.arcq_linear_otf_ws_kernel(12608, 800, 3072, 1) != phased
     pair = b"gemm_pair_kernel"        # several slices and at least eight row blocks per workgroup: two blocks per wave
-    assert lib.arcq_linear_otf_ws_kernel(12608, 768, 3072, 1) == pair                      # sixteen slices, six slabs
+    assert lib.arcq_linear_otf_ws_kernel(12608, 1024, 3072, 1) == pair                     # sixteen slices, eight slabs
     assert lib.arcq_linear_otf_ws_kernel(50432, 4096, 1024, 1) == pair                     # three slices
     monkeypatch.setenv("ARCQ_ROWS", "0")
     assert lib.arcq_linear_otf_ws_kernel(12608, 2304, 768, 1) == pair
