@@ -638,7 +638,8 @@ def kernel_note(name):
         return ("the WHOLE layer in one launch: stage 1 of 64 rows into LDS, the fp16 weights reconstructed cooperatively "
                 "into the workspace, fp16 MFMA GEMM + bias; its duration includes stage 1 and the reconstruction")
     if name == "otf_rows_phased_kernel":
-        return ("the WHOLE layer in one launch for K = 768 / 1536: the rows are quantized into LDS in slices of 384 values "
+        return ("the WHOLE layer in one launch for long rows and few outputs (K = 768 / 1536 with N <= 384, K = 3072 with "
+                "N <= 768): the rows are quantized into LDS in slices of 384 or 256 values "
                 "while the MFMAs of the previous slice run; weights reconstructed cooperatively into the workspace; "
                 "its duration includes stage 1 and the reconstruction")
     if name in ("gemm_slab8_kernel<copy>", "gemm_pair_kernel"):
