@@ -4,9 +4,9 @@
 Workload (the headline configuration): the 48 packed linears of DeiT-Small (12 blocks x qkv 384->1152,
 proj 384->384, fc1 384->1536, fc2 1536->384), W4A4, group size 64, fp16 activations in and out,
 batch 64 (M = 64*197 = 12608 tokens).  One step = one pass over all 48 layers through
-arcq_linear_otf_ws with both scratch workspaces lent; at this batch every DeiT-S layer runs as ONE launch
-(otf_rows_kernel / otf_rows_phased_kernel: stage 1 into LDS, the fp16 weights reconstructed cooperatively into
-the workspace, fp16 MFMA GEMM + bias), the wider models as two (stage 1 into the block layout with the weight
+arcq_linear_otf_ws with both scratch workspaces lent; at this batch every DeiT-S (and DeiT-B) layer runs as ONE
+launch (otf_rows_kernel / otf_rows_phased_kernel: stage 1 into LDS, the fp16 weights reconstructed cooperatively
+into the workspace, fp16 MFMA GEMM + bias), ViT-L's as two (stage 1 into the block layout with the weight
 reconstruction carried along, then a weight-stationary GEMM).  Inputs (one synthetic activation tensor per layer
 shape, packed weights of 48 distinct random layers) are resident in HBM before the timed region starts.
 
